@@ -1,0 +1,148 @@
+"""ctypes binding of ``libflexshard_hip.so`` (the C ABI in ``include/flexshard_hip.h``).
+
+The library is the only compute path of this package.  If it is missing or
+does not export a declared symbol, :func:`lib` raises ``RuntimeError``; there
+is no eager or CPU substitute.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "libflexshard_hip.so")
+
+FSH_OK = 0
+FSH_MAX_QUANT_CHUNKS = 24
+
+SRC_BF16, SRC_F32, SRC_F32_AS_BF16 = 0, 1, 2
+EPS_INPUT_DTYPE, EPS_FP32 = 0, 1
+DT_BF16, DT_F32 = 0, 1
+REDUCE_SUM, REDUCE_PREMUL, REDUCE_POSTMUL, REDUCE_POSTDIV = 0, 1, 2, 3
+
+
+class QuantChunk(Structure):
+    """``fsh_quant_chunk``."""
+
+    _fields_ = [
+        ("src_dev", c_void_p),
+        ("rows", c_int64),
+        ("in_dim", c_int64),
+        ("src_row_stride", c_int64),
+        ("qdata_offset", c_int64),
+        ("scale_offset", c_int64),
+        ("src_kind", c_int32),
+        ("reserved", c_int32),
+    ]
+
+
+class UnpackChunk(Structure):
+    """``fsh_unpack_chunk`` (seven int64 fields, 56 bytes)."""
+
+    _fields_ = [
+        ("src_qdata_offset", c_int64),
+        ("src_scale_offset", c_int64),
+        ("rows", c_int64),
+        ("in_dim", c_int64),
+        ("dst_qdata_offset", c_int64),
+        ("dst_scale_offset", c_int64),
+        ("dst_dequant_offset", c_int64),
+    ]
+
+
+UNPACK_CHUNK_INT64S = 7
+
+
+class GemmDesc(Structure):
+    """``fsh_gemm_desc``."""
+
+    _fields_ = [
+        ("a_dev", c_void_p),
+        ("b_dev", c_void_p),
+        ("d_dev", c_void_p),
+        ("c_dev", c_void_p),
+        ("ct_dev", c_void_p),
+        ("m", c_int64),
+        ("n", c_int64),
+        ("k", c_int64),
+        ("lda", c_int64),
+        ("ldb", c_int64),
+        ("ldd", c_int64),
+        ("ldc", c_int64),
+        ("ldct", c_int64),
+        ("batch", c_int64),
+        ("stride_a", c_int64),
+        ("stride_b", c_int64),
+        ("stride_d", c_int64),
+        ("stride_c", c_int64),
+        ("stride_ct", c_int64),
+        ("alpha", c_float),
+        ("beta", c_float),
+    ]
+
+
+# name -> (restype, argtypes); every symbol include/flexshard_hip.h declares.
+SIGNATURES: dict[str, tuple[object, list[object]]] = {
+    "fsh_version": (c_int32, []),
+    "fsh_last_error": (c_char_p, []),
+    "fsh_quantize_pack": (
+        c_int,
+        [POINTER(QuantChunk), c_int32, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int32, c_int32, c_void_p],
+    ),
+    "fsh_copy_segments": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_void_p]),
+    "fsh_zero_segments": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_void_p]),
+    "fsh_pack_segments": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int32, c_void_p, c_void_p],
+    ),
+    "fsh_unpack_dequant": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int32, c_int32, c_void_p],
+    ),
+    "fsh_accumulate_grad": (c_int, [c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p]),
+    "fsh_reduce_rows_f32": (c_int, [c_void_p, c_void_p, c_int64, c_int32, c_int64, c_int64, c_int32, c_float, c_void_p]),
+    "fsh_newton_schulz_workspace_bytes": (c_int64, [c_int64, c_int64, c_int64]),
+    "fsh_newton_schulz": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_int64, c_float, c_float, c_float, c_int32, c_float, c_void_p, c_int64, c_void_p],
+    ),
+    "fsh_gemm_bf16_nt": (c_int, [POINTER(GemmDesc), c_void_p]),
+    "fsh_muon_prepare": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_float, c_float, c_int32, c_void_p]),
+    "fsh_muon_apply": (c_int, [c_void_p, c_void_p, c_int64, c_float, c_float, c_float, c_void_p]),
+}
+
+_LIB: ctypes.CDLL | None = None
+
+
+class NativeError(RuntimeError):
+    """A C-ABI call returned a negative status."""
+
+
+def lib() -> ctypes.CDLL:
+    """Load the shared library once and bind every declared symbol."""
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `make -C flex_shard_amd/csrc` "
+            "(or __graft_entry__.build()). flex_shard_amd has no fallback compute path."
+        )
+    handle = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        try:
+            fn = getattr(handle, name)
+        except AttributeError as exc:
+            raise RuntimeError(f"{LIB_PATH} does not export {name}") from exc
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _LIB = handle
+    return handle
+
+
+def check(status: int, what: str) -> None:
+    if status != FSH_OK:
+        message = lib().fsh_last_error().decode("utf-8", "replace")
+        raise NativeError(f"{what} failed with status {status}: {message}")

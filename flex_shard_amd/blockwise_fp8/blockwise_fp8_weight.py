@@ -1,0 +1,158 @@
+"""Blockwise FP8 weight handed to consumers after an FP8 unshard.
+
+``blockwise_dequant_weight`` and ``BlockwiseFp8Weight`` keep the contract of the
+reference's ``blockwise_fp8/blockwise_fp8_weight.py`` (:25-54, :57-143): a
+tensor-subclass wrapper holding the gathered FP8 data (parameter shape) and the
+fp32 reciprocal scales of its flattened matrix, and a dequantization equal to
+``float32(fp8) * scale(tile)`` rounded once to the requested dtype.  The
+dequantization runs in the HIP unpack kernel.
+"""
+
+from __future__ import annotations
+
+from typing import Any
+
+import torch
+
+from .. import hip_ops
+from ..custom_placements._copy_kernels import _upload_i64
+from ..custom_placements.blockwise_quant_bucketed_block_shard import (
+    _matrix_shape,
+    _scale_shape,
+    _validate_2d_non_empty,
+    _validate_block_size,
+)
+
+
+def _check_scale(quant_shape, recip_scale: torch.Tensor, block_size: int) -> None:
+    expected = _scale_shape(quant_shape, block_size)
+    if tuple(recip_scale.shape) != expected:
+        raise ValueError(
+            f"scale shape must be {expected} for data {tuple(quant_shape)} "
+            f"and block_size {block_size}, got {tuple(recip_scale.shape)}"
+        )
+
+
+def blockwise_dequant_weight(
+    quant: torch.Tensor, recip_scale: torch.Tensor, block_size: int, out_dtype: torch.dtype = torch.float32
+) -> torch.Tensor:
+    """Dequantize a 2-D blockwise FP8 weight on the GPU.  The default output is
+    fp32 (the unrounded product, as the reference returns); bf16 rounds it once."""
+    _validate_block_size(block_size)
+    rows, cols = _validate_2d_non_empty(quant.shape, "blockwise_dequant_weight")
+    _check_scale(quant.shape, recip_scale, block_size)
+    if quant.device.type != "cuda" or recip_scale.device != quant.device:
+        raise RuntimeError("blockwise_dequant_weight runs on the GPU; this package has no CPU compute path.")
+    if quant.dtype not in (torch.float8_e4m3fn, torch.uint8):
+        raise NotImplementedError(f"the HIP dequantizer reads float8_e4m3fn bytes, not {quant.dtype}")
+    data = quant.contiguous().view(torch.uint8).view(-1)
+    scales = recip_scale.to(torch.float32).contiguous().view(-1)
+    tiles = _scale_shape(quant.shape, block_size)
+    # One chunk whose scale block is addressed relative to the data pointer
+    # (both live in the same device address space).
+    scale_delta = scales.data_ptr() - data.data_ptr()
+    table, table_host = _upload_i64([0, scale_delta, rows, cols, 0, 0, 0], quant.device)
+    starts, starts_host = _upload_i64([0, tiles[0] * tiles[1]], quant.device)
+    out = torch.empty(rows * cols, dtype=out_dtype, device=quant.device)
+    hip_ops.unpack_dequant(data, table.view(1, 7), starts, tiles[0] * tiles[1], None, out, block_size)
+    # `scales` and the pinned staging tensors stay referenced until the launch
+    # is queued; the caching allocator keeps their memory valid for it.
+    del table_host, starts_host
+    return out.view(rows, cols)
+
+
+class BlockwiseFp8Weight(torch.Tensor):
+    """Wrapper tensor subclass over FP8 data and per-tile reciprocal scales.
+
+    Stacked weights keep the parameter shape (``[num_linears, out, in]``);
+    their scales cover the flattened ``[num_linears * out, in]`` matrix.
+    """
+
+    __slots__ = ["_data", "_recip_scale", "_block_size", "_orig_dtype"]
+
+    @staticmethod
+    def __new__(
+        cls,
+        data: torch.Tensor,
+        recip_scale: torch.Tensor,
+        block_size: int,
+        orig_dtype: torch.dtype = torch.bfloat16,
+        requires_grad: bool = False,
+    ):
+        return torch.Tensor._make_wrapper_subclass(
+            cls, data.shape, dtype=orig_dtype, device=data.device, requires_grad=requires_grad
+        )
+
+    def __init__(
+        self,
+        data: torch.Tensor,
+        recip_scale: torch.Tensor,
+        block_size: int,
+        orig_dtype: torch.dtype = torch.bfloat16,
+        requires_grad: bool = False,
+    ) -> None:
+        if data.ndim < 2:
+            raise ValueError(f"BlockwiseFp8Weight expects 2D or stacked 2D data, got {data.shape}")
+        if block_size <= 0:
+            raise ValueError(f"block_size must be positive, got {block_size}")
+        _check_scale(_matrix_shape(data.shape), recip_scale, block_size)
+        if data.device != recip_scale.device:
+            raise ValueError(
+                f"data and scale must be on the same device, got {data.device} and {recip_scale.device}"
+            )
+        self._data = data
+        self._recip_scale = recip_scale
+        self._block_size = block_size
+        self._orig_dtype = orig_dtype
+
+    @property
+    def fp8_data(self) -> torch.Tensor:
+        return self._data
+
+    @property
+    def recip_scale(self) -> torch.Tensor:
+        return self._recip_scale
+
+    @property
+    def block_size(self) -> int:
+        return self._block_size
+
+    @property
+    def orig_dtype(self) -> torch.dtype:
+        return self._orig_dtype
+
+    def dequantize(self, dtype: torch.dtype | None = None) -> torch.Tensor:
+        target = dtype or self._orig_dtype
+        kernel_dtype = target if target in (torch.bfloat16, torch.float32) else torch.float32
+        flat = blockwise_dequant_weight(self._data.flatten(0, -2), self._recip_scale, self._block_size, kernel_dtype)
+        return flat.reshape(self._data.shape).to(target)
+
+    def __tensor_flatten__(self) -> tuple[list[str], dict[str, Any]]:
+        return ["_data", "_recip_scale"], {"block_size": self._block_size, "orig_dtype": self._orig_dtype}
+
+    @classmethod
+    def __tensor_unflatten__(cls, inner_tensors, metadata, outer_size, outer_stride):
+        return cls(inner_tensors["_data"], inner_tensors["_recip_scale"], metadata["block_size"], metadata["orig_dtype"])
+
+    @classmethod
+    def __torch_dispatch__(cls, func, types, args=(), kwargs=None):
+        raise NotImplementedError(
+            f"BlockwiseFp8Weight does not implement {func}; call dequantize() or pass fp8_data / recip_scale "
+            "to an FP8 GEMM."
+        )
+
+    def __repr__(self) -> str:  # the default repr would dispatch
+        return (
+            f"BlockwiseFp8Weight(shape={tuple(self.shape)}, block_size={self._block_size}, "
+            f"orig_dtype={self._orig_dtype})"
+        )
+
+
+def make_blockwise_fp8_weight(
+    fp8_data: torch.Tensor, recip_scale: torch.Tensor, block_size: int, *, orig_dtype: torch.dtype, requires_grad: bool
+) -> BlockwiseFp8Weight:
+    """A ``weight_factory`` for ``Fp8BucketedBlockShard`` that views its inputs."""
+    return BlockwiseFp8Weight(fp8_data, recip_scale, block_size, orig_dtype, requires_grad)
+
+
+__all__ = ["BlockwiseFp8Weight", "blockwise_dequant_weight", "make_blockwise_fp8_weight"]

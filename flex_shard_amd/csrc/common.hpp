@@ -1,0 +1,124 @@
+// Shared helpers of the gfx950 kernels: error reporting, launch checks, bit
+// conversions, cooperative byte copy/fill with run-time vector width.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/flexshard_hip.h"
+
+#define FSH_API extern "C" __attribute__((visibility("default")))
+
+namespace fsh {
+
+// Thread-local message of the last failed call.
+char* error_buffer();
+int fail(int code, const char* fmt, ...);
+int check_launch(const char* what);
+
+inline bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+__host__ __device__ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+constexpr int kWave = 64;
+
+// Native vector types (the nontemporal builtins reject HIP's struct vectors).
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// Streaming (nontemporal) 16/8-byte accesses: the hot kernels touch every
+// byte once, so nothing is worth keeping in the caches.
+__device__ __forceinline__ u32x4 load_stream_u32x4(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
+__device__ __forceinline__ f32x4 load_stream_f32x4(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
+}
+__device__ __forceinline__ void store_stream_u32x2(void* p, uint32_t a, uint32_t b) {
+  u32x2 v = {a, b};
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(p));
+}
+__device__ __forceinline__ void store_stream_u32x4(void* p, u32x4 v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+}
+
+// ---------------------------------------------------------------- bit casts
+__device__ __forceinline__ float u32_as_f32(uint32_t u) { return __uint_as_float(u); }
+__device__ __forceinline__ uint32_t f32_as_u32(float f) { return __float_as_uint(f); }
+
+// bf16 bits (low 16 of `h`) -> float, exact.
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return u32_as_f32(h << 16); }
+
+// float -> bf16 bits, round to nearest even, NaN -> 0x7FC0.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = f32_as_u32(f);
+  uint32_t r = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+  return (f != f) ? 0x7FC0u : r;
+}
+
+// Integer max across the 64 lanes of a wavefront.
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    uint32_t o = static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), off, kWave));
+    v = o > v ? o : v;
+  }
+  return v;
+}
+
+__device__ __forceinline__ float wave_sum_f32(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+// ------------------------------------------------- cooperative byte movers
+// All threads of the workgroup call these with identical arguments.  The
+// widest vector the relative alignment of src and dst allows is used for the
+// bulk; unaligned heads and tails move as bytes.
+template <typename V>
+__device__ __forceinline__ void copy_bulk(const uint8_t* src, uint8_t* dst, int64_t n, int tid,
+                                          int nthreads) {
+  // Precondition: src and dst are congruent modulo sizeof(V).
+  int64_t head = (sizeof(V) - (reinterpret_cast<uintptr_t>(dst) & (sizeof(V) - 1))) & (sizeof(V) - 1);
+  if (head > n) head = n;
+  for (int64_t i = tid; i < head; i += nthreads) dst[i] = src[i];
+  const int64_t body = (n - head) / static_cast<int64_t>(sizeof(V));
+  const V* s = reinterpret_cast<const V*>(src + head);
+  V* d = reinterpret_cast<V*>(dst + head);
+  for (int64_t i = tid; i < body; i += nthreads) d[i] = s[i];
+  const int64_t done = head + body * static_cast<int64_t>(sizeof(V));
+  for (int64_t i = done + tid; i < n; i += nthreads) dst[i] = src[i];
+}
+
+__device__ __forceinline__ void copy_bytes(const uint8_t* src, uint8_t* dst, int64_t n, int tid,
+                                           int nthreads) {
+  const uintptr_t rel = reinterpret_cast<uintptr_t>(src) ^ reinterpret_cast<uintptr_t>(dst);
+  if ((rel & 15) == 0)
+    copy_bulk<uint4>(src, dst, n, tid, nthreads);
+  else if ((rel & 7) == 0)
+    copy_bulk<uint2>(src, dst, n, tid, nthreads);
+  else if ((rel & 3) == 0)
+    copy_bulk<uint32_t>(src, dst, n, tid, nthreads);
+  else if ((rel & 1) == 0)
+    copy_bulk<uint16_t>(src, dst, n, tid, nthreads);
+  else
+    for (int64_t i = tid; i < n; i += nthreads) dst[i] = src[i];
+}
+
+__device__ __forceinline__ void zero_bytes(uint8_t* dst, int64_t n, int tid, int nthreads) {
+  int64_t head = (16 - (reinterpret_cast<uintptr_t>(dst) & 15)) & 15;
+  if (head > n) head = n;
+  for (int64_t i = tid; i < head; i += nthreads) dst[i] = 0;
+  const int64_t body = (n - head) / 16;
+  uint4* d = reinterpret_cast<uint4*>(dst + head);
+  const uint4 z = make_uint4(0, 0, 0, 0);
+  for (int64_t i = tid; i < body; i += nthreads) d[i] = z;
+  for (int64_t i = head + body * 16 + tid; i < n; i += nthreads) dst[i] = 0;
+}
+
+}  // namespace fsh

@@ -1,0 +1,374 @@
+// Fused blockwise FP8 (E4M3FN) tile quantization + packing into a rank's
+// flat send payload, one launch per bucket.
+//
+// One workgroup (256 threads = 4 wavefronts) owns one block x block tile of
+// one chunk.  For block = 128 each thread keeps its 64 tile elements in
+// registers between the amax pass and the cast pass, so the tile is read from
+// HBM exactly once: 16-byte loads (8 bf16), amax on raw magnitude bits with
+// packed 16-bit max, a 64-lane shuffle reduction plus a 4-entry LDS exchange,
+// one fp64 division per tile for the scale, then v_cvt_pk_fp8_f32 and 8-byte
+// stores straight into the payload.  Extra workgroups zero the payload's pad
+// gaps, so nothing else has to touch the buffer.
+//
+// Arithmetic contract (bit-exact with the reference's eager quantizer):
+//   amax   = max |x| in the quantization dtype
+//   amax   = amax < eps ? eps : amax            (NaN stays NaN)
+//   scale  = float(448.0 / double(amax))
+//   q      = e4m3fn_rne(float(x) * scale)       (the reference's clamp to
+//            +-448 never changes a finite product: |x| <= amax bounds it by
+//            448 * (1 + 2^-23), which rounds to 448 either way)
+//   stored = 1.0f / scale                       (IEEE fp32 division)
+#include "common.hpp"
+
+namespace fsh {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int64_t kZeroChunk = 65536;  // bytes zeroed per pad workgroup
+
+struct QuantChunkDev {
+  const uint8_t* src;
+  int64_t rows;
+  int64_t in_dim;
+  int64_t src_row_stride;  // elements
+  int64_t qdata_offset;
+  int64_t scale_offset;
+  int64_t tile_begin;  // index of the chunk's first tile in the launch
+  int32_t tiles_c;
+  int32_t src_kind;
+  int32_t fast;  // 128x128 vector path is legal for this chunk
+  int32_t pad_;
+};
+
+struct QuantParams {
+  QuantChunkDev chunks[FSH_MAX_QUANT_CHUNKS];
+  uint8_t* payload;
+  int64_t total_tiles;
+  int64_t zero_begin[2];
+  int64_t zero_len[2];
+  float eps[3];  // indexed by src_kind
+  int32_t nchunks;
+  int32_t block;
+};
+
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+  u16x2 va = __builtin_bit_cast(u16x2, a);
+  u16x2 vb = __builtin_bit_cast(u16x2, b);
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(va, vb));
+}
+
+// Two floats -> two E4M3FN bytes in the low (hi=false) or high half of `old`.
+__device__ __forceinline__ uint32_t cvt2_fp8(float a, float b, uint32_t old, bool hi) {
+  return hi ? static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, static_cast<int>(old), true))
+            : static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, static_cast<int>(old), false));
+}
+
+// Scale pair of a tile from its amax; identical on every lane.
+__device__ __forceinline__ void tile_scale(float amax, float eps, float& scale, float& recip) {
+  const float floored = (amax < eps) ? eps : amax;  // NaN fails the test and stays
+  scale = static_cast<float>(448.0 / static_cast<double>(floored));
+  recip = 1.0f / scale;
+}
+
+// Workgroup-wide maximum of one magnitude word per thread.
+__device__ __forceinline__ uint32_t block_max_u32(uint32_t v, uint32_t* lds) {
+  v = wave_max_u32(v);
+  const int tid = threadIdx.x;
+  if ((tid & 63) == 0) lds[tid >> 6] = v;
+  __syncthreads();
+  uint32_t a = lds[0] > lds[1] ? lds[0] : lds[1];
+  uint32_t b = lds[2] > lds[3] ? lds[2] : lds[3];
+  return a > b ? a : b;
+}
+
+// ---------------------------------------------------------------- fast path
+// Thread t owns columns 8*(t%16) .. +7 of rows (t/16) + 16k, k = 0..7.
+// Per load instruction a wavefront reads four full 256-byte tile rows.
+
+// bf16 source, or fp32 master rounded to bf16 on load: the tile lives in
+// registers as 32 dwords of packed bf16.
+template <int KIND>
+__device__ __forceinline__ void quant_tile128_bf16(const QuantChunkDev& ch, int64_t tr, int64_t tc,
+                                                   uint8_t* payload, float eps, uint32_t* lds) {
+  const int tid = threadIdx.x;
+  const int g = tid & 15;
+  const int r0 = tid >> 4;
+  const int64_t row_base = tr * 128 + r0;
+  const int64_t col = tc * 128 + g * 8;
+  const bool col_ok = col < ch.in_dim;
+
+  u32x4 v[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int64_t row = row_base + 16 * k;
+    v[k] = u32x4{0, 0, 0, 0};
+    if (col_ok && row < ch.rows) {
+      if (KIND == FSH_SRC_BF16) {
+        v[k] = load_stream_u32x4(ch.src + (row * ch.src_row_stride + col) * 2);
+      } else {
+        const uint8_t* p = ch.src + (row * ch.src_row_stride + col) * 4;
+        const f32x4 a = load_stream_f32x4(p);
+        const f32x4 b = load_stream_f32x4(p + 16);
+        v[k].x = f32_to_bf16_bits(a.x) | (f32_to_bf16_bits(a.y) << 16);
+        v[k].y = f32_to_bf16_bits(a.z) | (f32_to_bf16_bits(a.w) << 16);
+        v[k].z = f32_to_bf16_bits(b.x) | (f32_to_bf16_bits(b.y) << 16);
+        v[k].w = f32_to_bf16_bits(b.z) | (f32_to_bf16_bits(b.w) << 16);
+      }
+    }
+  }
+
+  // |x| as raw 15-bit magnitudes: integer order equals float order, and any
+  // NaN pattern exceeds infinity, so a NaN in the tile surfaces as a NaN amax.
+  uint32_t m = 0;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    m = pk_max_u16(m, v[k].x & 0x7FFF7FFFu);
+    m = pk_max_u16(m, v[k].y & 0x7FFF7FFFu);
+    m = pk_max_u16(m, v[k].z & 0x7FFF7FFFu);
+    m = pk_max_u16(m, v[k].w & 0x7FFF7FFFu);
+  }
+  const uint32_t lo = m & 0xFFFFu, hi = m >> 16;
+  m = block_max_u32(lo > hi ? lo : hi, lds);
+
+  float scale, recip;
+  tile_scale(bf16_bits_to_f32(m), eps, scale, recip);
+  if (tid == 0)
+    *reinterpret_cast<float*>(payload + ch.scale_offset + 4 * (tr * ch.tiles_c + tc)) = recip;
+
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int64_t row = row_base + 16 * k;
+    if (col_ok && row < ch.rows) {
+      const uint32_t d[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+      uint32_t w[2] = {0, 0};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float e0 = u32_as_f32(d[j] << 16) * scale;
+        const float e1 = u32_as_f32(d[j] & 0xFFFF0000u) * scale;
+        w[j >> 1] = cvt2_fp8(e0, e1, w[j >> 1], (j & 1) != 0);
+      }
+      store_stream_u32x2(payload + ch.qdata_offset + row * ch.in_dim + col, w[0], w[1]);
+    }
+  }
+}
+
+// fp32 source quantized as fp32: 64 floats per thread.
+__device__ __forceinline__ void quant_tile128_f32(const QuantChunkDev& ch, int64_t tr, int64_t tc,
+                                                  uint8_t* payload, float eps, uint32_t* lds) {
+  const int tid = threadIdx.x;
+  const int g = tid & 15;
+  const int r0 = tid >> 4;
+  const int64_t row_base = tr * 128 + r0;
+  const int64_t col = tc * 128 + g * 8;
+  const bool col_ok = col < ch.in_dim;
+
+  f32x4 v[8][2];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int64_t row = row_base + 16 * k;
+    v[k][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+    v[k][1] = v[k][0];
+    if (col_ok && row < ch.rows) {
+      const uint8_t* p = ch.src + (row * ch.src_row_stride + col) * 4;
+      v[k][0] = load_stream_f32x4(p);
+      v[k][1] = load_stream_f32x4(p + 16);
+    }
+  }
+  uint32_t m = 0;
+#pragma unroll
+  for (int k = 0; k < 8; ++k)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const float e[4] = {v[k][h].x, v[k][h].y, v[k][h].z, v[k][h].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t mag = f32_as_u32(e[j]) & 0x7FFFFFFFu;
+        m = mag > m ? mag : m;
+      }
+    }
+  m = block_max_u32(m, lds);
+
+  float scale, recip;
+  tile_scale(u32_as_f32(m), eps, scale, recip);
+  if (tid == 0)
+    *reinterpret_cast<float*>(payload + ch.scale_offset + 4 * (tr * ch.tiles_c + tc)) = recip;
+
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int64_t row = row_base + 16 * k;
+    if (col_ok && row < ch.rows) {
+      uint32_t w[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        uint32_t packed = 0;
+        packed = cvt2_fp8(v[k][h].x * scale, v[k][h].y * scale, packed, false);
+        packed = cvt2_fp8(v[k][h].z * scale, v[k][h].w * scale, packed, true);
+        w[h] = packed;
+      }
+      store_stream_u32x2(payload + ch.qdata_offset + row * ch.in_dim + col, w[0], w[1]);
+    }
+  }
+}
+
+// ------------------------------------------------------------- scalar path
+// Any block size, any alignment: two passes over the tile with element loads.
+__device__ __forceinline__ float load_as_quant_dtype(const QuantChunkDev& ch, int64_t row, int64_t col) {
+  const int64_t idx = row * ch.src_row_stride + col;
+  if (ch.src_kind == FSH_SRC_BF16)
+    return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(ch.src)[idx]);
+  const float f = reinterpret_cast<const float*>(ch.src)[idx];
+  if (ch.src_kind == FSH_SRC_F32_AS_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(f));
+  return f;
+}
+
+__device__ void quant_tile_scalar(const QuantChunkDev& ch, int64_t tr, int64_t tc, int block,
+                                  uint8_t* payload, float eps, uint32_t* lds) {
+  const int tid = threadIdx.x;
+  const int64_t row0 = tr * block, col0 = tc * block;
+  const int64_t nrows = (ch.rows - row0) < block ? (ch.rows - row0) : block;
+  const int64_t ncols = (ch.in_dim - col0) < block ? (ch.in_dim - col0) : block;
+  const int64_t n = nrows * ncols;
+  uint32_t m = 0;
+  for (int64_t i = tid; i < n; i += kThreads) {
+    const uint32_t mag = f32_as_u32(load_as_quant_dtype(ch, row0 + i / ncols, col0 + i % ncols)) & 0x7FFFFFFFu;
+    m = mag > m ? mag : m;
+  }
+  m = block_max_u32(m, lds);
+  float scale, recip;
+  tile_scale(u32_as_f32(m), eps, scale, recip);
+  if (tid == 0)
+    *reinterpret_cast<float*>(payload + ch.scale_offset + 4 * (tr * ch.tiles_c + tc)) = recip;
+  for (int64_t i = tid; i < n; i += kThreads) {
+    const int64_t row = row0 + i / ncols, col = col0 + i % ncols;
+    const float p = load_as_quant_dtype(ch, row, col) * scale;
+    payload[ch.qdata_offset + row * ch.in_dim + col] = static_cast<uint8_t>(cvt2_fp8(p, 0.0f, 0u, false) & 0xFFu);
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void quantize_pack_kernel(const QuantParams prm) {
+  __shared__ uint32_t lds[4];
+  const int64_t bid = blockIdx.x;
+  if (bid >= prm.total_tiles) {
+    // Pad workgroups: zero a slice of the two pad ranges laid end to end.
+    const int64_t begin = (bid - prm.total_tiles) * kZeroChunk;
+    const int64_t end = begin + kZeroChunk;
+    int64_t base = 0;
+#pragma unroll
+    for (int z = 0; z < 2; ++z) {
+      const int64_t lo = begin > base ? begin : base;
+      const int64_t limit = base + prm.zero_len[z];
+      const int64_t hi = end < limit ? end : limit;
+      if (lo < hi) zero_bytes(prm.payload + prm.zero_begin[z] + (lo - base), hi - lo, threadIdx.x, kThreads);
+      base = limit;
+    }
+    return;
+  }
+  int c = 0;
+  while (c + 1 < prm.nchunks && bid >= prm.chunks[c + 1].tile_begin) ++c;
+  const QuantChunkDev& ch = prm.chunks[c];
+  const int64_t t = bid - ch.tile_begin;
+  const int64_t tr = t / ch.tiles_c;
+  const int64_t tc = t - tr * ch.tiles_c;
+  const float eps = prm.eps[ch.src_kind];
+  if (ch.fast) {
+    if (ch.src_kind == FSH_SRC_BF16)
+      quant_tile128_bf16<FSH_SRC_BF16>(ch, tr, tc, prm.payload, eps, lds);
+    else if (ch.src_kind == FSH_SRC_F32_AS_BF16)
+      quant_tile128_bf16<FSH_SRC_F32_AS_BF16>(ch, tr, tc, prm.payload, eps, lds);
+    else
+      quant_tile128_f32(ch, tr, tc, prm.payload, eps, lds);
+  } else {
+    quant_tile_scalar(ch, tr, tc, prm.block, prm.payload, eps, lds);
+  }
+}
+
+float bf16_round_host(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  u = (u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+}  // namespace
+}  // namespace fsh
+
+FSH_API int fsh_quantize_pack(const fsh_quant_chunk* chunks, int32_t nchunks, void* payload_dev,
+                              int64_t payload_nbytes, int64_t zero0_begin, int64_t zero0_end,
+                              int64_t zero1_begin, int64_t zero1_end, int32_t block,
+                              int32_t eps_mode, void* stream) {
+  using namespace fsh;
+  if (nchunks < 0 || nchunks > FSH_MAX_QUANT_CHUNKS)
+    return fail(FSH_EINVAL, "fsh_quantize_pack: nchunks %d outside [0, %d]", nchunks, FSH_MAX_QUANT_CHUNKS);
+  if (nchunks > 0 && chunks == nullptr) return fail(FSH_EINVAL, "fsh_quantize_pack: null chunk table");
+  if (block <= 0) return fail(FSH_EINVAL, "fsh_quantize_pack: block must be positive, got %d", block);
+  if (eps_mode != FSH_EPS_INPUT_DTYPE && eps_mode != FSH_EPS_FP32)
+    return fail(FSH_EINVAL, "fsh_quantize_pack: unknown eps_mode %d", eps_mode);
+  if (payload_nbytes < 0 || (payload_nbytes > 0 && payload_dev == nullptr))
+    return fail(FSH_EINVAL, "fsh_quantize_pack: bad payload");
+  if (!aligned(payload_dev, 16)) return fail(FSH_EINVAL, "fsh_quantize_pack: payload must be 16-byte aligned");
+  const int64_t zb[2] = {zero0_begin, zero1_begin}, ze[2] = {zero0_end, zero1_end};
+  for (int z = 0; z < 2; ++z)
+    if (zb[z] < 0 || ze[z] < zb[z] || ze[z] > payload_nbytes)
+      return fail(FSH_EINVAL, "fsh_quantize_pack: zero range %d [%lld, %lld) outside payload of %lld bytes", z,
+                  (long long)zb[z], (long long)ze[z], (long long)payload_nbytes);
+
+  QuantParams prm;
+  memset(&prm, 0, sizeof(prm));
+  prm.payload = static_cast<uint8_t*>(payload_dev);
+  prm.nchunks = nchunks;
+  prm.block = block;
+  const float eps32 = 1e-12f;
+  const float eps_bf16 = eps_mode == FSH_EPS_FP32 ? eps32 : bf16_round_host(eps32);
+  prm.eps[FSH_SRC_BF16] = eps_bf16;
+  prm.eps[FSH_SRC_F32] = eps32;
+  prm.eps[FSH_SRC_F32_AS_BF16] = eps_bf16;
+
+  int64_t tiles = 0;
+  for (int i = 0; i < nchunks; ++i) {
+    const fsh_quant_chunk& in = chunks[i];
+    if (in.src_dev == nullptr || in.rows <= 0 || in.in_dim <= 0 || in.src_row_stride < in.in_dim)
+      return fail(FSH_EINVAL, "fsh_quantize_pack: chunk %d has bad shape (rows %lld, in_dim %lld, stride %lld)", i,
+                  (long long)in.rows, (long long)in.in_dim, (long long)in.src_row_stride);
+    if (in.src_kind < 0 || in.src_kind > FSH_SRC_F32_AS_BF16)
+      return fail(FSH_EINVAL, "fsh_quantize_pack: chunk %d has unknown src_kind %d", i, in.src_kind);
+    const int64_t tiles_r = ceil_div(in.rows, block), tiles_c = ceil_div(in.in_dim, block);
+    if (in.qdata_offset < 0 || in.qdata_offset + in.rows * in.in_dim > payload_nbytes)
+      return fail(FSH_EINVAL, "fsh_quantize_pack: chunk %d data [%lld, +%lld) outside payload", i,
+                  (long long)in.qdata_offset, (long long)(in.rows * in.in_dim));
+    if (in.scale_offset < 0 || (in.scale_offset & 3) != 0 ||
+        in.scale_offset + 4 * tiles_r * tiles_c > payload_nbytes)
+      return fail(FSH_EINVAL, "fsh_quantize_pack: chunk %d scales at %lld misaligned or outside payload", i,
+                  (long long)in.scale_offset);
+    const int64_t elem = in.src_kind == FSH_SRC_BF16 ? 2 : 4;
+    if (!aligned(in.src_dev, elem)) return fail(FSH_EINVAL, "fsh_quantize_pack: chunk %d source misaligned", i);
+    QuantChunkDev& out = prm.chunks[i];
+    out.src = static_cast<const uint8_t*>(in.src_dev);
+    out.rows = in.rows;
+    out.in_dim = in.in_dim;
+    out.src_row_stride = in.src_row_stride;
+    out.qdata_offset = in.qdata_offset;
+    out.scale_offset = in.scale_offset;
+    out.tile_begin = tiles;
+    out.tiles_c = static_cast<int32_t>(tiles_c);
+    out.src_kind = in.src_kind;
+    out.fast = block == 128 && aligned(in.src_dev, 16) && (in.src_row_stride * elem) % 16 == 0 &&
+               in.in_dim % 8 == 0 && in.qdata_offset % 8 == 0;
+    tiles += tiles_r * tiles_c;
+  }
+  prm.total_tiles = tiles;
+  int64_t zero_total = 0;
+  for (int z = 0; z < 2; ++z) {
+    prm.zero_begin[z] = zb[z];
+    prm.zero_len[z] = ze[z] - zb[z];
+    zero_total += prm.zero_len[z];
+  }
+  const int64_t grid = tiles + ceil_div(zero_total, kZeroChunk);
+  if (grid == 0) return FSH_OK;
+  if (grid > 0x7FFFFFFFLL) return fail(FSH_ENOTSUP, "fsh_quantize_pack: %lld workgroups exceed the grid limit", (long long)grid);
+  hipLaunchKernelGGL(quantize_pack_kernel, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), 0,
+                     static_cast<hipStream_t>(stream), prm);
+  return check_launch("fsh_quantize_pack");
+}

@@ -1,0 +1,777 @@
+"""Quantized all-gather on bucketed block sharding with blockwise scales.
+
+``BlockwiseQuantBucketedBlockShard`` keeps the reference's surface
+(custom_placements/blockwise_quant_bucketed_block_shard.py:154-1511): a bucket
+is cut into contiguous runs of ``shard_block_rows``-row units over the dense
+parameters, every rank owns whole block rows and quantizes its own shard with
+no cross-rank amax, and the gathered weight is bit-identical to "all-gather
+the dense weights, then quantize".
+
+What differs is the device work.  The local send payload is produced by *one*
+HIP launch (tile quantize fused with packing and pad zeroing) instead of one
+quantizer launch per chunk plus two foreach copies, and the gathered rank rows
+are compacted by one segment-copy launch, optionally fused with dequantization
+(``finish_prepared_unshard_with_dequant``).  There is no CPU compute path:
+tensors off the GPU raise.
+"""
+
+from __future__ import annotations
+
+from collections.abc import Sequence
+from dataclasses import dataclass
+from typing import TYPE_CHECKING, Any
+
+import torch
+import torch.distributed as dist
+import torch.nn as nn
+
+from .. import hip_ops
+from ..placement_contract import (
+    BucketParamStorageLayout,
+    BucketStorageLayout,
+    GlobalLayout,
+    PlacementPreparedUnshard,
+    PlacementUnshardResult,
+)
+from ..profiling import record_comm, record_copy_in, record_copy_out
+from . import quant_plan
+from ._copy_kernels import SegmentCopyDescriptor, copy_segments
+from .block_shard import BucketedBlockShard
+from .quant_plan import ScaleRegion as _ScaleRegion
+from .quant_plan import align_up as _align_up
+from .quant_plan import ceil_div as _ceil_div
+from .quant_plan import matrix_shape as _matrix_shape
+
+if TYPE_CHECKING:
+    from ..bucket_storage import ParamInfo
+    from ..placement_contract import Placement
+
+_VEC_COPY_DTYPE = torch.int32
+_VEC_COPY_NBYTES = _VEC_COPY_DTYPE.itemsize
+_VEC_ALIGN_BYTES = quant_plan.VEC_ALIGN_BYTES
+
+
+def _validate_block_size(block_size: int) -> None:
+    if not isinstance(block_size, int):
+        raise TypeError(f"block_size must be an int, got {type(block_size).__name__}")
+    if block_size <= 0:
+        raise ValueError(f"block_size must be positive, got {block_size}")
+
+
+def _validate_2d_non_empty(shape: Sequence[int], what: str) -> tuple[int, int]:
+    if len(shape) != 2:
+        raise ValueError(f"{what} expects 2D, got {tuple(shape)}")
+    rows, cols = shape
+    if rows <= 0 or cols <= 0:
+        raise ValueError(f"{what} requires non-empty 2D shape, got {tuple(shape)}")
+    return rows, cols
+
+
+def _unravel_index(index: int, shape: Sequence[int]) -> tuple[int, ...]:
+    coords = []
+    for size in reversed(shape):
+        index, coord = divmod(index, size)
+        coords.append(coord)
+    return tuple(reversed(coords))
+
+
+def _scale_shape(shape: Sequence[int], block_size: int) -> tuple[int, int]:
+    _validate_block_size(block_size)
+    rows, cols = _validate_2d_non_empty(shape, "blockwise scale")
+    return _ceil_div(rows, block_size), _ceil_div(cols, block_size)
+
+
+def _padded_shape(shape: Sequence[int], block_size: int) -> tuple[int, int]:
+    tiles_r, tiles_c = _scale_shape(shape, block_size)
+    return tiles_r * block_size, tiles_c * block_size
+
+
+def _callable_name(value: Any) -> str:
+    return getattr(value, "__qualname__", type(value).__qualname__)
+
+
+def _is_vec_copy_viewable(tensor: torch.Tensor) -> bool:
+    """Whether a uint8 tensor can be viewed as int32 (torch's dtype-view rules)."""
+    if torch.compiler.is_compiling():
+        return False
+    return (
+        tensor.dtype == torch.uint8
+        and tensor.ndim > 0
+        and tensor.stride(-1) == 1
+        and tensor.size(-1) % _VEC_COPY_NBYTES == 0
+        and tensor.storage_offset() % _VEC_COPY_NBYTES == 0
+        and all(stride % _VEC_COPY_NBYTES == 0 for stride in tensor.stride()[:-1])
+    )
+
+
+def _is_backward_graph_task() -> bool:
+    return torch._C._current_graph_task_id() >= 0
+
+
+def _require_gpu_rows(tensor: torch.Tensor, what: str) -> None:
+    if tensor.device.type != "cuda":
+        raise RuntimeError(
+            f"{what} runs on the GPU through libflexshard_hip.so; got a tensor on {tensor.device}. "
+            "This package has no CPU compute path."
+        )
+
+
+class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
+    """Bucketed block shard that all-gathers blockwise-quantized weights.
+
+    Subclasses define the format: ``_chunk_scale_numels``, ``_param_scale_view``,
+    ``_make_quantized_weight`` and the device hooks ``_quantize_pack_source_kind``
+    / ``_launch_quantize_pack``; ``_scale_regions`` may be overridden for scale
+    tensors whose per-rank chunks do not concatenate flat.
+    """
+
+    qdata_dtype: torch.dtype
+    scale_dtype: torch.dtype
+    num_scale_tensors: int = 1
+
+    _BlockRowParam = quant_plan.BlockRowParam
+    _BlockRowUnit = quant_plan.BlockRowUnit
+    _QuantChunk = quant_plan.QuantChunk
+    _QuantPackChunk = quant_plan.QuantPackChunk
+    _QuantRankPackPlan = quant_plan.QuantRankPackPlan
+    _QuantBucketMetadata = quant_plan.QuantBucketMetadata
+
+    @dataclass(frozen=True)
+    class _QuantMetadataPlan:
+        bucket_layout: Any
+        metadata: quant_plan.QuantBucketMetadata
+
+    @dataclass(frozen=True)
+    class _QuantUnshardState:
+        infos: list
+        pg: Any
+        debug_fqn: str | None
+        metadata: quant_plan.QuantBucketMetadata
+
+    @dataclass(frozen=True)
+    class _CopyOutPlan:
+        """Payload regions ``(rank, row byte offset, nbytes, out byte offset)``
+        of one bucket, with device descriptors keyed by (device, row stride,
+        copy unit) in bytes."""
+
+        metadata: quant_plan.QuantBucketMetadata
+        regions: tuple[tuple[int, int, int, int], ...]
+        vec_aligned: bool
+        descriptors: dict
+
+    @dataclass(frozen=True)
+    class _LocalPackedSourceState:
+        storage: Any
+        version: int
+        storage_offset: int
+        shape: torch.Size
+        stride: tuple[int, ...]
+        dtype: torch.dtype
+        is_conj: bool
+        is_neg: bool
+
+    @dataclass(frozen=True)
+    class _LocalPackedInfoState:
+        info: Any
+        unsharded_dtype: torch.dtype
+
+    @dataclass(frozen=True)
+    class _LocalPackedCacheEntry:
+        info_states: tuple
+        source_states: tuple
+        metadata: quant_plan.QuantBucketMetadata
+        packed: torch.Tensor
+
+    def __init__(self, *, world_size: int, shard_block_rows: int, qdata_dtype: torch.dtype) -> None:
+        if world_size <= 0:
+            raise ValueError(f"{type(self).__name__} world_size must be positive, got {world_size}.")
+        super().__init__(blocks_per_rank=(1,) * world_size)
+        _validate_block_size(shard_block_rows)
+        if qdata_dtype.itemsize != 1:
+            raise ValueError(f"{type(self).__name__} requires a one-byte qdata_dtype, got {qdata_dtype}.")
+        self.qdata_dtype = qdata_dtype
+        self.shard_block_rows = shard_block_rows
+        self._metadata_plans: dict[int, BlockwiseQuantBucketedBlockShard._QuantMetadataPlan] = {}
+        self._local_packed_cache: dict = {}
+        self._copy_out_plans: dict = {}
+        self._unpack_tables: dict = {}
+
+    @property
+    def world_size(self) -> int:
+        return len(self.blocks_per_rank)
+
+    @property
+    def _scale_itemsize(self) -> int:
+        return self.scale_dtype.itemsize
+
+    # ------------------------------------------------------------ format hooks
+    def _chunk_scale_numels(self, rows: int, in_dim: int) -> tuple[int, ...]:
+        """Element count of each scale tensor of a chunk starting on a unit edge."""
+        raise NotImplementedError
+
+    def _scale_regions(
+        self, scale_index: int, rank_pack_plans: tuple[quant_plan.QuantRankPackPlan, ...]
+    ) -> tuple[_ScaleRegion, ...]:
+        """Regions whose concatenation yields scale tensor ``scale_index`` of
+        every parameter in parameter order."""
+        return quant_plan.default_scale_regions(scale_index, rank_pack_plans, self._scale_itemsize)
+
+    def _param_scale_view(self, scale_index: int, scale: torch.Tensor, matrix_shape: torch.Size) -> torch.Tensor:
+        raise NotImplementedError
+
+    def _make_quantized_weight(
+        self, qdata: torch.Tensor, scales: tuple[torch.Tensor, ...], *, orig_dtype: torch.dtype, requires_grad: bool
+    ) -> torch.Tensor:
+        raise NotImplementedError
+
+    def _quantize_pack_source_kind(self, tensor_dtype: torch.dtype, quant_dtype: torch.dtype) -> int | None:
+        """The kernel's source kind for a shard stored in ``tensor_dtype`` and
+        quantized as ``quant_dtype``; None when the shard must be cast first."""
+        raise NotImplementedError
+
+    def _launch_quantize_pack(
+        self,
+        specs: list[hip_ops.QuantChunkSpec],
+        payload: torch.Tensor,
+        zero_ranges: tuple[tuple[int, int], tuple[int, int]],
+    ) -> None:
+        """Queue the format's fused quantize + pack kernel."""
+        raise NotImplementedError
+
+    # ----------------------------------------------------------------- planner
+    _can_partition_units = staticmethod(quant_plan.can_partition_units)
+    _min_partition_capacity = staticmethod(quant_plan.min_partition_capacity)
+    _rank_unit_cuts = staticmethod(quant_plan.rank_unit_cuts)
+
+    def _validate_param_shape(self, fqn: str, shape: Sequence[int]) -> None:
+        if len(shape) < 2:
+            raise ValueError(
+                f"{type(self).__name__} only supports 2D or stacked 2D weights, "
+                f"but {fqn!r} has shape {tuple(shape)}."
+            )
+        if 0 in shape:
+            raise ValueError(
+                f"{type(self).__name__} requires non-empty weights, but {fqn!r} has shape {tuple(shape)}."
+            )
+
+    def _build_block_row_units(self, params: Sequence[quant_plan.BlockRowParam]) -> list[quant_plan.BlockRowUnit]:
+        return quant_plan.build_block_row_units(
+            params, self.shard_block_rows, self.qdata_dtype.itemsize, self._scale_itemsize, self._chunk_scale_numels
+        )
+
+    def _block_row_params_from_named(
+        self,
+        named_params: list[tuple[str, nn.Parameter]],
+        param_placements: dict[str, tuple["Placement", ...]],
+    ) -> tuple[list[quant_plan.BlockRowParam], list[quant_plan.BlockRowUnit]]:
+        first_fqn, first = named_params[0]
+        params = []
+        offset = 0
+        for fqn, param in named_params:
+            if param.dtype != first.dtype:
+                raise ValueError(
+                    f"{type(self).__name__} requires one dtype per bucket: {first_fqn!r} uses {first.dtype} "
+                    f"but {fqn!r} uses {param.dtype}."
+                )
+            if param_placements[fqn] != (self,):
+                raise ValueError(
+                    f"{type(self).__name__} requires the same placement instance for every parameter "
+                    f"in a bucket; {fqn!r} uses {param_placements[fqn]!r}."
+                )
+            self._validate_param_shape(fqn, param.shape)
+            params.append(quant_plan.BlockRowParam(fqn=fqn, global_shape=param.shape, param_offset=offset))
+            offset += param.numel()
+        return params, self._build_block_row_units(params)
+
+    def _block_row_params_from_infos(
+        self, infos: list["ParamInfo"]
+    ) -> tuple[list[quant_plan.BlockRowParam], list[quant_plan.BlockRowUnit]]:
+        layout = self._bucket_layout(infos[0])
+        params = []
+        for info in infos:
+            self._validate_param_shape(info.fqn, info.global_shape)
+            params.append(
+                quant_plan.BlockRowParam(
+                    fqn=info.fqn,
+                    global_shape=info.global_shape,
+                    param_offset=layout.param_layouts[info.fqn].param_offset,
+                )
+            )
+        return params, self._build_block_row_units(params)
+
+    def _build_quant_metadata(
+        self,
+        params: Sequence[quant_plan.BlockRowParam],
+        units: Sequence[quant_plan.BlockRowUnit],
+        unit_cuts: Sequence[int],
+    ) -> quant_plan.QuantBucketMetadata:
+        return quant_plan.build_quant_metadata(
+            params,
+            units,
+            unit_cuts,
+            scale_itemsize=self._scale_itemsize,
+            num_scale_tensors=self.num_scale_tensors,
+            chunk_scale_numels=self._chunk_scale_numels,
+            scale_regions=self._scale_regions,
+        )
+
+    def _unit_cuts_from_rank_layout(
+        self, units: Sequence[quant_plan.BlockRowUnit], rank_offsets: Sequence[int], rank_numels: Sequence[int]
+    ) -> tuple[int, ...]:
+        return quant_plan.unit_cuts_from_rank_layout(units, rank_offsets, rank_numels)
+
+    def _quant_metadata_from_infos(self, infos: list["ParamInfo"]) -> quant_plan.QuantBucketMetadata:
+        layout = self._bucket_layout(infos[0])
+        plan = self._metadata_plans.get(id(layout))
+        if plan is not None and plan.bucket_layout is layout:
+            return plan.metadata
+        params, units = self._block_row_params_from_infos(infos)
+        cuts = self._unit_cuts_from_rank_layout(units, layout.rank_offsets, layout.rank_numels)
+        metadata = self._build_quant_metadata(params, units, cuts)
+        self._metadata_plans[id(layout)] = self._QuantMetadataPlan(bucket_layout=layout, metadata=metadata)
+        return metadata
+
+    def _chunk_numel(self, chunk: quant_plan.QuantChunk, in_dim: int) -> int:
+        return (chunk.row_end - chunk.row_start) * in_dim
+
+    # ---------------------------------------------------- storage / checkpoint
+    def bucket_storage_layout(
+        self,
+        named_params: list[tuple[str, nn.Parameter]],
+        param_placements: dict[str, tuple["Placement", ...]],
+        mesh: Any,
+    ) -> BucketStorageLayout:
+        from ..bucket_storage import BucketLayout, BucketParamLayout
+
+        if not named_params:
+            return BucketStorageLayout(param_layouts={}, total_bytes=0)
+        world_size = mesh.size()
+        self._validate_world_size(world_size)
+        rank = mesh.get_local_rank()
+        dtype = named_params[0][1].dtype
+        params, units = self._block_row_params_from_named(named_params, param_placements)
+        costs = [u.cost_bytes for u in units]
+        cuts = self._rank_unit_cuts(costs, world_size, self._min_partition_capacity(costs, world_size))
+        edges = [0]
+        for unit in units:
+            edges.append(edges[-1] + unit.dense_numel)
+        rank_offsets = tuple(edges[c] for c in cuts[:-1])
+        rank_numels = tuple(edges[hi] - edges[lo] for lo, hi in zip(cuts[:-1], cuts[1:], strict=True))
+        metadata = self._build_quant_metadata(params, units, cuts)
+        mine = {chunk.fqn: chunk for chunk in metadata.chunks if chunk.rank == rank}
+
+        bucket_params: dict[str, BucketParamLayout] = {}
+        shard_layouts: dict[str, tuple[torch.Size, int, int]] = {}
+        for param in params:
+            # A local shard is a row range of the flattened matrix; stacked
+            # dims stay as size-1 dims so the shard keeps the parameter's rank.
+            lead = (1,) * (len(param.global_shape) - 2)
+            in_dim = param.global_shape[-1]
+            chunk = mine.get(param.fqn)
+            if chunk is None:
+                shard_layouts[param.fqn] = (torch.Size([*lead, 0, in_dim]), 0, 0)
+                local_start = param.param_offset
+            else:
+                rows = chunk.row_end - chunk.row_start
+                shard_layouts[param.fqn] = (
+                    torch.Size([*lead, rows, in_dim]),
+                    rows * in_dim,
+                    chunk.rank_dense_offset * dtype.itemsize,
+                )
+                local_start = chunk.global_dense_offset
+            bucket_params[param.fqn] = BucketParamLayout(param_offset=param.param_offset, local_global_offset=local_start)
+
+        bucket_layout = BucketLayout(
+            global_numel=edges[-1],
+            local_numel=rank_numels[rank],
+            rank_offsets=rank_offsets,
+            rank_numels=rank_numels,
+            param_layouts=bucket_params,
+        )
+        self._metadata_plans[id(bucket_layout)] = self._QuantMetadataPlan(bucket_layout=bucket_layout, metadata=metadata)
+        return BucketStorageLayout(
+            param_layouts={
+                fqn: BucketParamStorageLayout(
+                    local_shape=shape,
+                    local_numel=numel,
+                    byte_offset=byte_offset,
+                    storage_nbytes=numel * dtype.itemsize,
+                    bucket_layout=bucket_layout,
+                )
+                for fqn, (shape, numel, byte_offset) in shard_layouts.items()
+            },
+            total_bytes=rank_numels[rank] * dtype.itemsize,
+        )
+
+    def global_layout(self, info: "ParamInfo", rank: int, world_size: int) -> GlobalLayout:
+        """One box per stacked matrix this rank's row range touches."""
+        shape = tuple(info.global_shape)
+        if info.local_numel == 0:
+            return GlobalLayout(shape, (), (), ())
+        *stack, out_dim, in_dim = shape
+        layout = self._param_layout(info)
+        row_lo = (layout.local_global_offset - layout.param_offset) // in_dim
+        row_hi = row_lo + info.local_numel // in_dim
+        zeros, ones = (0,) * len(stack), (1,) * len(stack)
+        g_off, l_off, sizes = [], [], []
+        for matrix in range(row_lo // out_dim, _ceil_div(row_hi, out_dim)):
+            base = matrix * out_dim
+            lo, hi = max(row_lo, base), min(row_hi, base + out_dim)
+            g_off.append((*_unravel_index(matrix, stack), lo - base, 0))
+            l_off.append((*zeros, lo - row_lo, 0))
+            sizes.append((*ones, hi - lo, in_dim))
+        return GlobalLayout(shape, tuple(g_off), tuple(l_off), tuple(sizes))
+
+    # ------------------------------------------------ local quantize + pack
+    @staticmethod
+    def _local_packed_source_state(tensor: torch.Tensor) -> "_LocalPackedSourceState":
+        # Holding the storage keeps its address from being reused by another
+        # tensor, which would otherwise look like an unchanged source.
+        return BlockwiseQuantBucketedBlockShard._LocalPackedSourceState(
+            storage=tensor.untyped_storage(),
+            version=tensor._version,
+            storage_offset=tensor.storage_offset(),
+            shape=tensor.shape,
+            stride=tensor.stride(),
+            dtype=tensor.dtype,
+            is_conj=tensor.is_conj(),
+            is_neg=tensor.is_neg(),
+        )
+
+    @staticmethod
+    def _local_packed_source_matches(tensor: torch.Tensor, state: "_LocalPackedSourceState") -> bool:
+        return (
+            tensor._version == state.version
+            and tensor.untyped_storage() is state.storage
+            and tensor.storage_offset() == state.storage_offset
+            and tensor.shape == state.shape
+            and tensor.stride() == state.stride
+            and tensor.dtype == state.dtype
+            and tensor.is_conj() == state.is_conj
+            and tensor.is_neg() == state.is_neg
+        )
+
+    @staticmethod
+    def _local_packed_info_state(info: "ParamInfo") -> "_LocalPackedInfoState":
+        return BlockwiseQuantBucketedBlockShard._LocalPackedInfoState(info=info, unsharded_dtype=info.unsharded_dtype)
+
+    @staticmethod
+    def _local_packed_info_matches(info: "ParamInfo", state: "_LocalPackedInfoState") -> bool:
+        return info is state.info and info.unsharded_dtype == state.unsharded_dtype
+
+    @staticmethod
+    def _local_packed_cache_context(tensors: list[torch.Tensor]) -> tuple[torch.device, Any]:
+        device = next((t.device for t in tensors if t.numel() > 0), tensors[0].device)
+        return device, torch.cuda.current_stream(device)
+
+    def _pack_local_quantized_chunks(
+        self,
+        tensors: list[torch.Tensor],
+        infos: list["ParamInfo"],
+        rank: int,
+        metadata: quant_plan.QuantBucketMetadata,
+    ) -> torch.Tensor:
+        """Quantize this rank's dense shards and pack them, in one launch, into
+        a fresh payload ``[data | pad | scales | pad]`` of the common row size."""
+        if len(tensors) != len(infos):
+            raise ValueError(
+                f"Quantized copy-in requires one tensor per ParamInfo, got {len(tensors)} tensors and {len(infos)} infos."
+            )
+        plan = metadata.rank_pack_plans[rank]
+        device = next((t.device for t in tensors if t.numel() > 0), tensors[0].device)
+        if device.type != "cuda":
+            raise RuntimeError(
+                "Quantized copy-in runs on the GPU through libflexshard_hip.so; got tensors on "
+                f"{device}. This package has no CPU compute path."
+            )
+        payload = torch.empty(metadata.packed_send_nbytes_per_rank, dtype=torch.uint8, device=device)
+        specs: list[hip_ops.QuantChunkSpec] = []
+        staged: list[torch.Tensor] = []
+        qdata_cursor = 0
+        scale_cursor = plan.scale_byte_offset
+        for chunk in plan.chunks:
+            info = infos[chunk.param_index]
+            if info.fqn != chunk.fqn:
+                raise AssertionError(
+                    f"Quantized pack plan parameter order changed: expected {chunk.fqn!r} at index "
+                    f"{chunk.param_index}, got {info.fqn!r}."
+                )
+            shard = tensors[chunk.param_index].reshape(chunk.local_shape)
+            if shard.numel() != chunk.qdata_numel:
+                raise AssertionError(
+                    f"Quantized local dense shard does not match planned chunk for {chunk.fqn!r}: "
+                    f"expected {chunk.qdata_numel} elements, got {shard.numel()}."
+                )
+            if len(chunk.scale_numels) != 1:
+                raise NotImplementedError("the fused quantize+pack kernel handles one scale tensor per chunk")
+            quant_dtype = info.unsharded_dtype
+            kind = self._quantize_pack_source_kind(shard.dtype, quant_dtype)
+            if kind is None or shard.stride(-1) != 1:
+                # Unusual dtype pair or a transposed view: stage a contiguous
+                # copy in the quantization dtype (the reference stages every
+                # non-contiguous or differently typed shard this way).
+                shard = shard.to(quant_dtype).contiguous()
+                staged.append(shard)
+                kind = self._quantize_pack_source_kind(quant_dtype, quant_dtype)
+                if kind is None:
+                    raise NotImplementedError(f"{type(self).__name__} cannot quantize {quant_dtype} shards")
+            specs.append(hip_ops.QuantChunkSpec(shard, qdata_cursor, scale_cursor, kind))
+            qdata_cursor += chunk.qdata_numel
+            scale_cursor += chunk.scale_numels[0] * self._scale_itemsize
+        if qdata_cursor != plan.qdata_numel or scale_cursor != plan.packed_nbytes:
+            raise AssertionError("Quantized pack plan sizes are inconsistent with its chunks.")
+        zero_ranges = ((plan.qdata_numel, plan.scale_byte_offset), (plan.packed_nbytes, payload.numel()))
+        self._launch_quantize_pack(specs, payload, zero_ranges)
+        # Staged copies were allocated and are consumed on the current stream,
+        # so the caching allocator may recycle them as soon as they go out of
+        # scope.
+        del staged
+        return payload
+
+    def _cached_local_quantized_chunks(
+        self, tensors: list[torch.Tensor], infos: list["ParamInfo"], rank: int
+    ) -> tuple[torch.Tensor, quant_plan.QuantBucketMetadata]:
+        """Forward always packs and remembers the payload; a backward re-gather
+        may take it back once if nothing about its sources changed."""
+        metadata = self._quant_metadata_from_infos(infos)
+        if torch.compiler.is_compiling():
+            return self._pack_local_quantized_chunks(tensors, infos, rank, metadata), metadata
+        device, stream = self._local_packed_cache_context(tensors)
+        prefix = (rank, id(metadata))
+        key = (*prefix, device, stream)
+        if not _is_backward_graph_task():
+            packed = self._pack_local_quantized_chunks(tensors, infos, rank, metadata)
+            for stale in [k for k in self._local_packed_cache if k[:2] == prefix]:
+                del self._local_packed_cache[stale]
+            self._local_packed_cache[key] = self._LocalPackedCacheEntry(
+                info_states=tuple(self._local_packed_info_state(i) for i in infos),
+                source_states=tuple(self._local_packed_source_state(t) for t in tensors),
+                metadata=metadata,
+                packed=packed,
+            )
+            return packed, metadata
+        entry = self._local_packed_cache.pop(key, None)
+        if (
+            entry is not None
+            and entry.metadata is metadata
+            and len(entry.info_states) == len(infos)
+            and len(entry.source_states) == len(tensors)
+            and all(self._local_packed_info_matches(i, s) for i, s in zip(infos, entry.info_states, strict=True))
+            and all(self._local_packed_source_matches(t, s) for t, s in zip(tensors, entry.source_states, strict=True))
+        ):
+            return entry.packed, metadata
+        return self._pack_local_quantized_chunks(tensors, infos, rank, metadata), metadata
+
+    # -------------------------------------------------------- unshard lifecycle
+    def prepare_unshard_bucket(
+        self, tensors: list[torch.Tensor], infos: list["ParamInfo"], mesh: Any, debug_fqn: str | None
+    ) -> PlacementPreparedUnshard:
+        """Quantize + pack the local shards and allocate the gather output."""
+        prepared = self._prepare_local_unshard_payload(tensors, infos, mesh, debug_fqn)
+        local = prepared.buffers[0]
+        prepared.buffers.append(torch.empty(mesh.size() * local.numel(), dtype=local.dtype, device=local.device))
+        return prepared
+
+    def _prepare_local_unshard_payload(
+        self, tensors: list[torch.Tensor], infos: list["ParamInfo"], mesh: Any, debug_fqn: str | None
+    ) -> PlacementPreparedUnshard:
+        rank = mesh.get_local_rank()
+        with record_copy_in():
+            local, metadata = self._cached_local_quantized_chunks(tensors, infos, rank)
+        return PlacementPreparedUnshard(
+            placement=self,
+            buffers=[local],
+            placement_state=BlockwiseQuantBucketedBlockShard._QuantUnshardState(
+                infos=infos, pg=mesh.get_group(), debug_fqn=debug_fqn, metadata=metadata
+            ),
+        )
+
+    def _unshard_state(self, prepared: PlacementPreparedUnshard) -> "_QuantUnshardState":
+        state = prepared.placement_state
+        if not isinstance(state, BlockwiseQuantBucketedBlockShard._QuantUnshardState):
+            raise AssertionError(f"Expected {type(self).__name__}._QuantUnshardState, got {type(state).__name__}")
+        return state
+
+    def run_prepared_unshard(self, prepared: PlacementPreparedUnshard, *, async_op: bool = False) -> Any | None:
+        """One uint8 all-gather of the equally sized payload rows."""
+        state = self._unshard_state(prepared)
+        local, gathered = prepared.buffers
+        with record_comm("FlexShard::all_gather", state.debug_fqn):
+            return dist.all_gather_into_tensor(
+                output_tensor=gathered, input_tensor=local, group=state.pg, async_op=async_op
+            )
+
+    def finish_prepared_unshard(self, prepared: PlacementPreparedUnshard) -> PlacementUnshardResult:
+        state = self._unshard_state(prepared)
+        rows = prepared.buffers[1].view(len(state.metadata.rank_qdata_numels), prepared.buffers[0].numel())
+        return self._finish_unshard_from_rank_rows(prepared, rows)
+
+    def _check_rank_rows(self, state: "_QuantUnshardState", rank_rows: torch.Tensor) -> None:
+        expected = (len(state.metadata.rank_qdata_numels), state.metadata.packed_send_nbytes_per_rank)
+        if tuple(rank_rows.shape) != expected:
+            raise ValueError(f"Expected gathered rank rows with shape {expected}, got {tuple(rank_rows.shape)}.")
+        if rank_rows.dtype != torch.uint8:
+            raise ValueError(f"Packed quantized gathered rank rows must use uint8 transport, got {rank_rows.dtype}.")
+
+    def _finish_unshard_from_rank_rows(
+        self, prepared: PlacementPreparedUnshard, rank_rows: torch.Tensor
+    ) -> PlacementUnshardResult:
+        """Unpack from rank-major rows (possibly strided, at odd byte offsets)."""
+        state = self._unshard_state(prepared)
+        self._check_rank_rows(state, rank_rows)
+        return self._finish_quant_unshard_from_rank_rows(prepared, rank_rows, state)
+
+    def _compact_sizes(self, metadata: quant_plan.QuantBucketMetadata) -> tuple[int, int, list[int]]:
+        """(data bytes, aligned scale start, bytes of each scale tensor group)."""
+        data = sum(metadata.rank_qdata_numels)
+        groups = [sum(r.nbytes for r in regions) for regions in metadata.scale_regions_by_index]
+        return data, _align_up(data, _VEC_ALIGN_BYTES), groups
+
+    def _compact_buffer(
+        self, prepared: PlacementPreparedUnshard, metadata: quant_plan.QuantBucketMetadata, device: torch.device
+    ) -> torch.Tensor:
+        if prepared.persistent_buffers is not None:
+            return prepared.persistent_buffers[0]
+        _, scale_start, groups = self._compact_sizes(metadata)
+        return torch.empty(scale_start + sum(groups), dtype=torch.uint8, device=device)
+
+    def _full_params_from_compact(self, state: "_QuantUnshardState", compact: torch.Tensor) -> list[torch.Tensor]:
+        """Per-parameter views of the compact buffer handed to the weight factory."""
+        data_nbytes, scale_start, groups = self._compact_sizes(state.metadata)
+        qdata_flat = compact[:data_nbytes].view(self.qdata_dtype)
+        flat_scales = [g.view(self.scale_dtype) for g in torch.split(compact[scale_start:], groups)]
+        shapes = [_matrix_shape(info.global_shape) for info in state.infos]
+        per_param_counts = [self._chunk_scale_numels(*shape) for shape in shapes]
+        # torch.split raises unless the parameters tile each buffer exactly.
+        qdata_params = torch.split(qdata_flat, [info.global_numel for info in state.infos])
+        scales_by_index = [
+            torch.split(flat, [counts[k] for counts in per_param_counts]) for k, flat in enumerate(flat_scales)
+        ]
+        full = []
+        for p, (info, qdata, shape) in enumerate(zip(state.infos, qdata_params, shapes, strict=True)):
+            scales = tuple(self._param_scale_view(k, per_param[p], shape) for k, per_param in enumerate(scales_by_index))
+            full.append(
+                self._make_quantized_weight_checked(
+                    qdata.view(info.global_shape), scales, orig_dtype=info.unsharded_dtype, requires_grad=info.requires_grad
+                )
+            )
+        return full
+
+    def _finish_quant_unshard_from_rank_rows(
+        self, prepared: PlacementPreparedUnshard, rank_rows: torch.Tensor, state: "_QuantUnshardState"
+    ) -> PlacementUnshardResult:
+        compact = self._compact_buffer(prepared, state.metadata, rank_rows.device)
+        with record_copy_out():
+            # Rank cuts partition one globally ordered stream of block rows, so
+            # joining each rank's valid region restores parameter order.
+            if not self._copy_out_rank_rows_fused(state.metadata, rank_rows, compact):
+                data_nbytes, scale_start, _ = self._compact_sizes(state.metadata)
+                self._copy_out_rank_rows_cat(
+                    state.metadata, rank_rows, compact, qdata_nbytes=data_nbytes, scale_byte_offset=scale_start
+                )
+        return PlacementUnshardResult(
+            full_params=self._full_params_from_compact(state, compact),
+            persistent_buffers=[compact] if prepared.persistent else [],
+        )
+
+    def _copy_out_plan(
+        self, metadata: quant_plan.QuantBucketMetadata, *, data_elem_nbytes: int, with_scales: bool
+    ) -> "_CopyOutPlan":
+        key = (id(metadata), data_elem_nbytes, with_scales)
+        plan = self._copy_out_plans.get(key)
+        if plan is not None and plan.metadata is metadata:
+            return plan
+        regions: list[tuple[int, int, int, int]] = []
+        cursor = 0
+        for rank, numel in enumerate(metadata.rank_qdata_numels):
+            regions.append((rank, 0, numel * data_elem_nbytes, cursor))
+            cursor += numel * data_elem_nbytes
+        if with_scales:
+            cursor = _align_up(cursor, _VEC_ALIGN_BYTES)
+            for group in metadata.scale_regions_by_index:
+                for region in group:
+                    regions.append((region.rank, region.offset, region.nbytes, cursor))
+                    cursor += region.nbytes
+        live = tuple(r for r in regions if r[2] > 0)
+        plan = BlockwiseQuantBucketedBlockShard._CopyOutPlan(
+            metadata=metadata,
+            regions=live,
+            vec_aligned=all(v % _VEC_COPY_NBYTES == 0 for r in live for v in r[1:]),
+            descriptors={},
+        )
+        self._copy_out_plans[key] = plan
+        return plan
+
+    def _copy_out_rank_rows_fused(
+        self,
+        metadata: quant_plan.QuantBucketMetadata,
+        rank_rows: torch.Tensor,
+        out: torch.Tensor,
+        *,
+        data_elem_nbytes: int = 1,
+        with_scales: bool = True,
+    ) -> bool:
+        """Join every rank's payload regions into ``out`` with one HIP launch.
+        ``rank_rows`` and ``out`` are uint8; data regions land in rank order,
+        the scale regions follow from the 16-byte aligned offset.  Returns
+        False only while compiling (the caller then uses ``torch.cat``)."""
+        if torch.compiler.is_compiling():
+            return False
+        _require_gpu_rows(rank_rows, "The rank-row copy-out")
+        plan = self._copy_out_plan(metadata, data_elem_nbytes=data_elem_nbytes, with_scales=with_scales)
+        row_stride = rank_rows.stride(0) if rank_rows.size(0) > 1 else rank_rows.size(1)
+        # The physical rows including any padding between them: plan offsets
+        # count from the first row's first byte.
+        source = rank_rows.as_strided(((rank_rows.size(0) - 1) * row_stride + rank_rows.size(1),), (1,))
+        if plan.vec_aligned and _is_vec_copy_viewable(rank_rows) and _is_vec_copy_viewable(out):
+            source = source.view(_VEC_COPY_DTYPE)
+            out = out.view(_VEC_COPY_DTYPE)
+        unit = source.element_size()
+        key = (rank_rows.device, row_stride, unit)
+        descriptor = plan.descriptors.get(key)
+        if descriptor is None:
+            descriptor = SegmentCopyDescriptor.create(
+                src_offsets=[(rank * row_stride + offset) // unit for rank, offset, _, _ in plan.regions],
+                numels=[nbytes // unit for _, _, nbytes, _ in plan.regions],
+                dst_offsets=[dst // unit for _, _, _, dst in plan.regions],
+                device=rank_rows.device,
+            )
+            plan.descriptors[key] = descriptor
+        copy_segments(source, out, descriptor)
+        return True
+
+    def _copy_out_rank_rows_cat(
+        self,
+        metadata: quant_plan.QuantBucketMetadata,
+        rank_rows: torch.Tensor,
+        compact: torch.Tensor,
+        *,
+        qdata_nbytes: int,
+        scale_byte_offset: int,
+    ) -> None:
+        """``torch.cat`` form of the copy-out, used only under ``torch.compile``
+        (a traced graph cannot call the HIP library)."""
+        data = [rank_rows[rank, :numel] for rank, numel in enumerate(metadata.rank_qdata_numels) if numel]
+        scales = [
+            rank_rows[region.rank, region.offset : region.offset + region.nbytes]
+            for group in metadata.scale_regions_by_index
+            for region in group
+            if region.nbytes
+        ]
+        if data:
+            torch.cat(data, out=compact[:qdata_nbytes])
+        if scales:
+            torch.cat(scales, out=compact[scale_byte_offset:])
+
+    def _make_quantized_weight_checked(
+        self, qdata: torch.Tensor, scales: tuple[torch.Tensor, ...], *, orig_dtype: torch.dtype, requires_grad: bool
+    ) -> torch.Tensor:
+        weight = self._make_quantized_weight(qdata, scales, orig_dtype=orig_dtype, requires_grad=requires_grad)
+        if not isinstance(weight, torch.Tensor):
+            raise TypeError(f"_make_quantized_weight must return a torch.Tensor, got {type(weight).__name__}.")
+        return weight
+
+
+_merge_adjacent_regions = quant_plan.merge_adjacent_regions
+
+__all__ = ["BlockwiseQuantBucketedBlockShard"]

@@ -1,0 +1,212 @@
+"""Muon math on an owner's whole matrices, on HIP kernels.
+
+The functions keep the names and argument meaning of the reference's
+optimizer math (dist_muon/optimizer.py:2031-2151, cost model :1147-1155):
+``_adjust_muon_learning_rate``, ``_prepare_muon_input``,
+``_compute_muon_direction``, ``_apply_muon_update``,
+``_zeropower_via_newtonschulz``.  ``OwnedMuon`` strings them together for the
+comm-free case the reference runs on ``BucketedOwned`` storage
+(dist_muon/_optimizer_reshard_runtime.py:645-661): every parameter is a whole
+matrix on this rank, so a step is prepare -> Newton-Schulz -> apply with no
+exchange.  Matrices of one shape are orthogonalized as one batch.
+"""
+
+from __future__ import annotations
+
+import math
+from collections.abc import Iterable, Sequence
+
+import torch
+
+from .. import hip_ops
+
+DEFAULT_NS_COEFFICIENTS = (3.4445, -4.7750, 2.0315)
+
+
+def _adjust_muon_learning_rate(lr: float, adjust_lr_fn: str | None, compute_matrix_shape: Sequence[int]) -> float:
+    """Scale ``lr`` for the matrix aspect ratio."""
+    rows, columns = compute_matrix_shape[-2:]
+    if adjust_lr_fn is None or adjust_lr_fn == "original":
+        ratio = math.sqrt(max(1.0, rows / columns))
+    elif adjust_lr_fn == "match_rms_adamw":
+        ratio = 0.2 * math.sqrt(max(rows, columns))
+    elif adjust_lr_fn == "spectral_unclamped":
+        ratio = math.sqrt(rows / columns)
+    else:
+        raise ValueError(f"unsupported adjust_lr_fn {adjust_lr_fn!r}")
+    return lr * ratio
+
+
+def _estimate_muon_compute_cost(matrix_shape: Sequence[int], ns_steps: int) -> int:
+    """Multiply-accumulate count of Newton-Schulz: per step two s*s*l products
+    and one s*s*s product (s the short side); FLOPs are twice this."""
+    *batch, rows, columns = matrix_shape
+    short, long = sorted((rows, columns))
+    return math.prod(batch) * ns_steps * short * short * (2 * long + short)
+
+
+def _require_bf16_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t.device.type != "cuda":
+            raise RuntimeError("Muon kernels run on the GPU; this package has no CPU compute path.")
+        if t.dtype != torch.bfloat16:
+            raise NotImplementedError(f"the Muon kernels operate on bf16 tensors, got {t.dtype}")
+        if not t.is_contiguous():
+            raise ValueError("the Muon kernels need contiguous tensors")
+
+
+def _prepare_muon_input(
+    gradient: torch.Tensor, momentum_buffer: torch.Tensor, *, momentum: float, nesterov: bool, out: torch.Tensor
+) -> torch.Tensor:
+    """``momentum_buffer.lerp_(gradient, 1 - momentum)`` and then either
+    ``lerp(gradient, momentum_buffer, momentum)`` (Nesterov) or a copy of the
+    buffer into ``out``; one fused launch."""
+    _require_bf16_gpu(gradient, momentum_buffer, out)
+    hip_ops.muon_prepare(momentum_buffer, gradient, out, momentum=momentum, nesterov=nesterov)
+    return out
+
+
+def _zeropower_via_newtonschulz(
+    update: torch.Tensor,
+    *,
+    ns_coefficients: tuple[float, float, float] = DEFAULT_NS_COEFFICIENTS,
+    ns_steps: int = 5,
+    eps: float = 1e-7,
+    workspace: torch.Tensor | None = None,
+    out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Approximate polar factor of each matrix of ``update`` ([..., rows, cols]):
+    bf16 copy, Frobenius normalization, ``ns_steps`` quintic iterations with
+    fp32-accumulated MFMA products rounded to bf16.  Returns a new bf16 tensor
+    (or ``out``); ``update`` is left untouched unless it *is* ``out``."""
+    if update.device.type != "cuda":
+        raise RuntimeError("Newton-Schulz runs on the GPU; this package has no CPU compute path.")
+    if update.ndim < 2:
+        raise ValueError(f"expected a matrix or a batch of matrices, got shape {tuple(update.shape)}")
+    if out is None:
+        out = update.to(dtype=torch.bfloat16, copy=True).contiguous()
+    elif out is not update:
+        out.copy_(update)
+    _require_bf16_gpu(out)
+    hip_ops.newton_schulz(out.view(-1, *out.shape[-2:]), ns_coefficients, ns_steps, eps, workspace)
+    return out
+
+
+def _compute_muon_direction(
+    prepared: torch.Tensor,
+    *,
+    lr_reference_shape: Sequence[int] | None = None,
+    adjust_lr_fn: str | None = None,
+    ns_coefficients: tuple[float, float, float] = DEFAULT_NS_COEFFICIENTS,
+    ns_steps: int = 5,
+    eps: float = 1e-7,
+    workspace: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Orthogonalize ``prepared`` ([..., rows, cols], bf16) in place.  When the
+    learning-rate shape factor of the matrices differs from the one of
+    ``lr_reference_shape`` the direction is rescaled by their ratio (whole
+    parameters use their own shape as reference, so the factor is 1)."""
+    _zeropower_via_newtonschulz(
+        prepared, ns_coefficients=ns_coefficients, ns_steps=ns_steps, eps=eps, workspace=workspace, out=prepared
+    )
+    if lr_reference_shape is not None:
+        ratio = _adjust_muon_learning_rate(1.0, adjust_lr_fn, prepared.shape[-2:])
+        reference = _adjust_muon_learning_rate(1.0, adjust_lr_fn, lr_reference_shape)
+        if ratio != reference:
+            prepared.mul_(ratio / reference)
+    return prepared
+
+
+def _apply_muon_update(
+    parameter: torch.Tensor,
+    direction: torch.Tensor,
+    *,
+    lr: float,
+    weight_decay: float,
+    adjust_lr_fn: str | None,
+    compute_matrix_shape: Sequence[int],
+) -> torch.Tensor:
+    """``parameter *= 1 - lr*weight_decay; parameter += -adjusted_lr * direction``
+    with a bf16 rounding after each, in one launch."""
+    _require_bf16_gpu(parameter, direction)
+    adjusted = _adjust_muon_learning_rate(lr, adjust_lr_fn, compute_matrix_shape)
+    hip_ops.muon_apply(parameter, direction, decay_factor=1 - lr * weight_decay, neg_adjusted_lr=-adjusted)
+    return parameter
+
+
+class OwnedMuon:
+    """Muon over whole bf16 matrices owned by this rank.
+
+    Defaults follow the reference (dist_muon/optimizer.py:205-222): lr 1e-3,
+    weight decay 0.1, momentum 0.95, Nesterov, 5 Newton-Schulz steps with the
+    quintic coefficients, eps 1e-7.  ``step(grads)`` takes one gradient per
+    parameter, in order; a missing gradient raises before anything is updated.
+    """
+
+    def __init__(
+        self,
+        params: Iterable[torch.Tensor],
+        *,
+        lr: float = 1e-3,
+        weight_decay: float = 0.1,
+        momentum: float = 0.95,
+        nesterov: bool = True,
+        ns_coefficients: tuple[float, float, float] = DEFAULT_NS_COEFFICIENTS,
+        ns_steps: int = 5,
+        eps: float = 1e-7,
+        adjust_lr_fn: str | None = None,
+    ) -> None:
+        self.params = list(params)
+        if not self.params:
+            raise ValueError("OwnedMuon needs at least one parameter")
+        for p in self.params:
+            if p.ndim != 2:
+                raise ValueError(f"Muon updates whole matrices; got a parameter of shape {tuple(p.shape)}")
+        _require_bf16_gpu(*self.params)
+        self.lr, self.weight_decay, self.momentum, self.nesterov = lr, weight_decay, momentum, nesterov
+        self.ns_coefficients, self.ns_steps, self.eps, self.adjust_lr_fn = ns_coefficients, ns_steps, eps, adjust_lr_fn
+        self.momentum_buffers = [torch.zeros_like(p) for p in self.params]
+        # One batch buffer and one Newton-Schulz workspace per matrix shape.
+        self._groups: dict[tuple[int, int], list[int]] = {}
+        for index, p in enumerate(self.params):
+            self._groups.setdefault(tuple(p.shape), []).append(index)
+        self._batch: dict[tuple[int, int], torch.Tensor] = {}
+        self._workspace: dict[tuple[int, int], torch.Tensor] = {}
+        for shape, members in self._groups.items():
+            device = self.params[members[0]].device
+            self._batch[shape] = torch.empty((len(members), *shape), dtype=torch.bfloat16, device=device)
+            need = hip_ops.newton_schulz_workspace_bytes(len(members), *shape)
+            self._workspace[shape] = torch.empty(need, dtype=torch.uint8, device=device)
+
+    def flops_per_step(self) -> int:
+        return 2 * sum(
+            _estimate_muon_compute_cost((len(members), *shape), self.ns_steps) for shape, members in self._groups.items()
+        )
+
+    @torch.no_grad()
+    def step(self, grads: Sequence[torch.Tensor | None]) -> None:
+        if len(grads) != len(self.params):
+            raise ValueError(f"expected {len(self.params)} gradients, got {len(grads)}")
+        missing = [i for i, g in enumerate(grads) if g is None]
+        if missing:
+            raise RuntimeError(f"Muon parameters {missing} have no gradient; no parameter was updated")
+        for p, g in zip(self.params, grads):
+            if g.shape != p.shape:
+                raise ValueError(f"gradient shape {tuple(g.shape)} does not match parameter {tuple(p.shape)}")
+        _require_bf16_gpu(*grads)
+        for shape, members in self._groups.items():
+            batch = self._batch[shape]
+            for slot, index in enumerate(members):
+                _prepare_muon_input(
+                    grads[index], self.momentum_buffers[index], momentum=self.momentum, nesterov=self.nesterov,
+                    out=batch[slot],
+                )
+            _compute_muon_direction(
+                batch, ns_coefficients=self.ns_coefficients, ns_steps=self.ns_steps, eps=self.eps,
+                workspace=self._workspace[shape],
+            )
+            for slot, index in enumerate(members):
+                _apply_muon_update(
+                    self.params[index], batch[slot], lr=self.lr, weight_decay=self.weight_decay,
+                    adjust_lr_fn=self.adjust_lr_fn, compute_matrix_shape=shape,
+                )

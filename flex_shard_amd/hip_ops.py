@@ -1,0 +1,340 @@
+"""Tensor-level wrappers over the C ABI.
+
+Each function checks on the host that operand shapes, dtypes, devices and
+bounds match what the kernel assumes, then queues the kernel on the current
+torch stream of the operands' device.  torch is used for memory and streams
+only.  Nothing here synchronizes the host.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Sequence
+
+import torch
+
+from . import _native
+from ._native import (
+    DT_BF16,
+    DT_F32,
+    EPS_FP32,
+    EPS_INPUT_DTYPE,
+    REDUCE_POSTDIV,
+    REDUCE_POSTMUL,
+    REDUCE_PREMUL,
+    REDUCE_SUM,
+    SRC_BF16,
+    SRC_F32,
+    SRC_F32_AS_BF16,
+)
+
+__all__ = [
+    "DT_BF16", "DT_F32", "EPS_FP32", "EPS_INPUT_DTYPE", "REDUCE_POSTDIV", "REDUCE_POSTMUL",
+    "REDUCE_PREMUL", "REDUCE_SUM", "SRC_BF16", "SRC_F32", "SRC_F32_AS_BF16",
+    "QuantChunkSpec", "accumulate_grad", "copy_segments", "gemm_nt", "muon_apply", "muon_prepare",
+    "newton_schulz", "newton_schulz_workspace_bytes", "pack_segments", "quantize_pack",
+    "reduce_rows", "stream_ptr", "unpack_dequant", "zero_segments",
+]
+
+
+def _require_gpu(*tensors: torch.Tensor) -> torch.device:
+    device = tensors[0].device
+    for t in tensors:
+        if t.device.type != "cuda":
+            raise RuntimeError(
+                "flex_shard_amd kernels run on the GPU only; got a tensor on "
+                f"{t.device}. There is no CPU path."
+            )
+        if t.device != device:
+            raise ValueError(f"tensors on different devices: {device} and {t.device}")
+    return device
+
+
+def stream_ptr(device: torch.device) -> int:
+    """The raw hipStream_t of torch's current stream on ``device``."""
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _dt(dtype: torch.dtype) -> int:
+    if dtype == torch.bfloat16:
+        return DT_BF16
+    if dtype == torch.float32:
+        return DT_F32
+    raise NotImplementedError(f"dtype {dtype} is not supported by the HIP kernels (bf16 and fp32 are)")
+
+
+class QuantChunkSpec:
+    """One chunk of a quantize+pack launch: a 2-D row-major view (unit column
+    stride) and where its FP8 bytes and scales go in the payload."""
+
+    __slots__ = ("tensor", "qdata_offset", "scale_offset", "src_kind")
+
+    def __init__(self, tensor: torch.Tensor, qdata_offset: int, scale_offset: int, src_kind: int) -> None:
+        self.tensor = tensor
+        self.qdata_offset = qdata_offset
+        self.scale_offset = scale_offset
+        self.src_kind = src_kind
+
+
+def quantize_pack(
+    chunks: Sequence[QuantChunkSpec],
+    payload: torch.Tensor,
+    zero_ranges: tuple[tuple[int, int], tuple[int, int]],
+    block: int,
+    eps_mode: int = EPS_INPUT_DTYPE,
+) -> None:
+    """Fused tile quantize + pack of every chunk into ``payload`` (uint8,
+    contiguous) and zeroing of the two pad ranges.  Launches are split when
+    there are more than FSH_MAX_QUANT_CHUNKS chunks."""
+    _require_gpu(payload, *[c.tensor for c in chunks])
+    if payload.dtype != torch.uint8 or not payload.is_contiguous() or payload.ndim != 1:
+        raise ValueError("payload must be a contiguous 1-D uint8 tensor")
+    lib = _native.lib()
+    stream = stream_ptr(payload.device)
+    cap = _native.FSH_MAX_QUANT_CHUNKS
+    groups = [list(chunks[i : i + cap]) for i in range(0, len(chunks), cap)] or [[]]
+    for index, group in enumerate(groups):
+        table = (_native.QuantChunk * max(len(group), 1))()
+        for slot, spec in zip(table, group):
+            t = spec.tensor
+            if t.ndim != 2 or t.stride(1) != 1 or t.shape[0] <= 0 or t.shape[1] <= 0:
+                raise ValueError(f"chunk must be a non-empty 2-D view with unit column stride, got {tuple(t.shape)} / {t.stride()}")
+            expected = torch.bfloat16 if spec.src_kind == SRC_BF16 else torch.float32
+            if t.dtype != expected:
+                raise ValueError(f"chunk dtype {t.dtype} does not match src_kind {spec.src_kind}")
+            slot.src_dev = t.data_ptr()
+            slot.rows, slot.in_dim = t.shape
+            slot.src_row_stride = t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+            slot.qdata_offset = spec.qdata_offset
+            slot.scale_offset = spec.scale_offset
+            slot.src_kind = spec.src_kind
+        zr = zero_ranges if index == 0 else ((0, 0), (0, 0))
+        status = lib.fsh_quantize_pack(
+            table, len(group), payload.data_ptr(), payload.numel(),
+            zr[0][0], zr[0][1], zr[1][0], zr[1][1], block, eps_mode, stream,
+        )
+        _native.check(status, "fsh_quantize_pack")
+
+
+def _check_i64_table(*tables: torch.Tensor) -> int:
+    n = tables[0].numel()
+    for t in tables:
+        if t.dtype != torch.int64 or not t.is_contiguous() or t.numel() != n:
+            raise ValueError("descriptor tables must be contiguous int64 tensors of equal length")
+    return n
+
+
+def copy_segments(
+    source: torch.Tensor, output: torch.Tensor, src_offsets: torch.Tensor, numels: torch.Tensor,
+    dst_offsets: torch.Tensor, max_segment_numel: int,
+) -> None:
+    """``output[dst+i] = source[src+i]`` per segment, in elements of the two
+    tensors' common item size.  Only the data pointers are used, so ``source``
+    may be a strided view whose offsets count from its first element."""
+    _require_gpu(source, output, src_offsets, numels, dst_offsets)
+    if source.element_size() != output.element_size():
+        raise ValueError("source and output must have the same element size")
+    n = _check_i64_table(src_offsets, numels, dst_offsets)
+    status = _native.lib().fsh_copy_segments(
+        source.data_ptr(), output.data_ptr(), src_offsets.data_ptr(), numels.data_ptr(), dst_offsets.data_ptr(),
+        n, max_segment_numel, source.element_size(), stream_ptr(output.device),
+    )
+    _native.check(status, "fsh_copy_segments")
+
+
+def zero_segments(output: torch.Tensor, numels: torch.Tensor, dst_offsets: torch.Tensor, max_segment_numel: int) -> None:
+    _require_gpu(output, numels, dst_offsets)
+    n = _check_i64_table(numels, dst_offsets)
+    status = _native.lib().fsh_zero_segments(
+        output.data_ptr(), numels.data_ptr(), dst_offsets.data_ptr(), n, max_segment_numel,
+        output.element_size(), stream_ptr(output.device),
+    )
+    _native.check(status, "fsh_zero_segments")
+
+
+def pack_segments(
+    input_ptrs: torch.Tensor, tensor_indices: torch.Tensor, src_offsets: torch.Tensor, numels: torch.Tensor,
+    dst_offsets: torch.Tensor, max_segment_numel: int, src_dtype: torch.dtype, output: torch.Tensor,
+) -> None:
+    _require_gpu(output, input_ptrs, tensor_indices, src_offsets, numels, dst_offsets)
+    n = _check_i64_table(tensor_indices, src_offsets, numels, dst_offsets)
+    status = _native.lib().fsh_pack_segments(
+        input_ptrs.data_ptr(), tensor_indices.data_ptr(), src_offsets.data_ptr(), numels.data_ptr(),
+        dst_offsets.data_ptr(), n, max_segment_numel, _dt(src_dtype), _dt(output.dtype), output.data_ptr(),
+        stream_ptr(output.device),
+    )
+    _native.check(status, "fsh_pack_segments")
+
+
+def unpack_dequant(
+    rows: torch.Tensor,
+    chunk_table: torch.Tensor,
+    tile_starts: torch.Tensor,
+    total_tiles: int,
+    compact: torch.Tensor | None,
+    dequant: torch.Tensor | None,
+    block: int,
+) -> None:
+    """``rows``: uint8 tensor whose data pointer is the first gathered row
+    (offsets in the table count from it).  ``chunk_table``: int64 [nchunks, 7]
+    device tensor of ``fsh_unpack_chunk`` records; ``tile_starts``: int64
+    [nchunks + 1].  ``compact`` (uint8) and ``dequant`` (bf16/fp32, flat) are
+    optional outputs; the caller guarantees the table stays inside them."""
+    present = [t for t in (compact, dequant) if t is not None]
+    _require_gpu(rows, chunk_table, tile_starts, *present)
+    if chunk_table.dtype != torch.int64 or chunk_table.ndim != 2 or chunk_table.shape[1] != _native.UNPACK_CHUNK_INT64S:
+        raise ValueError("chunk_table must be int64 [nchunks, 7]")
+    if not chunk_table.is_contiguous() or not tile_starts.is_contiguous() or tile_starts.dtype != torch.int64:
+        raise ValueError("tables must be contiguous int64 tensors")
+    nchunks = chunk_table.shape[0]
+    if tile_starts.numel() != nchunks + 1:
+        raise ValueError("tile_starts must have nchunks + 1 entries")
+    if compact is not None and (compact.dtype != torch.uint8 or not compact.is_contiguous()):
+        raise ValueError("compact must be contiguous uint8")
+    dq_dtype = DT_BF16
+    if dequant is not None:
+        if not dequant.is_contiguous():
+            raise ValueError("dequant must be contiguous")
+        dq_dtype = _dt(dequant.dtype)
+    status = _native.lib().fsh_unpack_dequant(
+        rows.data_ptr(), chunk_table.data_ptr(), tile_starts.data_ptr(), nchunks, total_tiles,
+        compact.data_ptr() if compact is not None else None,
+        dequant.data_ptr() if dequant is not None else None,
+        dq_dtype, block, stream_ptr(rows.device),
+    )
+    _native.check(status, "fsh_unpack_dequant")
+
+
+def accumulate_grad(acc: torch.Tensor, grad: torch.Tensor, *, overwrite: bool = False) -> None:
+    """``acc (+)= grad.float()`` over flat contiguous tensors of equal numel."""
+    _require_gpu(acc, grad)
+    if acc.dtype != torch.float32 or not acc.is_contiguous() or not grad.is_contiguous():
+        raise ValueError("acc must be contiguous fp32 and grad contiguous")
+    if acc.numel() != grad.numel():
+        raise ValueError(f"numel mismatch: acc {acc.numel()} vs grad {grad.numel()}")
+    status = _native.lib().fsh_accumulate_grad(
+        acc.data_ptr(), grad.data_ptr(), _dt(grad.dtype), acc.numel(), int(overwrite), stream_ptr(acc.device)
+    )
+    _native.check(status, "fsh_accumulate_grad")
+
+
+def reduce_rows(
+    out: torch.Tensor, contributions: torch.Tensor, column_offset: int, *, mode: int = REDUCE_SUM, factor: float = 1.0
+) -> None:
+    """``out[i] = fold_r contributions[r, column_offset + i]`` in rank order;
+    ``contributions`` is fp32 [W, row] with unit column stride."""
+    _require_gpu(out, contributions)
+    if out.dtype != torch.float32 or contributions.dtype != torch.float32:
+        raise NotImplementedError("the fixed-order reduction is implemented for fp32 gradients")
+    if contributions.ndim != 2 or contributions.stride(1) != 1 or not out.is_contiguous():
+        raise ValueError("contributions must be [W, row] with unit column stride and out contiguous")
+    world, row = contributions.shape
+    if column_offset < 0 or column_offset + out.numel() > row:
+        raise ValueError(f"range [{column_offset}, {column_offset + out.numel()}) outside rows of {row} elements")
+    stride = contributions.stride(0) if world > 1 else row
+    status = _native.lib().fsh_reduce_rows_f32(
+        out.data_ptr(), contributions.data_ptr(), stride, world, column_offset, out.numel(), mode, factor,
+        stream_ptr(out.device),
+    )
+    _native.check(status, "fsh_reduce_rows_f32")
+
+
+def newton_schulz_workspace_bytes(batch: int, rows: int, cols: int) -> int:
+    return int(_native.lib().fsh_newton_schulz_workspace_bytes(batch, rows, cols))
+
+
+def newton_schulz(
+    x: torch.Tensor,
+    coefficients: tuple[float, float, float],
+    steps: int,
+    eps: float,
+    workspace: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """In-place Newton-Schulz of a contiguous bf16 [batch, rows, cols] (or
+    [rows, cols]) tensor.  ``workspace`` (uint8) is allocated when not given."""
+    _require_gpu(x)
+    if x.dtype != torch.bfloat16 or not x.is_contiguous() or x.ndim not in (2, 3):
+        raise ValueError("x must be a contiguous bf16 matrix or batch of matrices")
+    batch = 1 if x.ndim == 2 else x.shape[0]
+    rows, cols = x.shape[-2:]
+    need = newton_schulz_workspace_bytes(batch, rows, cols)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    _require_gpu(x, workspace)
+    if workspace.dtype != torch.uint8 or not workspace.is_contiguous() or workspace.numel() < need:
+        raise ValueError(f"workspace must be contiguous uint8 with at least {need} bytes")
+    a, b, c = coefficients
+    status = _native.lib().fsh_newton_schulz(
+        x.data_ptr(), batch, rows, cols, a, b, c, steps, eps, workspace.data_ptr(), workspace.numel(),
+        stream_ptr(x.device),
+    )
+    _native.check(status, "fsh_newton_schulz")
+    return x
+
+
+def gemm_nt(
+    a: torch.Tensor, b: torch.Tensor, *, d: torch.Tensor | None = None, alpha: float = 1.0, beta: float = 0.0,
+    out: torch.Tensor | None = None, out_t: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """``bf16(alpha * a @ b^T + beta * d)`` for contiguous bf16 [batch, m, k] /
+    [batch, n, k] (or 2-D) operands; optionally also the transpose."""
+    _require_gpu(a, b)
+    if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16 or not a.is_contiguous() or not b.is_contiguous():
+        raise ValueError("a and b must be contiguous bf16")
+    a3 = a if a.ndim == 3 else a.unsqueeze(0)
+    b3 = b if b.ndim == 3 else b.unsqueeze(0)
+    batch, m, k = a3.shape
+    if b3.shape[0] != batch or b3.shape[2] != k:
+        raise ValueError(f"shape mismatch: a {tuple(a.shape)} vs b {tuple(b.shape)}")
+    n = b3.shape[1]
+    if out is None:
+        out = torch.empty((batch, m, n) if a.ndim == 3 else (m, n), dtype=torch.bfloat16, device=a.device)
+    for name, t, shape in (("d", d, (m, n)), ("out", out, (m, n)), ("out_t", out_t, (n, m))):
+        if t is None:
+            continue
+        _require_gpu(a, t)
+        if t.dtype != torch.bfloat16 or not t.is_contiguous() or tuple(t.shape[-2:]) != shape or t.numel() != batch * m * n:
+            raise ValueError(f"{name} must be contiguous bf16 with trailing shape {shape}")
+    desc = _native.GemmDesc()
+    desc.a_dev, desc.b_dev = a.data_ptr(), b.data_ptr()
+    desc.d_dev = d.data_ptr() if d is not None else None
+    desc.c_dev = out.data_ptr()
+    desc.ct_dev = out_t.data_ptr() if out_t is not None else None
+    desc.m, desc.n, desc.k = m, n, k
+    desc.lda, desc.ldb, desc.ldd, desc.ldc, desc.ldct = k, k, n, n, m
+    desc.batch = batch
+    desc.stride_a, desc.stride_b = m * k, n * k
+    desc.stride_d = desc.stride_c = desc.stride_ct = m * n
+    desc.alpha, desc.beta = alpha, beta
+    status = _native.lib().fsh_gemm_bf16_nt(ctypes.byref(desc), stream_ptr(a.device))
+    _native.check(status, "fsh_gemm_bf16_nt")
+    return out
+
+
+def muon_prepare(
+    momentum_buffer: torch.Tensor, grad: torch.Tensor, out: torch.Tensor, *, momentum: float, nesterov: bool
+) -> None:
+    _require_gpu(momentum_buffer, grad, out)
+    for t in (momentum_buffer, grad, out):
+        if t.dtype != torch.bfloat16 or not t.is_contiguous() or t.numel() != grad.numel():
+            raise ValueError("muon_prepare needs contiguous bf16 tensors of equal numel")
+    status = _native.lib().fsh_muon_prepare(
+        momentum_buffer.data_ptr(), grad.data_ptr(), out.data_ptr(), grad.numel(), 1 - momentum, momentum,
+        int(nesterov), stream_ptr(grad.device),
+    )
+    _native.check(status, "fsh_muon_prepare")
+
+
+def muon_apply(
+    param: torch.Tensor, direction: torch.Tensor, *, decay_factor: float, neg_adjusted_lr: float,
+    direction_scale: float = 1.0,
+) -> None:
+    _require_gpu(param, direction)
+    for t in (param, direction):
+        if t.dtype != torch.bfloat16 or not t.is_contiguous() or t.numel() != param.numel():
+            raise ValueError("muon_apply needs contiguous bf16 tensors of equal numel")
+    status = _native.lib().fsh_muon_apply(
+        param.data_ptr(), direction.data_ptr(), param.numel(), decay_factor, neg_adjusted_lr, direction_scale,
+        stream_ptr(param.device),
+    )
+    _native.check(status, "fsh_muon_apply")

@@ -1,0 +1,226 @@
+/*
+ * C ABI of libflexshard_hip.so: hand-written gfx950 (MI355X) kernels for the
+ * single-GPU hot path of FlexShard's bucketed placements.
+ *
+ * The reference has no FFI: its hot path is Python calling Triton kernels, one
+ * third-party Triton quantizer and ATen ops.  Each entry point below replaces
+ * the device work of the reference lines it cites (paths under the reference
+ * checkout, src/flex_shard/...).  The Python placements in flex_shard_amd/
+ * are the only callers.
+ *
+ * Conventions
+ *  - every function returns 0 on success and a negative FSH_E* code otherwise;
+ *    fsh_last_error() returns a thread-local message for the last failure;
+ *  - nothing here allocates or frees device memory, synchronizes the host, or
+ *    touches the null stream: `stream` is a hipStream_t passed as void*, and
+ *    all work is queued on it;
+ *  - pointers named *_dev are device pointers; plain struct tables are host
+ *    memory read during the call;
+ *  - sizes and offsets are int64_t; offsets are in bytes unless the name says
+ *    otherwise.
+ */
+#ifndef FLEXSHARD_HIP_H_
+#define FLEXSHARD_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FSH_OK 0
+#define FSH_EINVAL (-22)  /* bad argument, message in fsh_last_error() */
+#define FSH_ENOTSUP (-95) /* valid request this build cannot serve */
+#define FSH_EHIP (-5)     /* a HIP runtime call failed */
+
+/* Library version, (major << 16) | minor. */
+int32_t fsh_version(void);
+/* Message of the calling thread's last failed call ("" if none). */
+const char* fsh_last_error(void);
+
+/* ------------------------------------------------------------------------
+ * 1. Fused tile quantize + pack.
+ * Replaces custom_placements/blockwise_quant_bucketed_block_shard.py:792-897
+ * (_pack_local_quantized_chunks: pad zeroing, dtype staging, one quantizer
+ * launch per chunk, two foreach copies) and the quantizer it calls,
+ * custom_placements/fp8_bucketed_block_shard.py:66-88.  Arithmetic per
+ * block x block tile follows tests/test_flex_shard_fp8_allgather.py:45-90:
+ *   amax in the quantization dtype, floor 1e-12, scale = fp32(448 / fp64(amax)),
+ *   q = e4m3fn(fp32(x) * scale), stored scale = 1.0f / scale.
+ * One launch covers every chunk of a rank and zeroes the payload's two pad
+ * gaps.
+ * ---------------------------------------------------------------------- */
+
+/* Source element kinds. */
+#define FSH_SRC_BF16 0        /* bf16 shard, quantized as is                  */
+#define FSH_SRC_F32 1         /* fp32 shard, quantized as fp32                */
+#define FSH_SRC_F32_AS_BF16 2 /* fp32 master shard, rounded to bf16 first     */
+
+/* Floor applied to a tile's amax. */
+#define FSH_EPS_INPUT_DTYPE 0 /* 1e-12 rounded to the quantization dtype      */
+#define FSH_EPS_FP32 1        /* 1e-12 rounded to fp32 whatever the dtype     */
+
+typedef struct fsh_quant_chunk {
+  const void* src_dev;    /* first element of the chunk's [rows, in_dim] matrix */
+  int64_t rows;           /* > 0 */
+  int64_t in_dim;         /* > 0 */
+  int64_t src_row_stride; /* elements between consecutive rows, >= in_dim      */
+  int64_t qdata_offset;   /* byte offset of the chunk's FP8 bytes in payload   */
+  int64_t scale_offset;   /* byte offset of its fp32 scale block, 4-aligned    */
+  int32_t src_kind;       /* FSH_SRC_*                                        */
+  int32_t reserved;
+} fsh_quant_chunk;
+
+#define FSH_MAX_QUANT_CHUNKS 24
+
+/*
+ * payload_dev[qdata_offset + r*in_dim + c] = FP8 byte of element (r, c);
+ * scales of tile (tr, tc) at scale_offset + 4*(tr*ceil(in_dim/block) + tc).
+ * Bytes [zero0_begin, zero0_end) and [zero1_begin, zero1_end) of the payload
+ * are set to zero (the pad between data and scales, and the tail pad).
+ * nchunks <= FSH_MAX_QUANT_CHUNKS; block = 128 takes the vectorized path when
+ * a chunk's pointers, stride and offsets are 16-byte friendly, any other
+ * block size or alignment takes a scalar path with the same results.
+ */
+int fsh_quantize_pack(const fsh_quant_chunk* chunks, int32_t nchunks, void* payload_dev,
+                      int64_t payload_nbytes, int64_t zero0_begin, int64_t zero0_end,
+                      int64_t zero1_begin, int64_t zero1_end, int32_t block, int32_t eps_mode,
+                      void* stream);
+
+/* ------------------------------------------------------------------------
+ * 2. Segment copy / zero / cast-pack.
+ * Replaces the Triton kernels of custom_placements/_copy_kernels.py:
+ * _copy_segments_kernel (:123-142, launcher :436-461), _zero_segments_kernel
+ * (:145-161, :464-484) and the four _pack_segments_* kernels (:17-120,
+ * :249-359).  The three int64 device arrays are the same arrays the Triton
+ * kernels take, in units of `unit_nbytes` (1, 2, 4, 8 or 16).
+ * ---------------------------------------------------------------------- */
+int fsh_copy_segments(const void* src_dev, void* dst_dev, const int64_t* src_offsets_dev,
+                      const int64_t* numels_dev, const int64_t* dst_offsets_dev,
+                      int64_t nsegments, int64_t max_segment_numel, int32_t unit_nbytes,
+                      void* stream);
+
+int fsh_zero_segments(void* dst_dev, const int64_t* numels_dev, const int64_t* dst_offsets_dev,
+                      int64_t nsegments, int64_t max_segment_numel, int32_t unit_nbytes,
+                      void* stream);
+
+#define FSH_DT_BF16 0
+#define FSH_DT_F32 1
+/* out[dst_off[s]+i] = cast(inputs[tensor_idx[s]][src_off[s]+i]), i < numel[s];
+ * offsets in elements; input_ptrs_dev holds the inputs' device addresses.  A
+ * negative tensor index makes the segment a zero fill, so one launch can
+ * build a whole zero-padded send buffer. */
+int fsh_pack_segments(const int64_t* input_ptrs_dev, const int64_t* tensor_indices_dev,
+                      const int64_t* src_offsets_dev, const int64_t* numels_dev,
+                      const int64_t* dst_offsets_dev, int64_t nsegments,
+                      int64_t max_segment_numel, int32_t src_dtype, int32_t dst_dtype,
+                      void* dst_dev, void* stream);
+
+/* ------------------------------------------------------------------------
+ * 3. Unpack of gathered rank rows: compaction fused with bf16 dequantization.
+ * Replaces custom_placements/blockwise_quant_bucketed_block_shard.py:1237-1422
+ * (_finish_quant_unshard_from_rank_rows / _copy_out_rank_rows_triton) and
+ * blockwise_fp8/blockwise_fp8_weight.py:25-54,121-127 (blockwise_dequant_weight)
+ * in one pass over the FP8 bytes.
+ * ---------------------------------------------------------------------- */
+typedef struct fsh_unpack_chunk {
+  int64_t src_qdata_offset;   /* bytes from rows_dev to the chunk's FP8 rows    */
+  int64_t src_scale_offset;   /* bytes from rows_dev to its fp32 scale block    */
+  int64_t rows;
+  int64_t in_dim;
+  int64_t dst_qdata_offset;   /* bytes into compact_dev                         */
+  int64_t dst_scale_offset;   /* bytes into compact_dev                         */
+  int64_t dst_dequant_offset; /* elements into dequant_dev                      */
+} fsh_unpack_chunk;
+
+/*
+ * chunks_dev: device table of nchunks entries; total_tiles = sum over chunks
+ * of ceil(rows/block)*ceil(in_dim/block); tile_starts_dev[i] = first tile
+ * index of chunk i (nchunks+1 entries, exclusive prefix sum).
+ * compact_dev may be NULL (no compaction), dequant_dev may be NULL (no
+ * dequantization).  dequant dtype is FSH_DT_BF16 or FSH_DT_F32.
+ */
+int fsh_unpack_dequant(const void* rows_dev, const fsh_unpack_chunk* chunks_dev,
+                       const int64_t* tile_starts_dev, int32_t nchunks, int64_t total_tiles,
+                       void* compact_dev, void* dequant_dev, int32_t dequant_dtype,
+                       int32_t block, void* stream);
+
+/* ------------------------------------------------------------------------
+ * 4. fp32 gradient accumulation of one microbatch.
+ * Replaces the AccumulateGrad cast-and-add the runtime relies on
+ * (flex_shard/bucket_runtime.py:931-933, policy flex_shard/bucket_storage.py
+ * :59-77): acc[i] = acc[i] + float(grad[i]); with overwrite != 0,
+ * acc[i] = float(grad[i]) (first microbatch).
+ * ---------------------------------------------------------------------- */
+int fsh_accumulate_grad(float* acc_dev, const void* grad_dev, int32_t grad_dtype, int64_t numel,
+                        int32_t overwrite, void* stream);
+
+/* ------------------------------------------------------------------------
+ * 5. Fixed-order W-way reduction of one rank's range (single-GPU stand-in
+ * for the reduce-scatter).  Replaces custom_placements/utils.py:157-172
+ * (reduce_scatter_grads) with the op/divide choices of :116-144, and feeds
+ * the copy-out views of custom_placements/block_shard.py:1373-1380.
+ *   out[i] = fold over r = 0..world-1, in that order, of
+ *            src[r*contribution_stride + column_offset + i]
+ * ---------------------------------------------------------------------- */
+#define FSH_REDUCE_SUM 0     /* plain sum                                      */
+#define FSH_REDUCE_PREMUL 1  /* each term multiplied by `factor` before adding */
+#define FSH_REDUCE_POSTMUL 2 /* sum multiplied by `factor`                     */
+#define FSH_REDUCE_POSTDIV 3 /* sum divided by `factor`                        */
+int fsh_reduce_rows_f32(float* out_dev, const float* src_dev, int64_t contribution_stride,
+                        int32_t world, int64_t column_offset, int64_t numel, int32_t mode,
+                        float factor, void* stream);
+
+/* ------------------------------------------------------------------------
+ * 6. Newton-Schulz orthogonalization on MFMA.
+ * Replaces dist_muon/optimizer.py:2120-2151 (_zeropower_via_newtonschulz):
+ * bf16 operands, fp32 accumulation, every product rounded to bf16.
+ * x_dev: batch matrices [rows, cols] bf16, row-major, batch stride rows*cols,
+ * overwritten with the result.  Tall matrices (rows > cols) are iterated in
+ * place through X <- a X + X (b A + c A A), A = X^T X, which is the transpose
+ * of the reference's iteration on X^T.
+ * workspace_dev: at least fsh_newton_schulz_workspace_bytes(...) bytes.
+ * ---------------------------------------------------------------------- */
+int64_t fsh_newton_schulz_workspace_bytes(int64_t batch, int64_t rows, int64_t cols);
+int fsh_newton_schulz(void* x_dev, int64_t batch, int64_t rows, int64_t cols, float a, float b,
+                      float c, int32_t steps, float eps, void* workspace_dev,
+                      int64_t workspace_nbytes, void* stream);
+
+/* Batched bf16 "NT" GEMM, the building block of (6), exported for tests:
+ *   C[b] = bf16(alpha * A[b] . B[b]^T + beta * D[b])      fp32 accumulation
+ * A is [m, k] with row stride lda, B is [n, k] with row stride ldb (both
+ * k-contiguous), D and C are [m, n] with row strides ldd / ldc.  D may be NULL
+ * (beta ignored) or alias C.  ct_dev, when not NULL, also receives C[b]^T as
+ * an [n, m] matrix with row stride ldct.  Batch strides are in elements.
+ * k and all leading dimensions must be multiples of 8 and all pointers
+ * 16-byte aligned; m and n are arbitrary. */
+typedef struct fsh_gemm_desc {
+  const void* a_dev;
+  const void* b_dev;
+  const void* d_dev;
+  void* c_dev;
+  void* ct_dev;
+  int64_t m, n, k;
+  int64_t lda, ldb, ldd, ldc, ldct;
+  int64_t batch;
+  int64_t stride_a, stride_b, stride_d, stride_c, stride_ct;
+  float alpha, beta;
+} fsh_gemm_desc;
+int fsh_gemm_bf16_nt(const fsh_gemm_desc* desc, void* stream);
+
+/* ------------------------------------------------------------------------
+ * 7. Muon elementwise steps in bf16 (fp32 math, one rounding per reference
+ * tensor op).  Replace dist_muon/optimizer.py:2049-2068 (_prepare_muon_input:
+ * momentum.lerp_(grad, 1-mu); out = lerp(grad, momentum, mu) when nesterov)
+ * and :2100-2117 (_apply_muon_update: p *= 1 - lr*wd; p += -adjusted_lr*dir).
+ * ---------------------------------------------------------------------- */
+int fsh_muon_prepare(void* momentum_dev, const void* grad_dev, void* out_dev, int64_t numel,
+                     float lerp_weight /* 1 - mu */, float nesterov_weight /* mu */,
+                     int32_t nesterov, void* stream);
+int fsh_muon_apply(void* param_dev, const void* direction_dev, int64_t numel, float decay_factor,
+                   float neg_adjusted_lr, float direction_scale, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLEXSHARD_HIP_H_ */

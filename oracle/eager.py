@@ -1,0 +1,152 @@
+"""The hot path in eager torch CPU ops.  TEST INFRASTRUCTURE ONLY.
+
+Each function spells the reference algorithm with the same torch operators
+and dtypes the reference uses, so its results are what the reference's CPU
+path produces; it doubles as the timed CPU baseline of ``bench.py``.
+Citations are paths under the reference checkout (``src/flex_shard/...``).
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+FP8_MAX = 448.0
+EPS = 1e-12
+
+
+def _tile_view(matrix: torch.Tensor, block: int) -> tuple[torch.Tensor, int, int]:
+    """Zero-pad to whole tiles and view as [tile_row, block, tile_col, block]."""
+    rows, cols = matrix.shape
+    tiles_r, tiles_c = -(-rows // block), -(-cols // block)
+    if (rows, cols) == (tiles_r * block, tiles_c * block):
+        padded = matrix.contiguous()
+    else:
+        padded = matrix.new_zeros((tiles_r * block, tiles_c * block))
+        padded[:rows, :cols] = matrix
+    return padded.view(tiles_r, block, tiles_c, block), tiles_r, tiles_c
+
+
+def quantize_blockwise(
+    weight: torch.Tensor, block: int, fp8_dtype: torch.dtype = torch.float8_e4m3fn
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """tests/test_flex_shard_fp8_allgather.py:45-90 -- per-tile amax in the
+    input dtype, floor 1e-12 in the input dtype, float64 division, float32
+    scale, multiply, clamp, cast; returns (fp8 [rows, cols], recip fp32)."""
+    if weight.ndim != 2 or 0 in weight.shape:
+        raise ValueError(f"expects a non-empty 2D matrix, got {tuple(weight.shape)}")
+    rows, cols = weight.shape
+    tiles, tiles_r, tiles_c = _tile_view(weight, block)
+    fp8_max = torch.finfo(fp8_dtype).max
+    amax = tiles.abs().amax(dim=(1, 3), keepdim=True).clamp(min=EPS).to(torch.float64)
+    scale = (fp8_max / amax).to(torch.float32)
+    quant = (tiles.to(torch.float32) * scale).clamp(-fp8_max, fp8_max).to(fp8_dtype)
+    recip = (1.0 / scale).reshape(tiles_r, tiles_c).to(torch.float32)
+    quant = quant.reshape(tiles_r * block, tiles_c * block)[:rows, :cols]
+    return quant.contiguous(), recip.contiguous()
+
+
+def dequant_blockwise(
+    quant: torch.Tensor, recip_scale: torch.Tensor, block: int, out_dtype: torch.dtype = torch.bfloat16
+) -> torch.Tensor:
+    """blockwise_fp8/blockwise_fp8_weight.py:25-54,121-127 -- fp32 product of
+    the FP8 value and its tile's reciprocal scale, one cast to ``out_dtype``."""
+    rows, cols = quant.shape
+    tiles, tiles_r, tiles_c = _tile_view(quant, block)
+    deq = tiles.to(torch.float32) * recip_scale.reshape(tiles_r, 1, tiles_c, 1).to(torch.float32)
+    return deq.reshape(tiles_r * block, tiles_c * block)[:rows, :cols].to(out_dtype)
+
+
+def accumulate_microbatches(grads: list[torch.Tensor]) -> torch.Tensor:
+    """flex_shard/bucket_runtime.py:931-933 -- each microbatch's bf16 grad is
+    cast to the fp32 accumulation dtype and added in arrival order."""
+    acc = torch.zeros(grads[0].shape, dtype=torch.float32)
+    for grad in grads:
+        acc += grad.to(torch.float32)
+    return acc
+
+
+def reduce_rank_contributions(
+    contributions: list[torch.Tensor], offset: int, numel: int, *, divide: float | None = None,
+    premultiply: float | None = None,
+) -> torch.Tensor:
+    """custom_placements/utils.py:157-172 on one GPU: a left fold over ranks
+    0..W-1 of ``[offset, offset+numel)``; ``premultiply`` mirrors the
+    premul-sum op (:134), ``divide`` the post-division (:172)."""
+    total = None
+    for contribution in contributions:
+        piece = contribution[offset : offset + numel]
+        if premultiply is not None:
+            piece = piece * premultiply
+        total = piece.clone() if total is None else total + piece
+    if divide is not None:
+        total = total / divide
+    return total
+
+
+def newton_schulz(
+    update: torch.Tensor,
+    coefficients: tuple[float, float, float] = (3.4445, -4.7750, 2.0315),
+    steps: int = 5,
+    eps: float = 1e-7,
+) -> torch.Tensor:
+    """dist_muon/optimizer.py:2120-2151 -- bf16 copy, transpose tall inputs,
+    divide by the clamped Frobenius norm, then ``steps`` quintic iterations
+    with every product in bf16; 3-D+ inputs take the batched branch."""
+    a, b, c = coefficients
+    x = update.to(dtype=torch.bfloat16, copy=True)
+    tall = x.shape[-2] > x.shape[-1]
+    if tall:
+        x = x.transpose(-2, -1)
+    x.div_(x.norm(dim=(-2, -1), keepdim=True).clamp_min(eps))
+    if x.ndim == 2:
+        for _ in range(steps):
+            gram = x @ x.T
+            poly = torch.addmm(gram, gram, gram, beta=b, alpha=c)
+            x = torch.addmm(x, poly, x, beta=a)
+    else:
+        shape = x.shape
+        batch = x.reshape(-1, *shape[-2:])
+        for _ in range(steps):
+            gram = batch @ batch.transpose(-2, -1)
+            poly = torch.baddbmm(gram, gram, gram, beta=b, alpha=c)
+            batch = torch.baddbmm(batch, poly, batch, beta=a)
+        x = batch.reshape(shape)
+    return x.transpose(-2, -1) if tall else x
+
+
+def adjusted_lr(lr: float, adjust_lr_fn: str | None, shape) -> float:
+    """dist_muon/optimizer.py:2031-2046."""
+    rows, cols = shape[-2:]
+    if adjust_lr_fn is None or adjust_lr_fn == "original":
+        return lr * math.sqrt(max(1.0, rows / cols))
+    if adjust_lr_fn == "match_rms_adamw":
+        return lr * 0.2 * math.sqrt(max(rows, cols))
+    if adjust_lr_fn == "spectral_unclamped":
+        return lr * math.sqrt(rows / cols)
+    raise ValueError(f"unsupported adjust_lr_fn {adjust_lr_fn!r}")
+
+
+def muon_step(
+    param: torch.Tensor,
+    grad: torch.Tensor,
+    momentum_buffer: torch.Tensor,
+    *,
+    lr: float = 1e-3,
+    weight_decay: float = 0.1,
+    momentum: float = 0.95,
+    nesterov: bool = True,
+    coefficients: tuple[float, float, float] = (3.4445, -4.7750, 2.0315),
+    steps: int = 5,
+    eps: float = 1e-7,
+    adjust_lr_fn: str | None = None,
+) -> None:
+    """dist_muon/optimizer.py:2049-2117 for one whole matrix, in place:
+    momentum lerp, Nesterov lerp, Newton-Schulz, decoupled weight decay and
+    the scaled update, all in the parameter dtype."""
+    momentum_buffer.lerp_(grad, 1 - momentum)
+    update = torch.lerp(grad, momentum_buffer, momentum) if nesterov else momentum_buffer.clone()
+    direction = newton_schulz(update, coefficients, steps, eps).to(param.dtype)
+    param.mul_(1 - lr * weight_decay)
+    param.add_(direction, alpha=-adjusted_lr(lr, adjust_lr_fn, param.shape))
