@@ -533,9 +533,15 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
     ) -> tuple[torch.Tensor, quant_plan.QuantBucketMetadata]:
         """Forward always packs and remembers the payload; a backward re-gather
         may take it back once if nothing about its sources changed."""
+        if len(tensors) != len(infos):
+            raise ValueError(
+                f"Quantized copy-in requires one tensor per ParamInfo, got {len(tensors)} tensors and {len(infos)} infos."
+            )
         metadata = self._quant_metadata_from_infos(infos)
         if torch.compiler.is_compiling():
             return self._pack_local_quantized_chunks(tensors, infos, rank, metadata), metadata
+        for tensor in tensors:
+            _require_gpu_rows(tensor, "Quantized copy-in")
         device, stream = self._local_packed_cache_context(tensors)
         prefix = (rank, id(metadata))
         key = (*prefix, device, stream)

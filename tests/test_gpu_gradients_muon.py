@@ -1,0 +1,451 @@
+"""GPU parity of the gradient path (copy-in, fp32 accumulation, fixed-order
+reduce + copy-out) and of the Muon / Newton-Schulz kernels."""
+
+import pytest
+import torch
+import torch.nn as nn
+
+from flex_shard_amd import (
+    BucketedBlockShard,
+    Fp8BucketedBlockShard,
+    GradientReduction,
+    LocalReduceGroup,
+    hip_ops,
+)
+from flex_shard_amd.custom_placements.utils import gradient_reduce_plan, reduce_grads_on_one_rank
+from flex_shard_amd.dist_muon import (
+    OwnedMuon,
+    _apply_muon_update,
+    _estimate_muon_compute_cost,
+    _prepare_muon_input,
+    _zeropower_via_newtonschulz,
+)
+from flex_shard_amd.testing import LLAMA3_8B_LAYER, FakeMesh, make_param_infos, seeded_normal
+from oracle import cport, eager
+from oracle import layout as olayout
+
+pytestmark = pytest.mark.gpu
+import torch.distributed as dist  # noqa: E402
+
+COEFFS = (3.4445, -4.7750, 2.0315)
+
+
+def _factory(fp8_data, recip_scale, block_size, *, orig_dtype, requires_grad):
+    return fp8_data
+
+
+def _bucket(shapes, world, dtype, device_type="meta"):
+    pl = Fp8BucketedBlockShard(world_size=world, weight_factory=_factory, block_size=4)
+    named = [(f"w{i}", nn.Parameter(torch.empty(tuple(s), device=device_type, dtype=dtype))) for i, s in enumerate(shapes)]
+    return pl, make_param_infos(named, pl, FakeMesh(world))
+
+
+def _expected_rows(pl, grads, infos, dtype):
+    layout = infos[0].bucket_layout
+    return olayout.reduce_scatter_input(
+        [g.cpu() for g in grads],
+        [layout.param_layouts[i.fqn].param_offset for i in infos],
+        layout.global_numel, layout.rank_offsets, layout.rank_numels, dtype,
+    )
+
+
+def _grads(infos, dtype, device):
+    torch.manual_seed(0)
+    return [torch.randn(i.global_shape, dtype=dtype, device=device) for i in infos]
+
+
+# ------------------------------------------------------------------ copy-in
+def test_one_pass_copy_in_matches_reference_rows(device, golden):
+    cases = golden["reduce_copy_in_cases"]["fp8_layout_cases"]
+    for name, case in cases.items():
+        for dtype in (torch.bfloat16, torch.float32):
+            pl, infos = _bucket(case["shapes"], case["world_size"], dtype)
+            grads = _grads(infos, dtype, device)
+            prepared = pl.prepare_reduce_grad(grads, infos, FakeMesh(case["world_size"]), None)
+            want = _expected_rows(pl, grads, infos, dtype)
+            assert torch.equal(prepared.buffers[0].view(want.shape).cpu(), want), f"{name} {dtype}"
+            assert len(pl._reduce_copy_in_plans) == 1
+
+
+def test_copy_in_with_gaps_and_empty_rank(device, golden):
+    dense = golden["reduce_copy_in_cases"]["dense_case"]
+    pl = BucketedBlockShard(dims=(0,), blocks_per_rank=tuple(dense["blocks_per_rank"]))
+    named = [(f"w{i}", nn.Parameter(torch.empty(tuple(s), device="meta", dtype=torch.bfloat16))) for i, s in enumerate(dense["shapes"])]
+    infos = make_param_infos(named, pl, FakeMesh(4))
+    grads = _grads(infos, torch.bfloat16, device)
+    prepared = pl.prepare_reduce_grad(grads, infos, FakeMesh(4), None)
+    want = _expected_rows(pl, grads, infos, torch.bfloat16)
+    assert torch.equal(prepared.buffers[0].view(want.shape).cpu(), want)
+    (plan,) = pl._reduce_copy_in_plans.values()
+    assert len(plan.zero_segments) > 4
+
+
+def test_copy_in_into_wider_rows(device, golden):
+    pl, infos = _bucket([(16, 8), (8, 8), (12, 4)], 8, torch.bfloat16)
+    grads = _grads(infos, torch.bfloat16, device)
+    want = _expected_rows(pl, grads, infos, torch.bfloat16).to(device)
+    width = want.size(1)
+    for start, extra in golden["reduce_copy_in_cases"]["wider_rows"]:
+        rows = torch.full((8, start + width + extra), 7.0, dtype=torch.bfloat16, device=device)
+        send = rows[:, start : start + width]
+        pl._pack_reduce_scatter_grad(grads, infos, 8, send)
+        assert torch.equal(send, want)
+        assert (rows[:, :start] == 7.0).all() and (rows[:, start + width :] == 7.0).all()
+    assert len(pl._reduce_copy_in_plans) == 3  # one plan per row stride
+
+
+def test_copy_in_casts_to_the_reduce_dtype_in_the_same_launch(device):
+    """bf16 grads with an fp32 reduce dtype: the cast is fused into the copy
+    (the reference routes this through a zeroed bucket and a foreach copy)."""
+    pl, infos = _bucket([(16, 8), (8, 8), (12, 4)], 8, torch.bfloat16)
+    for info in infos:
+        info.reduce_dtype = torch.float32
+    grads = _grads(infos, torch.bfloat16, device)
+    assert pl._packs_reduce_scatter_grad_in_one_pass(grads, torch.float32)
+    prepared = pl.prepare_reduce_grad(grads, infos, FakeMesh(8), None)
+    want = _expected_rows(pl, grads, infos, torch.float32)
+    assert prepared.buffers[0].dtype == torch.float32
+    assert torch.equal(prepared.buffers[0].view(want.shape).cpu(), want)
+    # fp32 grads into a bf16 reduce dtype round to nearest even like torch
+    pl2, infos2 = _bucket([(16, 8), (5, 3)], 4, torch.bfloat16)
+    grads32 = _grads(infos2, torch.float32, device)
+    prepared = pl2.prepare_reduce_grad(grads32, infos2, FakeMesh(4), None)
+    want = _expected_rows(pl2, grads32, infos2, torch.bfloat16)
+    assert torch.equal(prepared.buffers[0].view(want.shape).cpu(), want)
+
+
+def test_copy_in_through_a_bucket_while_compiling(device):
+    from unittest.mock import patch
+
+    pl, infos = _bucket([(16, 8), (8, 8), (12, 4)], 8, torch.bfloat16)
+    grads = _grads(infos, torch.bfloat16, device)
+    with patch.object(torch.compiler, "is_compiling", return_value=True):
+        assert not pl._packs_reduce_scatter_grad_in_one_pass(grads, torch.bfloat16)
+        prepared = pl.prepare_reduce_grad(grads, infos, FakeMesh(8), None)
+    want = _expected_rows(pl, grads, infos, torch.bfloat16)
+    assert torch.equal(prepared.buffers[0].view(want.shape).cpu(), want)
+    assert pl._reduce_copy_in_plans == {}
+
+
+def test_zero_copy_when_grads_view_one_bucket(device):
+    pl = BucketedBlockShard(dims=(0,), blocks_per_rank=(1, 1))
+    named = [("a", nn.Parameter(torch.empty(4, 4, device="meta"))), ("b", nn.Parameter(torch.empty(4, 4, device="meta")))]
+    infos = make_param_infos(named, pl, FakeMesh(2))
+    bucket = torch.randn(infos[0].bucket_layout.global_numel, device=device)
+    grads = [bucket[0:16].view(4, 4), bucket[16:32].view(4, 4)]
+    prepared = pl.prepare_reduce_grad(grads, infos, FakeMesh(2), None)
+    assert prepared.buffers[0] is bucket
+
+
+# -------------------------------------------------- accumulate, reduce, copy-out
+def test_fp32_accumulation_known_answer(device, golden):
+    g = golden["fp32_accumulation"]
+    acc = torch.empty(1000, device=device)
+    hip_ops.accumulate_grad(acc, torch.full((1000,), g["first"], device=device).bfloat16(), overwrite=True)
+    hip_ops.accumulate_grad(acc, torch.full((1000,), g["second"], device=device).bfloat16())
+    assert (acc == g["fp32_sum"]).all()
+
+
+@pytest.mark.parametrize("n,offset", [(1 << 20, 0), (1000003, 0), (4099, 1), (7, 3)])
+def test_accumulate_is_exact_for_any_length_and_alignment(device, n, offset):
+    gen = torch.Generator().manual_seed(n)
+    grads = [(torch.randn(n + offset, generator=gen) * 1e-3).bfloat16() for _ in range(4)]
+    base = torch.zeros(n + offset + 8, device=device)
+    acc = base[offset : offset + n]
+    for k, g in enumerate(grads):
+        hip_ops.accumulate_grad(acc, g.to(device)[offset:], overwrite=(k == 0))
+    want = eager.accumulate_microbatches([g[offset:] for g in grads])
+    assert torch.equal(acc.cpu(), want)
+    check = torch.zeros(n)
+    for g in grads:
+        cport.accumulate_bf16(check, g[offset:].contiguous())
+    assert torch.equal(want, check)
+    assert (base[:offset] == 0).all() and (base[offset + n :] == 0).all()
+    # fp32 microbatch gradients accumulate too
+    g32 = torch.randn(n, generator=gen).to(device)
+    before = acc.clone()
+    hip_ops.accumulate_grad(acc, g32)
+    assert torch.equal(acc, before + g32)
+
+
+def test_fixed_order_reduce_and_modes(device):
+    gen = torch.Generator().manual_seed(5)
+    world, seg = 8, 12345
+    contrib = torch.randn(world, world * seg, generator=gen).to(device)
+    out = torch.empty(seg, device=device)
+    for rank in (0, 3, 7):
+        rows = [contrib[r, rank * seg : (rank + 1) * seg].cpu().contiguous() for r in range(world)]
+        hip_ops.reduce_rows(out, contrib, rank * seg)
+        assert torch.equal(out.cpu(), cport.reduce_rows(rows))
+        hip_ops.reduce_rows(out, contrib, rank * seg, mode=hip_ops.REDUCE_PREMUL, factor=1 / 3)
+        assert torch.equal(out.cpu(), cport.reduce_rows(rows, cport.REDUCE_PREMUL, 1 / 3))
+        hip_ops.reduce_rows(out, contrib, rank * seg, mode=hip_ops.REDUCE_POSTDIV, factor=3.0)
+        assert torch.equal(out.cpu(), cport.reduce_rows(rows, cport.REDUCE_POSTDIV, 3.0))
+        hip_ops.reduce_rows(out, contrib, rank * seg, mode=hip_ops.REDUCE_POSTMUL, factor=0.125)
+        assert torch.equal(out.cpu(), cport.reduce_rows(rows, cport.REDUCE_POSTMUL, 0.125))
+    # unaligned column offset and odd length take the scalar path
+    odd = torch.empty(1001, device=device)
+    hip_ops.reduce_rows(odd, contrib, 17)
+    assert torch.equal(odd.cpu(), cport.reduce_rows([contrib[r, 17:1018].cpu().contiguous() for r in range(world)]))
+    with pytest.raises(ValueError, match="outside rows"):
+        hip_ops.reduce_rows(out, contrib, world * seg - 10)
+
+
+def test_reduce_plan_table():
+    avg, sm = GradientReduction(), GradientReduction(op=dist.ReduceOp.SUM)
+    assert gradient_reduce_plan(sm, 8, torch.float32) == ("sum", None, None)
+    assert gradient_reduce_plan(avg, 8, torch.float32) == ("avg", None, None)
+    assert gradient_reduce_plan(avg, 1, torch.float32) == ("sum", None, None)
+    assert gradient_reduce_plan(GradientReduction(divide_factor=4.0), 1, torch.float32) == ("sum", None, 4.0)
+    assert gradient_reduce_plan(GradientReduction(divide_factor=16.0), 8, torch.bfloat16) == ("premul_sum", 16.0, None)
+    assert gradient_reduce_plan(GradientReduction(divide_factor=16.0), 8, torch.float16) == ("sum", 4, 4.0)
+    with pytest.raises(ValueError, match="requires gradient_reduce_op=AVG"):
+        GradientReduction(op=dist.ReduceOp.SUM, divide_factor=2.0)
+    with pytest.raises(ValueError, match="positive"):
+        GradientReduction(divide_factor=0.0)
+
+
+def test_reduce_prepared_grad_end_to_end_small(device):
+    """8 simulated ranks' copy-in rows, the fixed-order reduction on rank r and
+    the copy-out views, for SUM / AVG / a custom divide factor."""
+    world = 8
+    shapes = [(16, 8), (8, 8), (12, 4)]
+    for rank in (0, 5):
+        for reduction, post in ((GradientReduction(op=dist.ReduceOp.SUM), 1.0), (GradientReduction(), 8.0),
+                                (GradientReduction(divide_factor=16.0), 16.0)):
+            group = LocalReduceGroup(world, rank)
+            pl = Fp8BucketedBlockShard(world_size=world, weight_factory=_factory, block_size=4)
+            named = [(f"w{i}", nn.Parameter(torch.empty(s, device="meta"))) for i, s in enumerate(shapes)]
+            infos = make_param_infos(named, pl, FakeMesh(world, rank, group))
+            per_rank_grads, prepared_mine = [], None
+            for r in range(world):
+                torch.manual_seed(100 + r)
+                grads = [torch.randn(s, device=device) for s in shapes]
+                per_rank_grads.append(grads)
+                prepared = pl.prepare_reduce_grad(grads, infos, FakeMesh(world, rank, group), None)
+                group.deposit(r, prepared.buffers[0])
+                if r == rank:
+                    prepared_mine = prepared
+            result = pl.reduce_prepared_grad(prepared_mine, reduction)
+            layout = infos[0].bucket_layout
+            for i, (info, shard) in enumerate(zip(infos, result.sharded_grads)):
+                total = None
+                for r in range(world):
+                    term = per_rank_grads[r][i].cpu() * (1.0 / post) if post != 1.0 else per_rank_grads[r][i].cpu()
+                    total = term.clone() if total is None else total + term
+                lo = layout.param_layouts[info.fqn].local_global_offset - layout.param_layouts[info.fqn].param_offset
+                want = total.reshape(-1)[lo : lo + info.local_numel].view(info.local_shape)
+                assert torch.equal(shard.cpu(), want), (rank, i)
+                if shard.numel():
+                    assert shard.untyped_storage().data_ptr() == result.buffers[0].untyped_storage().data_ptr()
+    one = torch.full((4,), 8.0, device=device)
+    reduce_grads_on_one_rank(one, GradientReduction(divide_factor=4.0))
+    assert (one == 2.0).all()
+    with pytest.raises(ValueError, match="missing the contributions"):
+        group = LocalReduceGroup(2, 0)
+        group.allocate(8, torch.float32, device)
+        from flex_shard_amd.custom_placements.utils import reduce_scatter_grads
+
+        reduce_scatter_grads(torch.empty(4, device=device), torch.zeros(8, device=device), GradientReduction(), group)
+
+
+def test_llama_gradient_bucket_full_size(device, golden):
+    """Config 4 at full size, in the real placement layout (218 365 952
+    elements including zero gaps, rank range 27 295 744): 4 bf16 microbatches
+    accumulate into fp32, then 8 rank contributions are summed in rank order
+    into rank 0's range.  Checked against the same left fold in torch fp32 on
+    the GPU (bit-exact, and within rtol 1e-6 by construction) and against the C
+    oracle on a slice."""
+    g = golden["llama3_8b_dense_bucket"]
+    world = 8
+    pl = BucketedBlockShard(dims=(0,), blocks_per_rank=(1,) * world)
+    named = [(n, nn.Parameter(torch.empty(s, device="meta", dtype=torch.bfloat16))) for n, s in LLAMA3_8B_LAYER]
+    group = LocalReduceGroup(world, 0)
+    infos = make_param_infos(named, pl, FakeMesh(world, 0, group))
+    for info in infos:
+        info.reduce_dtype = torch.float32
+    layout = infos[0].bucket_layout
+    total, seg = layout.global_numel, layout.rank_numels[0]
+    assert total == g["global_numel"] and seg == g["rank_numel"]
+
+    # fp32 accumulation of 4 microbatches into a gradient bucket in this layout
+    acc = torch.zeros(total, device=device)
+    micro = [seeded_normal((total,), 1e-3, 500 + k, device) for k in range(4)]
+    for k, m in enumerate(micro):
+        hip_ops.accumulate_grad(acc, m, overwrite=(k == 0))
+    ref = micro[0].float()
+    for m in micro[1:]:
+        ref = ref + m.float()
+    assert torch.equal(acc, ref)
+    sl = slice(12345678, 12345678 + 100000)
+    check = torch.zeros(100000)
+    for m in micro:
+        cport.accumulate_bf16(check, m[sl].cpu().contiguous())
+    assert torch.equal(acc[sl].cpu(), check)
+    del micro, ref
+
+    # grads as views of the accumulated bucket: the copy-in is free
+    grads = [acc[layout.param_layouts[i.fqn].param_offset :][: i.global_numel].view(i.global_shape) for i in infos]
+    prepared = pl.prepare_reduce_grad(grads, infos, FakeMesh(world, 0, group), None)
+    assert prepared.buffers[0] is acc
+
+    # 8 rank contributions (this rank's accumulated bucket plus 7 seeded ones)
+    contributions = group.allocate(total, torch.float32, device)
+    contributions[0].copy_(acc)
+    for r in range(1, world):
+        contributions[r].copy_(seeded_normal((total,), 1e-3, 900 + r, device, torch.float32))
+    group.mark_deposited(*range(world))
+    result = pl.reduce_prepared_grad(prepared, GradientReduction(op=dist.ReduceOp.SUM))
+    recv = result.buffers[0]
+    want = contributions[0, :seg].clone()
+    for r in range(1, world):
+        want = want + contributions[r, :seg]
+    assert torch.equal(recv, want)
+    torch.testing.assert_close(recv, contributions[:, :seg].double().sum(0).float(), rtol=1e-6, atol=1e-8)
+    rows = [contributions[r, 777 : 777 + 50000].cpu().contiguous() for r in range(world)]
+    assert torch.equal(recv[777 : 777 + 50000].cpu(), cport.reduce_rows(rows))
+    # copy-out: q, k, v and the first 504 rows of o land on rank 0 as views of recv
+    numels = [i.local_numel for i in infos]
+    assert numels[0] == 4096 * 4096 and numels[1] == numels[2] == 1024 * 4096 and sum(numels) < seg
+    for info, shard in zip(infos, result.sharded_grads):
+        assert shard.shape == info.local_shape
+        if shard.numel():
+            start = info.byte_offset // 2
+            assert shard.data_ptr() == recv.data_ptr() + 4 * start
+
+
+# ------------------------------------------------------------ Newton-Schulz
+@pytest.mark.parametrize("shape", [(128, 256), (256, 128), (256, 256), (64, 96), (200, 136), (3, 512, 256), (2, 128, 384)])
+def test_newton_schulz_matches_torch_muon_routine(device, shape, golden):
+    from torch.optim._muon import _zeropower_via_newtonschulz as torch_ns
+
+    tol = golden["muon_tolerance"]["atol"]
+    gen = torch.Generator().manual_seed(3)
+    g = torch.randn(shape, generator=gen).bfloat16()
+    mine = _zeropower_via_newtonschulz(g.to(device)).cpu()
+    mats = g.view(-1, *shape[-2:])
+    ref = torch.stack([torch_ns(m, COEFFS, 5, 1e-7) for m in mats]).view(shape)
+    assert mine.shape == g.shape and mine.dtype == torch.bfloat16
+    assert (mine.float() - ref.float()).abs().max().item() <= tol
+    small = cport.newton_schulz(mats[0]) if mats[0].numel() <= 128 * 256 else None
+    if small is not None:
+        assert (mine.view(-1, *shape[-2:])[0].float() - small.float()).abs().max().item() <= tol
+
+
+def test_newton_schulz_leaves_its_input_untouched_and_handles_zero(device):
+    g = torch.randn(128, 128, device=device).bfloat16()
+    keep = g.clone()
+    _zeropower_via_newtonschulz(g)
+    assert torch.equal(g, keep)
+    z = _zeropower_via_newtonschulz(torch.zeros(64, 128, device=device, dtype=torch.bfloat16))
+    assert (z == 0).all()
+    with pytest.raises(RuntimeError, match="multiples of 8"):
+        _zeropower_via_newtonschulz(torch.randn(12, 20, device=device).bfloat16())
+
+
+def test_gemm_building_block(device):
+    gen = torch.Generator().manual_seed(4)
+    a = torch.randn(2, 200, 64, generator=gen).bfloat16().to(device)
+    b = torch.randn(2, 136, 64, generator=gen).bfloat16().to(device)
+    d = torch.randn(2, 200, 136, generator=gen).bfloat16().to(device)
+    ct = torch.empty(2, 136, 200, device=device, dtype=torch.bfloat16)
+    c = hip_ops.gemm_nt(a, b, d=d, alpha=0.5, beta=2.0, out_t=ct)
+    ref = 0.5 * (a.double() @ b.double().transpose(1, 2)) + 2.0 * d.double()
+    assert torch.allclose(c.double(), ref, rtol=2.0**-8, atol=1e-2)  # one bf16 rounding of the fp32 result
+    assert torch.equal(ct, c.transpose(1, 2).contiguous())
+    big = hip_ops.gemm_nt(a[0].repeat(3, 8)[:512], a[0].repeat(3, 8)[:384])
+    want = (a[0].repeat(3, 8)[:512].double() @ a[0].repeat(3, 8)[:384].double().t())
+    assert torch.allclose(big.double(), want, rtol=2.0**-7, atol=0.5)
+
+
+def test_newton_schulz_full_size_invariants(device):
+    """Config 5 shapes: [7168, 2048] (tall, iterated as its transpose) and
+    [2048, 2048].  Singular values of the result lie in the quintic's band and
+    the result correlates with the exact polar factor."""
+    for shape in ((7168, 2048), (2048, 2048)):
+        g = seeded_normal(shape, 1.0, 11, device)
+        x = _zeropower_via_newtonschulz(g).float()
+        sv = torch.linalg.svdvals(x)
+        assert sv.max().item() < 1.3
+        if shape[0] != shape[1]:
+            # a square Gaussian matrix has singular values near zero that five
+            # steps cannot lift; a 3.5:1 one does not
+            assert sv.min().item() > 0.3
+        u, _, vh = torch.linalg.svd(g.float(), full_matrices=False)
+        polar = u @ vh
+        cos = (x * polar).sum() / (x.norm() * polar.norm())
+        assert cos.item() > (0.97 if shape[0] != shape[1] else 0.9)
+    # one full-size matrix against torch's routine on the GPU (its hipBLAS path)
+    from torch.optim._muon import _zeropower_via_newtonschulz as torch_ns
+
+    g = seeded_normal((2048, 2048), 1.0, 12, device)
+    assert (_zeropower_via_newtonschulz(g).float() - torch_ns(g, COEFFS, 5, 1e-7).float()).abs().max().item() <= 2e-2
+
+
+# --------------------------------------------------------------- Muon steps
+def test_muon_elementwise_kernels(device):
+    """Momentum / Nesterov interpolation and the decayed update against the
+    same torch tensor ops the reference issues, run by torch on the GPU (the
+    reference's own execution target) and on the CPU.  bf16 results may differ
+    by one ulp where torch fuses a multiply-add; they must agree almost
+    everywhere.  (torch's CPU kernel rounds the decay factor 0.9999 to bf16,
+    i.e. to 1.0, so only the GPU comparison is tight for the update.)"""
+    gen = torch.Generator().manual_seed(6)
+    n = 100003
+    grad = torch.randn(n, generator=gen).bfloat16()
+    mom = (torch.randn(n, generator=gen) * 0.1).bfloat16()
+    for nesterov in (True, False):
+        m_gpu, out = mom.to(device), torch.empty(n, dtype=torch.bfloat16, device=device)
+        _prepare_muon_input(grad.to(device), m_gpu, momentum=0.95, nesterov=nesterov, out=out)
+        for where in (device, torch.device("cpu")):
+            m_ref, g_ref = mom.to(where).clone(), grad.to(where)
+            m_ref.lerp_(g_ref, 1 - 0.95)
+            o_ref = torch.lerp(g_ref, m_ref, 0.95) if nesterov else m_ref.clone()
+            assert torch.allclose(m_gpu.cpu().float(), m_ref.cpu().float(), rtol=2.0**-7, atol=1e-6)
+            assert torch.allclose(out.cpu().float(), o_ref.cpu().float(), rtol=2.0**-7, atol=1e-5)
+            assert (m_gpu.cpu() != m_ref.cpu()).float().mean() < 0.01
+            assert (out.cpu() != o_ref.cpu()).float().mean() < 0.02
+    p = (torch.randn(n, generator=gen) * 0.02).bfloat16()
+    d = torch.randn(n, generator=gen).bfloat16()
+    p_gpu = p.to(device)
+    _apply_muon_update(p_gpu.view(1, n), d.to(device).view(1, n), lr=1e-3, weight_decay=0.1, adjust_lr_fn=None,
+                       compute_matrix_shape=(7168, 2048))
+    alpha = -eager.adjusted_lr(1e-3, None, (7168, 2048))
+    p_ref = p.to(device).clone()
+    p_ref.mul_(1 - 1e-3 * 0.1)
+    p_ref.add_(d.to(device), alpha=alpha)
+    assert torch.allclose(p_gpu.float(), p_ref.float(), rtol=2.0**-7, atol=2e-5)
+    assert (p_gpu != p_ref).float().mean() < 0.01
+    p_cpu = p.clone()
+    p_cpu.mul_(1 - 1e-3 * 0.1)
+    p_cpu.add_(d, alpha=alpha)
+    assert torch.allclose(p_gpu.cpu().float(), p_cpu.float(), rtol=2.0**-7, atol=2e-5)
+
+
+def test_owned_muon_step_matches_torch_optim_muon(device, golden):
+    """Three steps on whole matrices of two shapes against torch.optim.Muon's
+    single-tensor path (same defaults), the reference's own oracle and bar."""
+    tol = golden["muon_tolerance"]["atol"]
+    gen = torch.Generator().manual_seed(7)
+    shapes = [(256, 128), (128, 128), (256, 128), (128, 128)]
+    start = [(torch.randn(s, generator=gen) * 0.02).bfloat16() for s in shapes]
+    mine = [p.clone().to(device) for p in start]
+    theirs = [nn.Parameter(p.clone()) for p in start]
+    opt_mine = OwnedMuon(mine)
+    opt_theirs = torch.optim.Muon(theirs, lr=1e-3, weight_decay=0.1, momentum=0.95, nesterov=True)
+    for _ in range(3):
+        grads = [torch.randn(s, generator=gen).bfloat16() for s in shapes]
+        opt_mine.step([g.to(device) for g in grads])
+        for p, g in zip(theirs, grads):
+            p.grad = g.clone()
+        opt_theirs.step()
+    for a, b in zip(mine, theirs):
+        assert (a.cpu().float() - b.detach().float()).abs().max().item() <= tol
+        assert torch.allclose(a.cpu().float(), b.detach().float(), atol=1e-3)  # a few bf16 ulps of the weights
+    assert opt_mine.flops_per_step() == 2 * (
+        _estimate_muon_compute_cost((2, 256, 128), 5) + _estimate_muon_compute_cost((2, 128, 128), 5)
+    )
+    with pytest.raises(RuntimeError, match="no gradient"):
+        before = [p.clone() for p in mine]
+        opt_mine.step([None] + [torch.zeros_like(p) for p in mine[1:]])
+    assert all(torch.equal(a, b) for a, b in zip(mine, before))

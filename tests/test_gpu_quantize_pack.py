@@ -1,0 +1,336 @@
+"""GPU parity of the fused tile quantize + pack path (through the C ABI) with
+the CPU oracle: bit-exact FP8 bytes and scale bits."""
+
+import pytest
+import torch
+import torch.nn as nn
+
+from flex_shard_amd import Fp8BucketedBlockShard, hip_ops
+from flex_shard_amd.custom_placements.fp8_bucketed_block_shard import _quantize_dense_weight_to_blockwise_fp8
+from flex_shard_amd.testing import (
+    DEEPSEEK_V3_EXPERTS,
+    LLAMA3_8B_LAYER,
+    FakeMesh,
+    add_outliers_and_zero_tiles,
+    local_rows,
+    make_param_infos,
+    prepare_unshard_on_each_rank,
+    seeded_bucket,
+    seeded_normal,
+)
+from oracle import cport, eager
+from oracle import layout as olayout
+
+pytestmark = pytest.mark.gpu
+E4M3 = torch.float8_e4m3fn
+
+
+def _factory(fp8_data, recip_scale, block_size, *, orig_dtype, requires_grad):
+    return fp8_data
+
+
+def _bits(t):
+    return t.contiguous().view(torch.int32)
+
+
+def _quant_gpu(w, block, eps_mode=hip_ops.EPS_INPUT_DTYPE):
+    q, s = _quantize_dense_weight_to_blockwise_fp8(w, block, E4M3, eps_mode=eps_mode)
+    return q.view(torch.uint8).cpu(), s.cpu()
+
+
+def _assert_matches_oracle(w_cpu, block, device, **kw):
+    q, s = _quant_gpu(w_cpu.to(device), block)
+    oq, osc = cport.quantize_blockwise(w_cpu, block, **kw)
+    assert torch.equal(q, oq), f"FP8 bytes differ in {(q != oq).sum().item()} places"
+    assert torch.equal(_bits(s), _bits(osc)), "scale bits differ"
+
+
+def test_config1_plumbing_case(device):
+    """bf16 [2048, 2048], N(0, 0.02), 128x128 tiles, world size 1: payload is
+    4 194 304 FP8 bytes + [16, 16] scales = 4 195 328 bytes."""
+    gen = torch.Generator().manual_seed(0)
+    w = (torch.randn(2048, 2048, generator=gen) * 0.02).bfloat16()
+    pl = Fp8BucketedBlockShard(world_size=1, weight_factory=_factory)
+    param = nn.Parameter(w.to(device), requires_grad=False)
+    infos = make_param_infos([("w", param)], pl, FakeMesh(1))
+    prepared = pl.prepare_unshard_bucket([param.detach()], infos, FakeMesh(1), None)
+    payload = prepared.buffers[0].cpu()
+    assert payload.numel() == 4195328 and prepared.buffers[1].numel() == 4195328
+    oq, osc = cport.quantize_blockwise(w, 128)
+    eq, esc = eager.quantize_blockwise(w, 128)
+    assert torch.equal(payload[:4194304], oq.reshape(-1)) and torch.equal(oq, eq.view(torch.uint8))
+    assert torch.equal(payload[4194304:].view(torch.float32), osc.reshape(-1))
+    assert torch.equal(_bits(osc), _bits(esc)) and osc.shape == (16, 16)
+
+
+@pytest.mark.parametrize(
+    "shape,block",
+    [((6, 4), 4), ((12, 6), 4), ((6, 6), 4), ((9, 32), 2), ((256, 384), 128), ((200, 136), 128), ((130, 129), 128),
+     ((1, 3), 4), ((128, 8), 128), ((257, 4096), 128), ((64, 64), 16), ((300, 200), 64)],
+)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_matches_oracle_on_shapes(device, shape, block, dtype):
+    gen = torch.Generator().manual_seed(hash((shape, block)) % 1000)
+    w = (torch.randn(shape, generator=gen) * 0.02).to(dtype)
+    _assert_matches_oracle(w, block, device)
+
+
+def test_scale_arithmetic_for_every_bf16_amax(device):
+    """One 4x4 tile per non-negative bf16 value (including values below the
+    1e-12 floor, the largest finite value and infinity) holding that value as
+    its amax: scale bits and bytes must match the oracle for all 32 641."""
+    amax = torch.arange(0, 0x7F81, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    n = amax.numel()
+    gen = torch.Generator().manual_seed(1)
+    frac = torch.rand(n, 4, 4, generator=gen) * 2 - 1
+    tiles = (frac * amax.float().clamp(max=3e38).view(n, 1, 1)).bfloat16()
+    tiles[:, 1, 2] = amax
+    w = tiles.view(n * 4, 4)
+    q, s = _quant_gpu(w.to(device), 4)
+    oq, osc = cport.quantize_blockwise(w, 4)
+    assert torch.equal(_bits(s), _bits(osc))
+    finite = ~osc.isinf().view(-1)
+    rows = finite.repeat_interleave(4)
+    assert torch.equal(q[rows], oq[rows])
+    # amax = inf: finite entries become 0, the inf itself NaN (sign aside)
+    assert torch.equal(q[~rows] & 0x7F, oq[~rows] & 0x7F)
+
+
+def test_element_rounding_for_every_bf16_value(device):
+    """Tiles whose amax is a power of two (exact scale): every bf16 value with
+    |x| <= amax goes through the hardware FP8 conversion and must equal both
+    the oracle and torch's own cast of x * scale."""
+    all_bf16 = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+    for k in (0, -7, 6):
+        amax = 2.0**k
+        values = all_bf16[all_bf16.abs() <= amax]
+        values = values[: values.numel() // 16 * 16].view(-1, 4).clone()
+        values[0::4, 0] = amax
+        w = values.bfloat16()
+        q, _ = _quant_gpu(w.to(device), 4)
+        oq, _ = cport.quantize_blockwise(w, 4)
+        assert torch.equal(q, oq)
+        assert torch.equal(q, (w.float() * (448.0 / amax)).to(E4M3).view(torch.uint8))
+
+
+def test_zero_tile_eps_modes(device, golden):
+    g = golden["quant_eps_constants"]
+    z = torch.zeros(128, 256, dtype=torch.bfloat16, device=device)
+    z[:, 128:] = 0.5
+    q, s = _quant_gpu(z, 128)
+    assert (q[:, :128] == 0).all() and s.view(torch.int32)[0, 0].item() == int(g["zero_tile_recip_bits_bf16_input"], 16)
+    _, s = _quant_gpu(z, 128, hip_ops.EPS_FP32)
+    assert s.view(torch.int32)[0, 0].item() == int(g["zero_tile_recip_bits_fp32_input"], 16)
+    _, s = _quant_gpu(z.float(), 128)
+    assert s.view(torch.int32)[0, 0].item() == int(g["zero_tile_recip_bits_fp32_input"], 16)
+    # sub-floor but non-zero amax is clamped too, and tiny values quantize to signed zero
+    tiny = torch.full((4, 4), -1e-20, dtype=torch.bfloat16, device=device)
+    q, s = _quant_gpu(tiny, 4)
+    oq, osc = cport.quantize_blockwise(tiny.cpu(), 4)
+    assert torch.equal(q, oq) and torch.equal(_bits(s), _bits(osc)) and (q == 0x80).all()
+
+
+def test_nan_tile_is_poisoned_like_the_oracle(device):
+    w = torch.ones(8, 4).bfloat16()
+    w[0, 0] = float("nan")
+    q, s = _quant_gpu(w.to(device), 4)
+    oq, osc = cport.quantize_blockwise(w, 4)
+    assert ((q[:4] & 0x7F) == 0x7F).all() and s[0, 0].isnan()
+    assert torch.equal(q[4:], oq[4:]) and torch.equal(_bits(s[1:]), _bits(osc[1:]))
+
+
+def test_fp32_master_is_quantized_as_bf16(device, golden):
+    """Reference known answer: an fp32 shard with param_dtype bf16 quantizes
+    its bf16 rounding (and differs from quantizing the fp32 values)."""
+    g = golden["fp8_quantizes_param_dtype"]
+    block = g["block"]
+    full = torch.full((block, block), g["fill"], dtype=torch.float32, device=device)
+    full[0, 0] = g["outlier"]
+    pl = Fp8BucketedBlockShard(world_size=1, weight_factory=_factory, block_size=block)
+    param = nn.Parameter(full.clone())
+    (info,) = make_param_infos([("w", param)], pl, FakeMesh(1))
+    info.param_dtype = torch.bfloat16
+    prepared = pl.prepare_unshard_bucket([full], [info], FakeMesh(1), None)
+    md = prepared.placement_state.metadata
+    payload = prepared.buffers[0].cpu()
+    fp8 = payload[: md.rank_qdata_numels[0]].view(block, block)
+    scale = payload[md.rank_scale_byte_offsets[0] : md.rank_packed_nbytes[0]].view(torch.float32)
+    ref_q, ref_s = eager.quantize_blockwise(full.cpu().bfloat16(), block)
+    _, fp32_s = eager.quantize_blockwise(full.cpu(), block)
+    assert torch.equal(fp8, ref_q.view(torch.uint8)) and fp8[0, 0].item() == g["outlier_byte"]
+    assert torch.equal(_bits(scale), _bits(ref_s.view(-1))) and scale.item() == torch.tensor(1 / 448.0).item()
+    assert not torch.equal(_bits(scale), _bits(fp32_s.view(-1)))
+    # larger, vector-path version of the same dtype pair
+    gen = torch.Generator().manual_seed(3)
+    big = torch.randn(256, 256, generator=gen) * 0.02
+    pl = Fp8BucketedBlockShard(world_size=1, weight_factory=_factory)
+    param = nn.Parameter(big.to(device))
+    (info,) = make_param_infos([("w", param)], pl, FakeMesh(1))
+    info.param_dtype = torch.bfloat16
+    payload = pl.prepare_unshard_bucket([param.detach()], [info], FakeMesh(1), None).buffers[0].cpu()
+    oq, osc = cport.quantize_blockwise(big, 128, cast_to_bf16=True)
+    assert torch.equal(payload[: 256 * 256], oq.reshape(-1))
+    assert torch.equal(payload[256 * 256 :].view(torch.int32), _bits(osc).view(-1))
+
+
+def test_strided_and_offset_sources(device):
+    """Shards that are row-strided views (unit column stride) or start at an
+    odd element are read in place; results equal the contiguous copy."""
+    gen = torch.Generator().manual_seed(4)
+    parent = (torch.randn(300, 400, generator=gen) * 0.02).bfloat16().to(device)
+    for view in (parent[:, 8:264], parent[3:259, 1:130], parent[::2, :128]):
+        q, s = _quantize_dense_weight_to_blockwise_fp8(view, 128, E4M3)
+        oq, osc = cport.quantize_blockwise(view.cpu().contiguous(), 128)
+        assert torch.equal(q.view(torch.uint8).cpu(), oq) and torch.equal(_bits(s.cpu()), _bits(osc))
+
+
+def test_pack_format_and_pad_zeroing(device):
+    """The payload of every rank equals the oracle's naive pack of whole-matrix
+    quantization, pads included, even when the buffer held garbage."""
+    shapes, block, world = [(16, 8), (8, 8), (12, 4), (1, 3)], 4, 8
+    gen = torch.Generator().manual_seed(5)
+    params = [torch.randn(s, generator=gen).bfloat16() for s in shapes]
+    named = [(f"w{i}", nn.Parameter(p.to(device), requires_grad=False)) for i, p in enumerate(params)]
+    pl = Fp8BucketedBlockShard(world_size=world, weight_factory=_factory, block_size=block)
+    # poison the allocator's free blocks so stale bytes would show up in pads
+    junk = torch.full((1 << 20,), 0xAB, dtype=torch.uint8, device=device)
+    del junk
+    prepared = prepare_unshard_on_each_rank(pl, named, world)
+    lay = olayout.quant_layout(shapes, block, world)
+    qs, ss = zip(*[cport.quantize_blockwise(p, block) for p in params])
+    for rank in range(world):
+        want = olayout.pack_rank_payload(lay, rank, list(qs), list(ss), block)
+        assert torch.equal(prepared[rank].buffers[0].cpu(), want), f"rank {rank}"
+        assert prepared[rank].buffers[1].numel() == world * lay.row_nbytes
+
+
+def test_many_chunks_split_into_several_launches(device):
+    """More chunks than one launch table holds (30 parameters on one rank)."""
+    gen = torch.Generator().manual_seed(6)
+    params = [(torch.randn(8, 16, generator=gen)).bfloat16() for _ in range(30)]
+    named = [(f"w{i}", nn.Parameter(p.to(device), requires_grad=False)) for i, p in enumerate(params)]
+    pl = Fp8BucketedBlockShard(world_size=1, weight_factory=_factory, block_size=8)
+    (prepared,) = prepare_unshard_on_each_rank(pl, named, 1)
+    lay = olayout.quant_layout([(8, 16)] * 30, 8, 1)
+    qs, ss = zip(*[cport.quantize_blockwise(p, 8) for p in params])
+    assert torch.equal(prepared.buffers[0].cpu(), olayout.pack_rank_payload(lay, 0, list(qs), list(ss), 8))
+
+
+def test_payload_cache_forward_backward(device):
+    """Forward always repacks; a backward graph task may take the cached
+    payload back once; compiling bypasses the cache."""
+    from unittest.mock import patch
+
+    from flex_shard_amd.custom_placements import blockwise_quant_bucketed_block_shard as mod
+
+    pl = Fp8BucketedBlockShard(world_size=1, weight_factory=_factory, block_size=4)
+    param = nn.Parameter(torch.arange(64, dtype=torch.float32, device=device).view(8, 8))
+    (info,) = make_param_infos([("w", param)], pl, FakeMesh(1))
+    mesh = FakeMesh(1)
+    cached = pl.prepare_unshard_bucket([param.detach()], [info], mesh, None)
+    with patch.object(torch.compiler, "is_compiling", return_value=True):
+        first = pl.prepare_unshard_bucket([param.detach()], [info], mesh, None)
+        second = pl.prepare_unshard_bucket([param.detach()], [info], mesh, None)
+    with patch.object(mod, "_is_backward_graph_task", return_value=True):
+        restored = pl.prepare_unshard_bucket([param.detach()], [info], mesh, None)
+        again = pl.prepare_unshard_bucket([param.detach()], [info], mesh, None)
+    assert first.buffers[0] is not second.buffers[0] and first.buffers[0] is not cached.buffers[0]
+    assert restored.buffers[0] is cached.buffers[0]
+    assert again.buffers[0] is not cached.buffers[0]  # the entry is consumed once
+    assert torch.equal(again.buffers[0], cached.buffers[0])
+
+
+def test_argument_errors(device):
+    pl = Fp8BucketedBlockShard(world_size=1, weight_factory=_factory, block_size=4)
+    param = nn.Parameter(torch.zeros(8, 8, device=device))
+    infos = make_param_infos([("w", param)], pl, FakeMesh(1))
+    with pytest.raises(ValueError, match="one tensor per ParamInfo"):
+        pl.prepare_unshard_bucket([], infos, FakeMesh(1), None)
+    with pytest.raises((AssertionError, RuntimeError)):
+        pl.prepare_unshard_bucket([torch.zeros(4, 8, device=device)], infos, FakeMesh(1), None)
+    payload = torch.empty(10, dtype=torch.uint8, device=device)
+    spec = hip_ops.QuantChunkSpec(torch.zeros(4, 4, dtype=torch.bfloat16, device=device), 0, 16, hip_ops.SRC_BF16)
+    with pytest.raises(RuntimeError, match="outside payload"):
+        hip_ops.quantize_pack([spec], payload, ((0, 0), (0, 0)), 4)
+
+
+# ------------------------------------------------------------ full-size cases
+def test_llama_layer_bucket_rank0_and_worst_rank(device, golden):
+    """Config 2 at full size: rank 0's share (27 262 976 elements, 4 chunks)
+    bit-exact against the C oracle, every rank's payload consistent with
+    whole-matrix quantization on the GPU (quantize-then-gather ==
+    gather-then-quantize)."""
+    g = golden["llama3_8b_layer_plan"]
+    named = seeded_bucket(LLAMA3_8B_LAYER, 0.02, 100, device)
+    pl = Fp8BucketedBlockShard(world_size=8, weight_factory=_factory)
+    prepared = prepare_unshard_on_each_rank(pl, named, 8)
+    md = prepared[0].placement_state.metadata
+    assert md.packed_send_nbytes_per_rank == g["row_nbytes"] and md.rank_qdata_numels[0] == g["rank0_numel"]
+    # rank 0 against the oracle, chunk by chunk
+    payload0 = prepared[0].buffers[0].cpu()
+    infos0 = make_param_infos(named, pl, FakeMesh(8, 0))
+    cursor, scale_cursor = 0, md.rank_scale_byte_offsets[0]
+    for (fqn, param), info in zip(named, infos0):
+        if info.local_numel == 0:
+            continue
+        shard = local_rows(param, info).cpu().flatten(0, -2)
+        oq, osc = cport.quantize_blockwise(shard, 128)
+        assert torch.equal(payload0[cursor : cursor + oq.numel()], oq.reshape(-1)), fqn
+        sb = osc.reshape(-1).view(torch.uint8)
+        assert torch.equal(payload0[scale_cursor : scale_cursor + sb.numel()], sb), fqn
+        cursor += oq.numel()
+        scale_cursor += sb.numel()
+    assert cursor == g["rank0_numel"] and (payload0[scale_cursor:] == 0).all()
+    # every rank against whole-matrix quantization on the GPU
+    whole = [_quantize_dense_weight_to_blockwise_fp8(p.detach(), 128, E4M3) for _, p in named]
+    data = torch.cat([q.view(torch.uint8).reshape(-1) for q, _ in whole])
+    scales = torch.cat([s.reshape(-1) for _, s in whole])
+    d_cursor = s_cursor = 0
+    for rank in range(8):
+        row = prepared[rank].buffers[0]
+        n, sn = md.rank_qdata_numels[rank], md.rank_scale_numels[rank]
+        assert torch.equal(row[:n], data[d_cursor : d_cursor + n]), f"rank {rank} data"
+        s0 = md.rank_scale_byte_offsets[rank]
+        assert torch.equal(row[s0 : s0 + 4 * sn].view(torch.float32), scales[s_cursor : s_cursor + sn]), f"rank {rank}"
+        d_cursor += n
+        s_cursor += sn
+    assert d_cursor == g["global_numel"]
+    # one whole matrix against the oracle as an anchor for the GPU-vs-GPU check
+    oq, osc = cport.quantize_blockwise(named[1][1].detach().cpu(), 128)
+    assert torch.equal(whole[1][0].view(torch.uint8).cpu(), oq) and torch.equal(_bits(whole[1][1].cpu()), _bits(osc))
+
+
+def test_deepseek_expert_bucket_edge_tiles(device):
+    """Config 3: stacked [32, 2048, 7168] / [32, 7168, 2048] experts with 50x
+    outliers and all-zero tiles; rank 0's share (w1 rows 0..24 575) is checked
+    against the oracle on sampled block rows that cover the edge cases."""
+    named = seeded_bucket(DEEPSEEK_V3_EXPERTS, 0.006, 300, device)
+    for i, (_, p) in enumerate(named):
+        add_outliers_and_zero_tiles(p, 400 + i)
+    w1 = named[0][1]
+    w1.data[0, :128, :] = 0  # one all-zero chunk row band on rank 0
+    pl = Fp8BucketedBlockShard(world_size=8, weight_factory=_factory)
+    mesh = FakeMesh(8, 0)
+    infos = make_param_infos(named, pl, mesh)
+    assert infos[0].local_numel == 24576 * 7168 and infos[1].local_numel == 0 and infos[2].local_numel == 0
+    shards = [local_rows(p, i) for (_, p), i in zip(named, infos)]
+    prepared = pl.prepare_unshard_bucket(shards, infos, mesh, None)
+    md = prepared.placement_state.metadata
+    assert md.rank_qdata_numels[0] == 176160768 and md.rank_scale_numels[0] == 10752
+    payload = prepared.buffers[0]
+    flat = w1.detach().flatten(0, -2)
+    gen = torch.Generator().manual_seed(7)
+    bands = sorted({0, 1, 191, *torch.randint(0, 192, (10,), generator=gen).tolist()})
+    s0 = md.rank_scale_byte_offsets[0]
+    scales = payload[s0 : s0 + 4 * 10752].view(torch.float32).view(192, 56)
+    zero_scale_bits = 0x27212492
+    saw_zero_tile = False
+    for band in bands:
+        rows = flat[band * 128 : (band + 1) * 128].cpu()
+        oq, osc = cport.quantize_blockwise(rows, 128)
+        got = payload[band * 128 * 7168 : (band + 1) * 128 * 7168].view(128, 7168).cpu()
+        assert torch.equal(got, oq), f"band {band}"
+        assert torch.equal(_bits(scales[band].cpu()), _bits(osc.view(-1))), f"band {band}"
+        saw_zero_tile |= bool((_bits(osc) == zero_scale_bits).any())
+    assert saw_zero_tile
+    assert (scales[0].view(torch.int32) == zero_scale_bits).all()

@@ -1,0 +1,325 @@
+"""GPU parity of the unpack side: rank-row compaction (segment copy), the fused
+compaction + dequantization kernel, and the dequantizer, against the oracle."""
+
+import pytest
+import torch
+import torch.nn as nn
+
+from flex_shard_amd import Fp8BucketedBlockShard
+from flex_shard_amd.blockwise_fp8 import BlockwiseFp8Weight, blockwise_dequant_weight, make_blockwise_fp8_weight
+from flex_shard_amd.custom_placements._copy_kernels import SegmentCopyDescriptor, copy_segments, zero_segments
+from flex_shard_amd.testing import (
+    LLAMA3_8B_LAYER,
+    FakeMesh,
+    gather_rank_rows,
+    make_param_infos,
+    prepare_unshard_on_each_rank,
+    seeded_bucket,
+)
+from oracle import cport
+from oracle import layout as olayout
+
+pytestmark = pytest.mark.gpu
+E4M3 = torch.float8_e4m3fn
+
+
+class RecordingFactory:
+    def __init__(self):
+        self.calls = []
+
+    def __call__(self, fp8_data, recip_scale, block_size, *, orig_dtype, requires_grad):
+        self.calls.append((fp8_data, recip_scale, block_size, orig_dtype, requires_grad))
+        return fp8_data
+
+
+def _return_fp8(fp8_data, recip_scale, block_size, *, orig_dtype, requires_grad):
+    return fp8_data
+
+
+def _bits(t):
+    return t.contiguous().view(torch.int32)
+
+
+def test_compacts_strided_rank_rows_into_shared_storage(device, golden):
+    """Reference case: W=8, block 4, params 16x8, 8x8, 1x3 of arange values,
+    gathered rows strided and starting at an odd byte; the compact buffer is
+    align16(sum numel) + 4 * sum scales bytes, every factory view shares its
+    storage, and bytes/scales equal whole-matrix quantization."""
+    g = golden["compact_unshard_case"]
+    block, world = g["block"], g["world_size"]
+    factory = RecordingFactory()
+    pl = Fp8BucketedBlockShard(world_size=world, weight_factory=factory, block_size=block)
+    named = []
+    for i, shape in enumerate(g["shapes"]):
+        n = shape[0] * shape[1]
+        named.append((f"w{i + 1}", nn.Parameter(torch.arange(n, dtype=torch.float32, device=device).reshape(shape))))
+    prepared_by_rank = prepare_unshard_on_each_rank(pl, named, world)
+    prepared = prepared_by_rank[0]
+    md = prepared.placement_state.metadata
+    row = md.packed_send_nbytes_per_rank
+    parent = torch.full((world, row + g["row_extra_bytes"]), 0xFF, dtype=torch.uint8, device=device)
+    rank_rows = parent[:, g["row_byte_offset"] : row + g["row_byte_offset"]]
+    assert not rank_rows.is_contiguous() and rank_rows.storage_offset() % 4 == 1
+    for rank, p in enumerate(prepared_by_rank):
+        local = p.buffers[0]
+        n, s0, end = md.rank_qdata_numels[rank], md.rank_scale_byte_offsets[rank], md.rank_packed_nbytes[rank]
+        rank_rows[rank, :n].copy_(local[:n])
+        rank_rows[rank, s0:end].copy_(local[s0:end])
+    prepared.persistent = True
+    result = pl._finish_unshard_from_rank_rows(prepared, rank_rows)
+    (compact,) = result.persistent_buffers
+    fp8_nbytes = sum(p.numel() for _, p in named)
+    assert fp8_nbytes % 4 != 0 and 0 in md.rank_qdata_numels
+    scale_numel = sum(-(-p.shape[0] // block) * -(-p.shape[1] // block) for _, p in named)
+    assert compact.dtype == torch.uint8 and compact.numel() == -(-fp8_nbytes // 16) * 16 + 4 * scale_numel
+    base = compact.untyped_storage().data_ptr()
+    for weight, call, (_, full) in zip(result.full_params, factory.calls, named, strict=True):
+        fp8, recip, blk, orig_dtype, requires_grad = call
+        oq, osc = cport.quantize_blockwise(full.detach().cpu(), block)
+        assert weight is fp8 and blk == block and orig_dtype == full.dtype and requires_grad == full.requires_grad
+        assert fp8.is_contiguous() and recip.is_contiguous()
+        assert fp8.untyped_storage().data_ptr() == base and recip.untyped_storage().data_ptr() == base
+        assert torch.equal(fp8.view(torch.uint8).cpu(), oq) and torch.equal(_bits(recip.cpu()), _bits(osc))
+    # a persistent refill writes the same buffer in place and returns it
+    prepared.persistent_buffers = [compact]
+    compact.fill_(0x55)
+    again = pl._finish_unshard_from_rank_rows(prepared, rank_rows)
+    assert again.persistent_buffers[0] is compact
+    assert torch.equal(factory.calls[-3][0].view(torch.uint8).cpu(), cport.quantize_blockwise(named[0][1].detach().cpu(), block)[0])
+
+
+def test_stacked_weight_is_quantized_as_flattened_matrix(device):
+    factory = RecordingFactory()
+    pl = Fp8BucketedBlockShard(world_size=3, weight_factory=factory, block_size=4)
+    torch.manual_seed(0)
+    param = nn.Parameter(torch.randn(2, 6, 8, device=device))
+    prepared = prepare_unshard_on_each_rank(pl, [("w13", param)], 3)
+    pl._finish_unshard_from_rank_rows(prepared[0], gather_rank_rows(prepared))
+    ((fp8, recip, *_),) = factory.calls
+    oq, osc = cport.quantize_blockwise(param.detach().cpu().flatten(0, -2), 4)
+    assert fp8.shape == param.shape
+    assert torch.equal(fp8.flatten(0, -2).view(torch.uint8).cpu(), oq) and torch.equal(_bits(recip.cpu()), _bits(osc))
+
+
+def test_fused_copy_out_matches_oracle_for_every_row_layout(device, golden):
+    """Aligned and odd region sizes x contiguous / spaced / odd-offset rows:
+    the one-launch copy-out equals the oracle's compaction byte for byte, and
+    bytes outside the written regions keep their old value."""
+    g = golden["fused_copy_out_cases"]
+    for case_name, case in g["cases"].items():
+        pl = Fp8BucketedBlockShard(world_size=g["world_size"], weight_factory=_return_fp8, block_size=g["block"])
+        named = [(f"w{i}", nn.Parameter(torch.empty(tuple(s), device="meta"))) for i, s in enumerate(case["shapes"])]
+        infos = make_param_infos(named, pl, FakeMesh(g["world_size"]))
+        md = pl._quant_metadata_from_infos(infos)
+        lay = olayout.quant_layout(case["shapes"], g["block"], g["world_size"])
+        world, row = g["world_size"], md.packed_send_nbytes_per_rank
+        assert row == lay.row_nbytes
+        for layout_name, (offset, padding) in g["row_layouts"].items():
+            gen = torch.Generator().manual_seed(1)
+            parent = torch.randint(0, 256, (world, offset + row + padding), dtype=torch.uint8, generator=gen)
+            rows_cpu = parent[:, offset : offset + row]
+            rows_gpu = parent.to(device)[:, offset : offset + row]
+            want = olayout.compact_from_rank_rows(lay, rows_cpu, fill=0xAB)
+            fused = torch.full((want.numel(),), 0xAB, dtype=torch.uint8, device=device)
+            assert pl._copy_out_rank_rows_fused(md, rows_gpu, fused)
+            assert torch.equal(fused.cpu(), want), f"{case_name} / {layout_name}"
+            plan = pl._copy_out_plan(md, data_elem_nbytes=1, with_scales=True)
+            unit = case["aligned_unit"] if offset == 0 else 1
+            assert (rows_gpu.device, rows_gpu.stride(0), unit) in plan.descriptors
+            # the torch.cat form used under torch.compile agrees
+            cat = torch.full_like(fused, 0xAB)
+            data_total = sum(md.rank_qdata_numels)
+            pl._copy_out_rank_rows_cat(md, rows_gpu, cat, qdata_nbytes=data_total, scale_byte_offset=-(-data_total // 16) * 16)
+            assert torch.equal(cat, fused)
+
+
+def test_copy_plan_is_built_once_per_row_stride(device):
+    pl = Fp8BucketedBlockShard(world_size=8, weight_factory=_return_fp8, block_size=4)
+    named = [(f"w{i}", nn.Parameter(torch.empty(s, device="meta"))) for i, s in enumerate([(16, 8), (8, 8), (6, 4)])]
+    md = pl._quant_metadata_from_infos(make_param_infos(named, pl, FakeMesh(8)))
+    row = md.packed_send_nbytes_per_rank
+    compact = torch.empty(row * 8, dtype=torch.uint8, device=device)
+    rows = torch.zeros((8, row), dtype=torch.uint8, device=device)
+    pl._copy_out_rank_rows_fused(md, rows, compact)
+    plan = pl._copy_out_plan(md, data_elem_nbytes=1, with_scales=True)
+    (descriptor,) = plan.descriptors.values()
+    pl._copy_out_rank_rows_fused(md, rows, compact)
+    assert list(plan.descriptors.values()) == [descriptor]
+    spaced = torch.zeros((8, row + 16), dtype=torch.uint8, device=device)[:, :row]
+    pl._copy_out_rank_rows_fused(md, spaced, compact)
+    assert len(plan.descriptors) == 2
+
+
+def test_copy_out_falls_back_only_while_compiling(device):
+    from unittest.mock import patch
+
+    pl = Fp8BucketedBlockShard(world_size=8, weight_factory=_return_fp8, block_size=4)
+    named = [("w0", nn.Parameter(torch.empty(16, 8, device="meta")))]
+    md = pl._quant_metadata_from_infos(make_param_infos(named, pl, FakeMesh(8)))
+    rows = torch.zeros((8, md.packed_send_nbytes_per_rank), dtype=torch.uint8, device=device)
+    compact = torch.empty(rows.numel(), dtype=torch.uint8, device=device)
+    with patch.object(torch.compiler, "is_compiling", return_value=True):
+        assert not pl._copy_out_rank_rows_fused(md, rows, compact)
+    with pytest.raises(RuntimeError, match="no CPU compute path"):
+        pl._copy_out_rank_rows_fused(md, rows.cpu(), compact)
+    with pytest.raises(ValueError, match="shape"):
+        prepared = prepare_unshard_on_each_rank(
+            pl, [("w0", nn.Parameter(torch.zeros(16, 8, device=device)))], 8
+        )[0]
+        pl._finish_unshard_from_rank_rows(prepared, rows[:, :-16])
+    with pytest.raises(ValueError, match="uint8"):
+        pl._finish_unshard_from_rank_rows(prepared, rows.view(torch.int8))
+
+
+def test_dense_rows_join_with_wider_elements(device):
+    """data_elem_nbytes=2 without scales: joins bf16 rank rows (the dense
+    all-gather reference layout) in rank order."""
+    pl = Fp8BucketedBlockShard(world_size=8, weight_factory=_return_fp8, block_size=4)
+    named = [(f"w{i}", nn.Parameter(torch.empty(s, device="meta"))) for i, s in enumerate([(16, 8), (8, 8), (1, 3)])]
+    md = pl._quant_metadata_from_infos(make_param_infos(named, pl, FakeMesh(8)))
+    for row_numel in (max(md.rank_qdata_numels) + 5, 64):
+        rows = torch.randn((8, row_numel), dtype=torch.bfloat16, device=device)
+        joined = rows.new_empty(sum(md.rank_qdata_numels))
+        assert pl._copy_out_rank_rows_fused(
+            md, rows.view(torch.uint8), joined.view(torch.uint8), data_elem_nbytes=2, with_scales=False
+        )
+        want = torch.cat([rows[r, :n] for r, n in enumerate(md.rank_qdata_numels)])
+        assert torch.equal(joined.view(torch.int16), want.view(torch.int16))
+
+
+def test_segment_copy_splits_long_segments(device, golden):
+    g = golden["segment_split_case"]
+    gen = torch.Generator().manual_seed(2)
+    source = torch.randint(-(2**31), 2**31 - 1, (g["source_numel"],), dtype=torch.int32, generator=gen).to(device)
+    segs = g["segments"]
+    desc = SegmentCopyDescriptor.create(
+        src_offsets=[s for s, _, _ in segs], numels=[n for _, n, _ in segs], dst_offsets=[d for _, _, d in segs],
+        device=device, block_size=g["block_size"], max_chunks_per_segment=g["max_chunks_per_segment"],
+    )
+    assert desc.nsegments > len(segs) and desc.max_segment_numel == g["max_segment_numel"]
+    out = torch.zeros(g["output_numel"], dtype=torch.int32, device=device)
+    copy_segments(source, out, desc)
+    want = torch.zeros_like(out)
+    for s, n, d in segs:
+        want[d : d + n] = source[s : s + n]
+    assert torch.equal(out, want)
+    # every unit size, odd relative alignment, and the zero kernel
+    for dtype in (torch.uint8, torch.int16, torch.int32, torch.int64):
+        src = torch.randint(0, 100, (5000,), generator=gen).to(dtype).to(device)
+        dst = torch.full((6000,), 7, dtype=dtype, device=device)
+        d2 = SegmentCopyDescriptor.create(src_offsets=[3, 1001], numels=[997, 3333], dst_offsets=[10, 1500], device=device)
+        copy_segments(src, dst, d2)
+        ref = torch.full((6000,), 7, dtype=dtype, device=device)
+        ref[10:1007] = src[3:1000]
+        ref[1500:4833] = src[1001:4334]
+        assert torch.equal(dst, ref)
+        zero_segments(dst, d2)
+        ref[10:1007] = 0
+        ref[1500:4833] = 0
+        assert torch.equal(dst, ref)
+
+
+# ---------------------------------------------------------------- dequantize
+def test_dequant_known_answers(device, golden):
+    g = golden["dequant_flat"]
+    fp8 = torch.arange(128, dtype=torch.bfloat16).reshape(g["shape"]).to(E4M3).to(device)
+    scale = torch.full(g["scale_shape"], g["scale"], dtype=torch.float32, device=device)
+    wrapped = BlockwiseFp8Weight(fp8, scale, g["block"], orig_dtype=torch.bfloat16, requires_grad=True)
+    assert wrapped.dtype == torch.bfloat16 and wrapped.requires_grad and wrapped.block_size == 4
+    assert torch.equal(wrapped.dequantize(torch.float32), fp8.float() * g["scale"])
+    assert torch.equal(wrapped.dequantize(), (fp8.float() * g["scale"]).bfloat16())
+
+    g = golden["dequant_stacked"]
+    fp8 = torch.arange(96, dtype=torch.bfloat16).reshape(g["shape"]).to(E4M3).to(device)
+    scale = torch.tensor(g["scales"], dtype=torch.float32, device=device)
+    wrapped = make_blockwise_fp8_weight(fp8, scale, g["block"], orig_dtype=torch.bfloat16, requires_grad=False)
+    per_elem = scale.repeat_interleave(4, 0).repeat_interleave(4, 1).view(g["shape"])
+    assert wrapped.shape == tuple(g["shape"])
+    assert torch.equal(wrapped.dequantize(torch.float32), fp8.float() * per_elem)
+    with pytest.raises(ValueError, match="scale shape"):
+        BlockwiseFp8Weight(fp8, scale[:2], 4)
+
+
+@pytest.mark.parametrize("shape,block", [((256, 384), 128), ((200, 136), 128), ((130, 129), 128), ((16, 32), 4), ((300, 208), 64)])
+def test_dequant_is_bit_exact_with_oracle(device, shape, block):
+    """Every FP8 byte value times random scales, fp32 and bf16 outputs: 0 ULP."""
+    gen = torch.Generator().manual_seed(3)
+    data = torch.randint(0, 256, shape, dtype=torch.uint8, generator=gen)
+    data[(data & 0x7F) == 0x7F] = 0x3C  # NaN encodings are compared separately
+    scale = torch.rand(-(-shape[0] // block), -(-shape[1] // block), generator=gen) * 1e-3 + 1e-6
+    for dtype in (torch.float32, torch.bfloat16):
+        got = blockwise_dequant_weight(data.to(device).view(E4M3), scale.to(device), block, dtype).cpu()
+        want = cport.dequant_blockwise(data, scale, block, dtype)
+        view = torch.int32 if dtype == torch.float32 else torch.int16
+        assert torch.equal(got.view(view), want.view(view))
+    nan = torch.full((4, 4), 0x7F, dtype=torch.uint8)
+    assert blockwise_dequant_weight(nan.to(device).view(E4M3), torch.ones(1, 1, device=device), 4).isnan().all()
+
+
+def test_fused_unpack_with_dequant_matches_oracle(device):
+    """finish_prepared_unshard_with_dequant: FP8 views as in the plain finish,
+    plus bf16 weights equal to dequantizing the gathered weight (0 ULP), from
+    strided rows at an odd offset as well."""
+    for shapes, block, world in (([(16, 8), (8, 8), (1, 3)], 4, 8), ([(512, 256), (256, 384), (130, 136)], 128, 4),
+                                 ([(1024, 512), (3, 256, 256)], 128, 8)):
+        factory = RecordingFactory()
+        pl = Fp8BucketedBlockShard(world_size=world, weight_factory=factory, block_size=block)
+        gen = torch.Generator().manual_seed(4)
+        named = [
+            (f"w{i}", nn.Parameter((torch.randn(s, generator=gen) * 0.02).bfloat16().to(device), requires_grad=False))
+            for i, s in enumerate(shapes)
+        ]
+        prepared = prepare_unshard_on_each_rank(pl, named, world)
+        rows = gather_rank_rows(prepared)
+        parent = torch.zeros((world, rows.shape[1] + 5), dtype=torch.uint8, device=device)
+        parent[:, 3 : 3 + rows.shape[1]] = rows
+        for rank_rows in (rows, parent[:, 3 : 3 + rows.shape[1]]):
+            factory.calls.clear()
+            result, dequant = pl.finish_prepared_unshard_with_dequant(prepared[0], rank_rows)
+            plain = pl._finish_unshard_from_rank_rows(prepared[0], rank_rows)
+            for (_, p), call, deq, plain_fp8 in zip(named, factory.calls, dequant, plain.full_params):
+                oq, osc = cport.quantize_blockwise(p.detach().cpu().flatten(0, -2), block)
+                assert torch.equal(call[0].flatten(0, -2).view(torch.uint8).cpu(), oq)
+                assert torch.equal(_bits(call[1].cpu()), _bits(osc))
+                assert torch.equal(plain_fp8.view(torch.uint8), call[0].view(torch.uint8))
+                want = cport.dequant_blockwise(oq, osc, block)
+                assert deq.shape == p.shape and deq.dtype == torch.bfloat16
+                assert torch.equal(deq.flatten(0, -2).cpu().view(torch.int16), want.view(torch.int16))
+        _, only_dequant = pl.finish_prepared_unshard_with_dequant(prepared[0], rows, compact=False)
+        assert all(torch.equal(a, b) for a, b in zip(only_dequant, dequant))
+
+
+def test_llama_gathered_layout_unpack_full_size(device, golden):
+    """Config 2 unpack: the 8-rank gathered layout [8, 27 531 840] built from 8
+    locally quantized seeded shards; the compact buffer must equal whole-matrix
+    quantization, the fused dequant must equal dequantizing it, and
+    encode -> gather -> decode must stay within the FP8 error bound."""
+    g = golden["llama3_8b_layer_plan"]
+    factory = RecordingFactory()
+    pl = Fp8BucketedBlockShard(world_size=8, weight_factory=factory)
+    named = seeded_bucket(LLAMA3_8B_LAYER, 0.02, 100, device)
+    prepared = prepare_unshard_on_each_rank(pl, named, 8)
+    rows = gather_rank_rows(prepared)
+    assert tuple(rows.shape) == (8, g["row_nbytes"])
+    result, dequant = pl.finish_prepared_unshard_with_dequant(prepared[0], rows)
+    plain = pl._finish_unshard_from_rank_rows(prepared[0], rows)
+    from flex_shard_amd.custom_placements.fp8_bucketed_block_shard import _quantize_dense_weight_to_blockwise_fp8
+
+    for index, ((fqn, p), fp8, deq) in enumerate(zip(named, result.full_params, dequant)):
+        wq, ws = _quantize_dense_weight_to_blockwise_fp8(p.detach(), 128, E4M3)
+        recip = factory.calls[index][1]
+        assert torch.equal(fp8.view(torch.uint8), wq.view(torch.uint8)), fqn
+        assert torch.equal(recip.view(torch.int32), ws.view(torch.int32)), fqn
+        assert torch.equal(plain.full_params[index].view(torch.uint8), fp8.view(torch.uint8)), fqn
+        ref = blockwise_dequant_weight(wq, ws, 128, torch.bfloat16)
+        assert torch.equal(deq.view(torch.int16), ref.view(torch.int16)), fqn
+        # round trip: |deq - w| <= amax_tile / 16 (+ bf16 rounding of the result)
+        tiles_r, tiles_c = p.shape[0] // 128, p.shape[1] // 128
+        amax = p.detach().float().view(tiles_r, 128, tiles_c, 128).abs().amax(dim=(1, 3))
+        bound = (amax / 16 * 1.01).repeat_interleave(128, 0).repeat_interleave(128, 1)
+        assert ((deq.float() - p.detach().float()).abs() <= bound).all(), fqn
+    # anchor one gathered parameter against the CPU oracle
+    k = named[1][1].detach().cpu()
+    oq, osc = cport.quantize_blockwise(k, 128)
+    assert torch.equal(result.full_params[1].view(torch.uint8).cpu(), oq)
+    assert torch.equal(dequant[1].cpu().view(torch.int16), cport.dequant_blockwise(oq, osc, 128).view(torch.int16))
