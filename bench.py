@@ -1,0 +1,328 @@
+#!/usr/bin/env python3
+"""Benchmark of the single-GPU hot path on one MI355X.
+
+Headline: fused FP8 tile quantize + pack of one rank's share (rank 0 of 8) of a
+Llama-3-8B layer bucket: q, k, v and the first 512 rows of o = 27 262 976 bf16
+elements in 4 chunks, packed into a 27 531 840-byte payload.  A step is one
+such launch on one layer's shards; steps rotate over `--layers` distinct layer
+buckets so the inputs come from HBM, not from the 256 MB last-level cache.
+`value` is algorithmic bytes moved per second over the whole timed region,
+inputs resident in HBM.
+
+One JSON line is printed.  Besides the contract fields it carries
+  roofline      the dominant kernel against the 8 TB/s HBM peak, timed with
+                events on the launch stream over the same timed region
+  cpu_baseline  the oracle's eager-torch restatement of the reference path on
+                the host cores, on the same rank-0 share
+  secondary     unpack+dequant of the 8-rank gathered layout, the fp32
+                gradient path, and the 48-matrix Muon / Newton-Schulz step
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor figure
+BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
+
+
+def _factory(fp8_data, recip_scale, block_size, *, orig_dtype, requires_grad):
+    return fp8_data
+
+
+def _event_ms(fn, steps: int, warmup: int) -> tuple[float, float]:
+    """(wall ms, event ms) for `steps` calls of fn(i) after `warmup` calls."""
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(steps):
+        fn(i)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3
+    return wall, start.elapsed_time(stop)
+
+
+def build_quant_workload(device, layers: int):
+    """Per layer: rank 0's local shards as views of one flat bf16 storage (the
+    sharded bucket storage layout), their ParamInfos, and a reusable payload."""
+    import torch.nn as nn
+
+    from flex_shard_amd import Fp8BucketedBlockShard
+    from flex_shard_amd.testing import LLAMA3_8B_LAYER, FakeMesh, make_param_infos, seeded_normal
+
+    placement = Fp8BucketedBlockShard(world_size=8, weight_factory=_factory)
+    mesh = FakeMesh(8, 0)
+    meta = [(n, nn.Parameter(torch.empty(s, device="meta", dtype=torch.bfloat16))) for n, s in LLAMA3_8B_LAYER]
+    infos = make_param_infos(meta, placement, mesh)
+    local_numel = infos[0].bucket_layout.local_numel
+    work = []
+    for layer in range(layers):
+        storage = seeded_normal((local_numel,), 0.02, 1000 + layer, device)
+        shards = [
+            storage[i.byte_offset // 2 : i.byte_offset // 2 + i.local_numel].view(i.local_shape) for i in infos
+        ]
+        work.append((storage, shards))
+    return placement, mesh, infos, work
+
+
+def bench_quant_pack(device, steps, warmup, layers):
+    placement, mesh, infos, work = build_quant_workload(device, layers)
+    metadata = placement._quant_metadata_from_infos(infos)
+    plan = metadata.rank_pack_plans[0]
+    elems = plan.qdata_numel
+    scales = sum(sum(c.scale_numels) for c in plan.chunks)
+    algo_bytes = 3 * elems + 4 * scales  # 2 B read + 1 B write per element, 4 B per tile scale
+    payloads = [torch.empty(metadata.packed_send_nbytes_per_rank, dtype=torch.uint8, device=device) for _ in work]
+
+    def step(i):
+        _, shards = work[i % len(work)]
+        # The placement's own entry point; the payload buffer is recycled the
+        # way the caching allocator recycles it in a training loop.
+        payloads[i % len(work)] = placement._pack_local_quantized_chunks(shards, infos, 0, metadata)
+
+    wall_ms, event_ms = _event_ms(step, steps, warmup)
+    # Hot-cache variant (one layer over and over) for the record.
+    _, hot_ms = _event_ms(lambda i: step(0), steps, 5)
+    return {
+        "elems": elems,
+        "algo_bytes": algo_bytes,
+        "wall_ms": wall_ms,
+        "event_ms": event_ms,
+        "hot_event_ms": hot_ms,
+        "payload_nbytes": metadata.packed_send_nbytes_per_rank,
+        "chunks": len(plan.chunks),
+        "work": (placement, infos, work, metadata, payloads),
+    }
+
+
+def check_against_oracle(placement, infos, work, metadata, payloads):
+    """Bit-exactness gate before any timing is reported: one chunk of the last
+    payload against the C oracle."""
+    from oracle import cport
+
+    storage, shards = work[0]
+    payload = placement._pack_local_quantized_chunks(shards, infos, 0, metadata).cpu()
+    k = shards[1].detach().cpu().flatten(0, -2)
+    oq, osc = cport.quantize_blockwise(k, 128)
+    start = shards[0].numel()
+    ok = torch.equal(payload[start : start + oq.numel()], oq.reshape(-1))
+    s0 = metadata.rank_scale_byte_offsets[0] + 4 * (32 * 32)
+    ok &= torch.equal(payload[s0 : s0 + 4 * osc.numel()].view(torch.float32), osc.reshape(-1))
+    if not ok:
+        raise SystemExit("bench: GPU payload differs from the oracle; refusing to report a timing")
+
+
+def cpu_baseline_quant(work, infos, metadata, budget_s: float = 20.0):
+    """The reference path in eager torch on the host: per chunk quantize
+    (pad, amax, clamp, fp64 divide, multiply, clamp, cast), then copy data and
+    scale bytes into the payload.  Same rank-0 share as the GPU step."""
+    from oracle import eager
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    _, shards = work[0]
+    cpu_shards = [s.detach().cpu() for s in shards]
+    plan = metadata.rank_pack_plans[0]
+    payload = torch.zeros(metadata.packed_send_nbytes_per_rank, dtype=torch.uint8)
+
+    def run():
+        cursor, scale_cursor = 0, plan.scale_byte_offset
+        for chunk in plan.chunks:
+            q, s = eager.quantize_blockwise(cpu_shards[chunk.param_index].reshape(chunk.local_shape), 128)
+            payload[cursor : cursor + q.numel()] = q.view(torch.uint8).reshape(-1)
+            sb = s.reshape(-1).view(torch.uint8)
+            payload[scale_cursor : scale_cursor + sb.numel()] = sb
+            cursor += q.numel()
+            scale_cursor += sb.numel()
+
+    run()  # warm-up
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 15):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    return times[len(times) // 2], len(times), torch.get_num_threads()
+
+
+def bench_unpack(device, placement, infos, reps=10):
+    """Unpack of the 8-rank gathered layout + bf16 dequant: 218 103 808 FP8
+    elements, 1 B read + 1 B compact write + 2 B dequant write per element."""
+    import torch.nn as nn
+
+    from flex_shard_amd.testing import LLAMA3_8B_LAYER, FakeMesh, make_param_infos
+
+    md = placement._quant_metadata_from_infos(infos)
+    rows = torch.randint(0, 120, (8, md.packed_send_nbytes_per_rank), dtype=torch.uint8, device=device)
+    for r in range(8):
+        s0 = md.rank_scale_byte_offsets[r]
+        rows[r, s0 : s0 + 4 * md.rank_scale_numels[r]].view(torch.float32).fill_(1e-4)
+    prepared = placement._prepare_local_unshard_payload
+    from flex_shard_amd.placement_contract import PlacementPreparedUnshard
+
+    state = placement._QuantUnshardState(infos=infos, pg=None, debug_fqn=None, metadata=md)
+    local = rows[0]
+    prep = PlacementPreparedUnshard(placement=placement, buffers=[local, rows.view(-1)], placement_state=state)
+    total = sum(i.global_numel for i in infos)
+    out = torch.empty(total, dtype=torch.bfloat16, device=device)
+    prep.persistent = True
+    result, _ = placement.finish_prepared_unshard_with_dequant(prep, rows, dequant_out=out)
+    prep.persistent_buffers = result.persistent_buffers
+    _, fused_ms = _event_ms(lambda i: placement.finish_prepared_unshard_with_dequant(prep, rows, dequant_out=out), reps, 2)
+    _, compact_ms = _event_ms(lambda i: placement._finish_unshard_from_rank_rows(prep, rows), reps, 2)
+    scales = sum(md.rank_scale_numels)
+    return {
+        "elems": total,
+        "fused_unpack_dequant_ms": fused_ms / reps,
+        "fused_GBps": (4 * total + 8 * scales) / (fused_ms / reps) / 1e6,
+        "compact_only_ms": compact_ms / reps,
+        "compact_GBps": (2 * total + 8 * scales) / (compact_ms / reps) / 1e6,
+    }
+
+
+def bench_gradients(device, reps=5):
+    """Config 4: 4 bf16 microbatches accumulated in fp32 over the 218 365 952
+    element bucket (placement layout), then the 8-way fixed-order reduction of
+    rank 0's 27 295 744-element range."""
+    from flex_shard_amd import hip_ops
+    from flex_shard_amd.testing import seeded_normal
+
+    total, seg, world = 218365952, 27295744, 8
+    acc = torch.zeros(total, device=device)
+    micro = [seeded_normal((total,), 1e-3, 500 + k, device) for k in range(4)]
+    _, acc_ms = _event_ms(lambda i: hip_ops.accumulate_grad(acc, micro[i % 4], overwrite=(i % 4 == 0)), 4 * reps, 4)
+    del micro
+    contrib = torch.empty((world, total), device=device)
+    contrib.normal_(0, 1e-3)
+    out = torch.empty(seg, device=device)
+    _, red_ms = _event_ms(lambda i: hip_ops.reduce_rows(out, contrib, 0), reps * 4, 2)
+    acc_per = acc_ms / (4 * reps)
+    red_per = red_ms / (reps * 4)
+    return {
+        "accumulate_ms_per_microbatch": acc_per,
+        "accumulate_GBps": 10 * total / acc_per / 1e6,  # 2 B grad + 4 B read + 4 B write (6 B on the first)
+        "reduce_ms": red_per,
+        "reduce_GBps": 36 * seg / red_per / 1e6,  # 8 x 4 B read + 4 B write per output element
+    }
+
+
+def bench_muon(device, reps=3):
+    """Config 5: 24 x [7168, 2048] + 24 x [2048, 2048] bf16 whole matrices, one
+    Muon step (momentum, Nesterov, 5 Newton-Schulz steps, update)."""
+    from flex_shard_amd.dist_muon import OwnedMuon
+    from flex_shard_amd.testing import seeded_normal
+
+    shapes = [(7168, 2048)] * 24 + [(2048, 2048)] * 24
+    params = [seeded_normal(s, 0.02, 2000 + i, device) for i, s in enumerate(shapes)]
+    grads = [seeded_normal(s, 1.0, 3000 + i, device) for i, s in enumerate(shapes)]
+    opt = OwnedMuon(params)
+    _, ms = _event_ms(lambda i: opt.step(grads), reps, 1)
+    per = ms / reps
+    flops = opt.flops_per_step()
+    return {"step_ms": per, "ns_flop": flops, "ns_TFLOPs": flops / per / 1e9,
+            "frac_of_bf16_mfma_peak": flops / per / 1e9 / BF16_MFMA_PEAK_TFLOPS}
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--layers", type=int, default=8, help="distinct layer buckets the steps rotate over")
+    ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--skip-secondary", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit(
+            "bench.py measures one rank's share of the path on one GPU; this build has no collectives, "
+            "so --gpus must be 1."
+        )
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs an MI355X; no GPU is visible.")
+    from flex_shard_amd import _native
+
+    _native.lib()  # fail loudly if the HIP library is missing
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    q = bench_quant_pack(device, args.steps, args.warmup, args.layers)
+    placement, infos, work, metadata, payloads = q.pop("work")
+    check_against_oracle(placement, infos, work, metadata, payloads)
+    ms_per_step = q["wall_ms"] / args.steps
+    value = q["algo_bytes"] / (ms_per_step * 1e-3) / 1e9
+    kernel_ms = q["event_ms"] / args.steps
+    achieved = q["algo_bytes"] / (kernel_ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "FP8 quantize+pack GB/s (% HBM peak), Llama-3-8B layer bucket; Muon NS TFLOP/s",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16->fp8_e4m3fn (fp32 scales)",
+        "data": "synthetic: seeded N(0, 0.02) bf16 shards, random-init",
+        "config": {
+            "workload": "Llama-3-8B layer bucket (q,k,v,o,gate,up,down), rank 0 of 8: q, k, v, o[0:512] = "
+            f"{q['elems']} bf16 elements in {q['chunks']} chunks -> {q['payload_nbytes']}-byte FP8 payload, "
+            f"128x128 tiles; steps rotate over {args.layers} layer buckets (cold HBM)",
+            "device": torch.cuda.get_device_name(0),
+            "percent_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 1),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "quantize_pack_kernel",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "algorithmic_bytes_per_launch": q["algo_bytes"],
+            "avg_launch_us": round(kernel_ms * 1e3, 2),
+            "avg_launch_us_hot_cache": round(q["hot_event_ms"] / args.steps * 1e3, 2),
+        },
+    }
+    if not args.skip_cpu:
+        median_s, reps, threads = cpu_baseline_quant(work, infos, metadata)
+        result["cpu_baseline"] = {
+            "value": round(q["algo_bytes"] / median_s / 1e9, 3),
+            "unit": "GB/s",
+            "cores": threads,
+            "kind": "port",
+            "sample": f"eager-torch restatement of the reference path on the same rank-0 share "
+            f"({q['elems']} elements), median of {reps} runs, {threads} threads of {os.cpu_count()} logical CPUs",
+        }
+    del work, payloads
+    torch.cuda.empty_cache()
+    if not args.skip_secondary:
+        secondary = {}
+        secondary["unpack_gathered_layout"] = {k: round(v, 3) if isinstance(v, float) else v
+                                               for k, v in bench_unpack(device, placement, infos).items()}
+        torch.cuda.empty_cache()
+        secondary["gradient_path"] = {k: round(v, 3) for k, v in bench_gradients(device).items()}
+        torch.cuda.empty_cache()
+        muon = bench_muon(device)
+        secondary["muon_newton_schulz"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in muon.items()}
+        result["secondary"] = secondary
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

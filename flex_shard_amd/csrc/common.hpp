@@ -60,14 +60,23 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   return (f != f) ? 0x7FC0u : r;
 }
 
-// Integer max across the 64 lanes of a wavefront.
+// Integer max across the 64 lanes of a wavefront, result in every lane.
+// Data-parallel-primitive moves: two quad permutes, two mirrors inside each
+// row of 16 lanes, then two row broadcasts leave the total in lane 63.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_max_u32(uint32_t v) {
+  const uint32_t o = static_cast<uint32_t>(
+      __builtin_amdgcn_update_dpp(static_cast<int>(v), static_cast<int>(v), CTRL, ROW_MASK, 0xF, false));
+  return o > v ? o : v;
+}
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) {
-    uint32_t o = static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), off, kWave));
-    v = o > v ? o : v;
-  }
-  return v;
+  v = dpp_max_u32<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
+  v = dpp_max_u32<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
+  v = dpp_max_u32<0x141, 0xF>(v);  // row_half_mirror
+  v = dpp_max_u32<0x140, 0xF>(v);  // row_mirror
+  v = dpp_max_u32<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3
+  v = dpp_max_u32<0x143, 0xC>(v);  // row_bcast31 into rows 2 and 3
+  return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), 63));
 }
 
 __device__ __forceinline__ float wave_sum_f32(float v) {

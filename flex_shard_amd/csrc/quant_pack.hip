@@ -5,7 +5,7 @@
 // one chunk.  For block = 128 each thread keeps its 64 tile elements in
 // registers between the amax pass and the cast pass, so the tile is read from
 // HBM exactly once: 16-byte loads (8 bf16), amax on raw magnitude bits with
-// packed 16-bit max, a 64-lane shuffle reduction plus a 4-entry LDS exchange,
+// packed 16-bit max, a 64-lane DPP reduction plus a 4-entry LDS exchange,
 // one fp64 division per tile for the scale, then v_cvt_pk_fp8_f32 and 8-byte
 // stores straight into the payload.  Extra workgroups zero the payload's pad
 // gaps, so nothing else has to touch the buffer.
@@ -247,6 +247,12 @@ __device__ void quant_tile_scalar(const QuantChunkDev& ch, int64_t tr, int64_t t
   }
 }
 
+// ALL_BF16_FAST: every chunk is a bf16 shard on the vector path.  That
+// instantiation carries only the 32-dword tile, stays under 64 VGPRs and so
+// keeps 8 workgroups resident per compute unit: the ~1700 tiles of a
+// Llama-sized rank share are then all in flight at once instead of running in
+// two uneven rounds.
+template <bool ALL_BF16_FAST>
 __global__ __launch_bounds__(kThreads) void quantize_pack_kernel(const QuantParams prm) {
   __shared__ uint32_t lds[4];
   const int64_t bid = blockIdx.x;
@@ -271,6 +277,10 @@ __global__ __launch_bounds__(kThreads) void quantize_pack_kernel(const QuantPara
   const int64_t t = bid - ch.tile_begin;
   const int64_t tr = t / ch.tiles_c;
   const int64_t tc = t - tr * ch.tiles_c;
+  if (ALL_BF16_FAST) {
+    quant_tile128_bf16<FSH_SRC_BF16>(ch, tr, tc, prm.payload, prm.eps[FSH_SRC_BF16], lds);
+    return;
+  }
   const float eps = prm.eps[ch.src_kind];
   if (ch.fast) {
     if (ch.src_kind == FSH_SRC_BF16)
@@ -327,6 +337,7 @@ FSH_API int fsh_quantize_pack(const fsh_quant_chunk* chunks, int32_t nchunks, vo
   prm.eps[FSH_SRC_F32_AS_BF16] = eps_bf16;
 
   int64_t tiles = 0;
+  bool all_bf16_fast = true;
   for (int i = 0; i < nchunks; ++i) {
     const fsh_quant_chunk& in = chunks[i];
     if (in.src_dev == nullptr || in.rows <= 0 || in.in_dim <= 0 || in.src_row_stride < in.in_dim)
@@ -356,6 +367,7 @@ FSH_API int fsh_quantize_pack(const fsh_quant_chunk* chunks, int32_t nchunks, vo
     out.src_kind = in.src_kind;
     out.fast = block == 128 && aligned(in.src_dev, 16) && (in.src_row_stride * elem) % 16 == 0 &&
                in.in_dim % 8 == 0 && in.qdata_offset % 8 == 0;
+    all_bf16_fast = all_bf16_fast && out.fast && in.src_kind == FSH_SRC_BF16;
     tiles += tiles_r * tiles_c;
   }
   prm.total_tiles = tiles;
@@ -368,7 +380,11 @@ FSH_API int fsh_quantize_pack(const fsh_quant_chunk* chunks, int32_t nchunks, vo
   const int64_t grid = tiles + ceil_div(zero_total, kZeroChunk);
   if (grid == 0) return FSH_OK;
   if (grid > 0x7FFFFFFFLL) return fail(FSH_ENOTSUP, "fsh_quantize_pack: %lld workgroups exceed the grid limit", (long long)grid);
-  hipLaunchKernelGGL(quantize_pack_kernel, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), 0,
-                     static_cast<hipStream_t>(stream), prm);
+  if (all_bf16_fast)
+    hipLaunchKernelGGL(quantize_pack_kernel<true>, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), 0,
+                       static_cast<hipStream_t>(stream), prm);
+  else
+    hipLaunchKernelGGL(quantize_pack_kernel<false>, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), 0,
+                       static_cast<hipStream_t>(stream), prm);
   return check_launch("fsh_quantize_pack");
 }

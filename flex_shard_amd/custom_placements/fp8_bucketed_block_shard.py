@@ -176,8 +176,8 @@ class Fp8BucketedBlockShard(BlockwiseQuantBucketedBlockShard):
             raise NotImplementedError(f"the HIP quantizer quantizes bf16 or fp32 values, not {quant_dtype}")
         return table.get((tensor_dtype, quant_dtype))
 
-    def _launch_quantize_pack(self, specs, payload, zero_ranges) -> None:
-        hip_ops.quantize_pack(specs, payload, zero_ranges, self.block_size, self.eps_mode)
+    def _make_quantize_pack_launch(self, specs, payload_nbytes, zero_ranges, device) -> hip_ops.QuantPackPlan:
+        return hip_ops.QuantPackPlan(specs, payload_nbytes, zero_ranges, self.block_size, self.eps_mode, device=device)
 
     # --------------------------------------------- fused compaction + dequant
     def _unpack_table(

@@ -31,7 +31,7 @@ from ._native import (
 __all__ = [
     "DT_BF16", "DT_F32", "EPS_FP32", "EPS_INPUT_DTYPE", "REDUCE_POSTDIV", "REDUCE_POSTMUL",
     "REDUCE_PREMUL", "REDUCE_SUM", "SRC_BF16", "SRC_F32", "SRC_F32_AS_BF16",
-    "QuantChunkSpec", "accumulate_grad", "copy_segments", "gemm_nt", "muon_apply", "muon_prepare",
+    "QuantChunkSpec", "QuantPackPlan", "accumulate_grad", "copy_segments", "gemm_nt", "muon_apply", "muon_prepare",
     "newton_schulz", "newton_schulz_workspace_bytes", "pack_segments", "quantize_pack",
     "reduce_rows", "stream_ptr", "unpack_dequant", "zero_segments",
 ]
@@ -76,6 +76,71 @@ class QuantChunkSpec:
         self.src_kind = src_kind
 
 
+class QuantPackPlan:
+    """A validated, reusable launch of the fused quantize + pack kernel for
+    fixed source shards: the ``fsh_quant_chunk`` tables are built once, so a
+    steady-state launch is one C call.  The shards' data pointers are baked
+    into the tables: the caller launches a plan only while tensors of the same
+    shape live at those addresses (``keep_alive`` makes the plan hold them)."""
+
+    __slots__ = ("_tables", "_zero_ranges", "_block", "_eps_mode", "_payload_nbytes", "_device", "_keep")
+
+    def __init__(
+        self,
+        chunks: Sequence[QuantChunkSpec],
+        payload_nbytes: int,
+        zero_ranges: tuple[tuple[int, int], tuple[int, int]],
+        block: int,
+        eps_mode: int = EPS_INPUT_DTYPE,
+        device: torch.device | None = None,
+        keep_alive: bool = False,
+    ) -> None:
+        if chunks:
+            device = _require_gpu(*[c.tensor for c in chunks])
+        if device is None or device.type != "cuda":
+            raise RuntimeError("flex_shard_amd kernels run on the GPU only; there is no CPU path.")
+        self._device = device
+        self._keep = [c.tensor for c in chunks] if keep_alive else None
+        self._zero_ranges = zero_ranges
+        self._block, self._eps_mode, self._payload_nbytes = block, eps_mode, payload_nbytes
+        cap = _native.FSH_MAX_QUANT_CHUNKS
+        groups = [list(chunks[i : i + cap]) for i in range(0, len(chunks), cap)] or [[]]
+        self._tables = []
+        for group in groups:
+            table = (_native.QuantChunk * max(len(group), 1))()
+            for slot, spec in zip(table, group):
+                t = spec.tensor
+                if t.ndim != 2 or t.stride(1) != 1 or t.shape[0] <= 0 or t.shape[1] <= 0:
+                    raise ValueError(
+                        f"chunk must be a non-empty 2-D view with unit column stride, got {tuple(t.shape)} / {t.stride()}"
+                    )
+                expected = torch.bfloat16 if spec.src_kind == SRC_BF16 else torch.float32
+                if t.dtype != expected:
+                    raise ValueError(f"chunk dtype {t.dtype} does not match src_kind {spec.src_kind}")
+                slot.src_dev = t.data_ptr()
+                slot.rows, slot.in_dim = t.shape
+                slot.src_row_stride = t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+                slot.qdata_offset = spec.qdata_offset
+                slot.scale_offset = spec.scale_offset
+                slot.src_kind = spec.src_kind
+            self._tables.append((table, len(group)))
+
+    def launch(self, payload: torch.Tensor) -> None:
+        if payload.device != self._device or payload.dtype != torch.uint8 or payload.ndim != 1:
+            raise ValueError("payload must be a 1-D uint8 tensor on the plan's device")
+        if not payload.is_contiguous() or payload.numel() != self._payload_nbytes:
+            raise ValueError(f"payload must be contiguous with {self._payload_nbytes} bytes")
+        fn = _native.lib().fsh_quantize_pack
+        stream = stream_ptr(self._device)
+        ptr, nbytes = payload.data_ptr(), self._payload_nbytes
+        for index, (table, count) in enumerate(self._tables):
+            zr = self._zero_ranges if index == 0 else ((0, 0), (0, 0))
+            status = fn(table, count, ptr, nbytes, zr[0][0], zr[0][1], zr[1][0], zr[1][1], self._block,
+                        self._eps_mode, stream)
+            if status != 0:
+                _native.check(status, "fsh_quantize_pack")
+
+
 def quantize_pack(
     chunks: Sequence[QuantChunkSpec],
     payload: torch.Tensor,
@@ -86,34 +151,8 @@ def quantize_pack(
     """Fused tile quantize + pack of every chunk into ``payload`` (uint8,
     contiguous) and zeroing of the two pad ranges.  Launches are split when
     there are more than FSH_MAX_QUANT_CHUNKS chunks."""
-    _require_gpu(payload, *[c.tensor for c in chunks])
-    if payload.dtype != torch.uint8 or not payload.is_contiguous() or payload.ndim != 1:
-        raise ValueError("payload must be a contiguous 1-D uint8 tensor")
-    lib = _native.lib()
-    stream = stream_ptr(payload.device)
-    cap = _native.FSH_MAX_QUANT_CHUNKS
-    groups = [list(chunks[i : i + cap]) for i in range(0, len(chunks), cap)] or [[]]
-    for index, group in enumerate(groups):
-        table = (_native.QuantChunk * max(len(group), 1))()
-        for slot, spec in zip(table, group):
-            t = spec.tensor
-            if t.ndim != 2 or t.stride(1) != 1 or t.shape[0] <= 0 or t.shape[1] <= 0:
-                raise ValueError(f"chunk must be a non-empty 2-D view with unit column stride, got {tuple(t.shape)} / {t.stride()}")
-            expected = torch.bfloat16 if spec.src_kind == SRC_BF16 else torch.float32
-            if t.dtype != expected:
-                raise ValueError(f"chunk dtype {t.dtype} does not match src_kind {spec.src_kind}")
-            slot.src_dev = t.data_ptr()
-            slot.rows, slot.in_dim = t.shape
-            slot.src_row_stride = t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
-            slot.qdata_offset = spec.qdata_offset
-            slot.scale_offset = spec.scale_offset
-            slot.src_kind = spec.src_kind
-        zr = zero_ranges if index == 0 else ((0, 0), (0, 0))
-        status = lib.fsh_quantize_pack(
-            table, len(group), payload.data_ptr(), payload.numel(),
-            zr[0][0], zr[0][1], zr[1][0], zr[1][1], block, eps_mode, stream,
-        )
-        _native.check(status, "fsh_quantize_pack")
+    _require_gpu(payload)
+    QuantPackPlan(chunks, payload.numel(), zero_ranges, block, eps_mode, device=payload.device).launch(payload)
 
 
 def _check_i64_table(*tables: torch.Tensor) -> int:
