@@ -236,6 +236,21 @@ def bench_muon(device, reps=3):
             "frac_of_bf16_mfma_peak": flops / per / 1e9 / BF16_MFMA_PEAK_TFLOPS}
 
 
+def calibrate_copy(device, nbytes: int = 256 << 20, reps: int = 4) -> None:
+    """A plain copy of known size through copy_segments_kernel: reads `nbytes`
+    and writes `nbytes` per launch."""
+    from flex_shard_amd.custom_placements._copy_kernels import SegmentCopyDescriptor, copy_segments
+
+    src = torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=device)
+    dst = torch.empty_like(src)
+    desc = SegmentCopyDescriptor.create(src_offsets=[0], numels=[nbytes // 4], dst_offsets=[0], device=device)
+    for _ in range(reps):
+        copy_segments(src.view(torch.int32), dst.view(torch.int32), desc)
+    torch.cuda.synchronize()
+    if not torch.equal(src, dst):
+        raise SystemExit("bench: calibration copy produced wrong bytes")
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -244,6 +259,9 @@ def main() -> None:
     ap.add_argument("--layers", type=int, default=8, help="distinct layer buckets the steps rotate over")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-secondary", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB -> 256 MiB segment copy, the known-size kernel that the "
+                    "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit(
@@ -258,6 +276,8 @@ def main() -> None:
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
+    if args.calibrate_copy:
+        calibrate_copy(device)
     q = bench_quant_pack(device, args.steps, args.warmup, args.layers)
     placement, infos, work, metadata, payloads = q.pop("work")
     check_against_oracle(placement, infos, work, metadata, payloads)

@@ -12,12 +12,16 @@
 // A tall input is its own X^T, so no transpose kernel is needed in either
 // case, and the result lands in the caller's buffer without a copy.
 //
-// GEMM kernel: 256 threads (2x2 wavefronts), 128x128 block tile, BK = 32,
-// v_mfma_f32_32x32x16_bf16, each wave a 64x64 tile (2x2 MFMA tiles, 64 fp32
-// accumulators per lane).  Global->register->LDS double buffering with one
-// barrier per k-tile; LDS rows padded by 16 bytes so the 64 lanes of a
-// ds_read_b128 hit distinct banks.
+// GEMM kernels: 256 threads (2x2 wavefronts) on v_mfma_f32_32x32x16_bf16, in
+// two tile configurations (256x256x64 for large problems, 128x128x32 when
+// there are too few tiles to fill the chip) and two bodies: a predicated one
+// for any shape, and a predicate-free, software-pipelined one for problems
+// whose dimensions are multiples of the tile.  Global->register->LDS double
+// buffering with one barrier per k-tile; LDS rows padded by 16 bytes so the
+// 64 lanes of a ds_read_b128 hit distinct banks.
 #include "common.hpp"
+
+#include <type_traits>
 
 namespace fsh {
 namespace {
@@ -38,22 +42,48 @@ struct GemmParams {
   int32_t tiles_m, tiles_n;
 };
 
-constexpr int BM = 128, BN = 128, BK = 32;
-constexpr int kGemmThreads = 256;
-constexpr int kLdsStride = BK + 8;  // bf16 elements per LDS row (80 bytes)
+// Tile configuration of one GEMM kernel instantiation.
+//   BM x BN block tile, BK k-tile, WM x WN wavefronts, each wave owns a
+//   (BM/WM) x (BN/WN) sub-tile made of 32x32 MFMA tiles.
+template <int BM_, int BN_, int BK_, int WM_, int WN_>
+struct GemmCfg {
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
+  static constexpr int kThreads = WM * WN * 64;
+  static constexpr int kWaveM = BM / WM, kWaveN = BN / WN;
+  static constexpr int TM = kWaveM / 32, TN = kWaveN / 32;
+  static constexpr int kLdsStride = BK + 8;  // bf16 per LDS row: 16 bytes of padding
+  static constexpr int kStageElems = (BM + BN) * kLdsStride;
+  static constexpr int kLdsBytes = 2 * kStageElems * 2;  // double buffered
+  static constexpr int kChunksPerRow = BK / 8;
+  static constexpr int kChunksA = BM * kChunksPerRow / kThreads;
+  static constexpr int kChunksB = BN * kChunksPerRow / kThreads;
+  static_assert(BM * kChunksPerRow % kThreads == 0 && BN * kChunksPerRow % kThreads == 0, "chunk split");
+};
 
-__global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(const GemmParams p) {
-  __shared__ __attribute__((aligned(16))) uint16_t smem[2][(BM + BN) * kLdsStride];
+// Large problems: 256x256x64, four waves of 128x128 (256 fp32 accumulators per
+// lane).  Per 16-wide k step a wave issues 8 ds_read_b128 for 16 MFMAs, so LDS
+// traffic is half of what 64x64 wave tiles need, and a k-tile lasts ~2000
+// cycles, long enough for the next tile's global loads to land.
+using BigCfg = GemmCfg<256, 256, 64, 2, 2>;
+// Small problems (few tiles): 128x128x32, four waves of 64x64.
+using SmallCfg = GemmCfg<128, 128, 32, 2, 2>;
+
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::kThreads) void gemm_nt_kernel(const GemmParams p) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, TM = Cfg::TM, TN = Cfg::TN;
+  constexpr int kLdsStride = Cfg::kLdsStride;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
   const int64_t batch = blockIdx.y;
 
-  // Tiles are numbered so that the 8 workgroups that land on one XCD in a row
-  // (round-robin dispatch) walk down one column block: they share the B
-  // operand rows in that XCD's L2.
+  // Consecutive workgroup ids go round-robin to the 8 XCDs.  With tm the fast
+  // index and tiles_m a multiple of 8, every workgroup of one XCD works on
+  // A row-blocks {x, x+8, ...}: those stay in that XCD's L2 while the B
+  // row-blocks stream through.
   const int tile = blockIdx.x;
   const int tm = tile % p.tiles_m;
   const int tn = tile / p.tiles_m;
@@ -63,42 +93,47 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(const GemmParams 
   const uint16_t* A = p.A + batch * p.sA;
   const uint16_t* B = p.B + batch * p.sB;
 
-  // Global -> register staging: 16-byte chunks, 4 per LDS row.
-  constexpr int kChunksPerRow = BK / 8;
-  constexpr int kChunks = BM * kChunksPerRow / kGemmThreads;  // 2 (BM == BN)
-  u32x4 ra[kChunks], rb[kChunks];
-  int lrow[kChunks], lkc[kChunks];
-#pragma unroll
-  for (int i = 0; i < kChunks; ++i) {
-    const int c = tid + i * kGemmThreads;
-    lrow[i] = c / kChunksPerRow;
-    lkc[i] = c % kChunksPerRow;
-  }
-
+  // Global -> register staging in 16-byte chunks.
+  u32x4 ra[Cfg::kChunksA], rb[Cfg::kChunksB];
   auto load_global = [&](int64_t k0) {
 #pragma unroll
-    for (int i = 0; i < kChunks; ++i) {
-      const int64_t gk = k0 + lkc[i] * 8;
-      const int64_t ar = m0 + lrow[i], br = n0 + lrow[i];
+    for (int i = 0; i < Cfg::kChunksA; ++i) {
+      const int c = tid + i * Cfg::kThreads;
+      const int64_t row = m0 + c / Cfg::kChunksPerRow, gk = k0 + (c % Cfg::kChunksPerRow) * 8;
       ra[i] = u32x4{0, 0, 0, 0};
+      if (row < p.M && gk < p.K) ra[i] = *reinterpret_cast<const u32x4*>(A + row * p.lda + gk);
+    }
+#pragma unroll
+    for (int i = 0; i < Cfg::kChunksB; ++i) {
+      const int c = tid + i * Cfg::kThreads;
+      const int64_t row = n0 + c / Cfg::kChunksPerRow, gk = k0 + (c % Cfg::kChunksPerRow) * 8;
       rb[i] = u32x4{0, 0, 0, 0};
-      if (ar < p.M && gk < p.K) ra[i] = *reinterpret_cast<const u32x4*>(A + ar * p.lda + gk);
-      if (br < p.N && gk < p.K) rb[i] = *reinterpret_cast<const u32x4*>(B + br * p.ldb + gk);
+      if (row < p.N && gk < p.K) rb[i] = *reinterpret_cast<const u32x4*>(B + row * p.ldb + gk);
     }
   };
   auto store_lds = [&](int buf) {
+    uint16_t* base = smem + buf * Cfg::kStageElems;
 #pragma unroll
-    for (int i = 0; i < kChunks; ++i) {
-      *reinterpret_cast<u32x4*>(&smem[buf][lrow[i] * kLdsStride + lkc[i] * 8]) = ra[i];
-      *reinterpret_cast<u32x4*>(&smem[buf][(BM + lrow[i]) * kLdsStride + lkc[i] * 8]) = rb[i];
+    for (int i = 0; i < Cfg::kChunksA; ++i) {
+      const int c = tid + i * Cfg::kThreads;
+      *reinterpret_cast<u32x4*>(&base[(c / Cfg::kChunksPerRow) * kLdsStride + (c % Cfg::kChunksPerRow) * 8]) = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < Cfg::kChunksB; ++i) {
+      const int c = tid + i * Cfg::kThreads;
+      *reinterpret_cast<u32x4*>(&base[(BM + c / Cfg::kChunksPerRow) * kLdsStride + (c % Cfg::kChunksPerRow) * 8]) = rb[i];
     }
   };
 
-  f32x16 acc[2][2];
+  // acc[i][j] accumulates (B sub-tile j) x (A sub-tile i)^T, i.e. the
+  // transposed 32x32 block: a lane then owns one output row (m) and runs of
+  // four consecutive columns (n), which makes the epilogue's C stores 8 bytes
+  // wide.
+  f32x16 acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
@@ -113,62 +148,295 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(const GemmParams 
   for (int64_t kt = 0; kt < ktiles; ++kt) {
     const int buf = static_cast<int>(kt & 1);
     if (kt + 1 < ktiles) load_global((kt + 1) * BK);
-    const uint16_t* As = &smem[buf][0];
-    const uint16_t* Bs = &smem[buf][BM * kLdsStride];
+    const uint16_t* As = smem + buf * Cfg::kStageElems;
+    const uint16_t* Bs = As + BM * kLdsStride;
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
-      bf16x8 af[2], bf[2];
+      bf16x8 af[TM], bf[TN];
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
-        af[i] = *reinterpret_cast<const bf16x8*>(&As[(wm * 64 + i * 32 + frag_row) * kLdsStride + ks * 16 + frag_k]);
+      for (int i = 0; i < TM; ++i)
+        af[i] = *reinterpret_cast<const bf16x8*>(
+            &As[(wm * Cfg::kWaveM + i * 32 + frag_row) * kLdsStride + ks * 16 + frag_k]);
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-        bf[j] = *reinterpret_cast<const bf16x8*>(&Bs[(wn * 64 + j * 32 + frag_row) * kLdsStride + ks * 16 + frag_k]);
+      for (int j = 0; j < TN; ++j)
+        bf[j] = *reinterpret_cast<const bf16x8*>(
+            &Bs[(wn * Cfg::kWaveN + j * 32 + frag_row) * kLdsStride + ks * 16 + frag_k]);
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[j], af[i], acc[i][j], 0, 0, 0);
     }
     if (kt + 1 < ktiles) store_lds(buf ^ 1);
     __syncthreads();
   }
 
-  // Epilogue.  Accumulator r of a 32x32 MFMA tile belongs to column lane%32
-  // and row 8*(r/4) + 4*(lane/32) + r%4.
+  // Epilogue.  Accumulator r of block (i, j) belongs to output row
+  // m = lane%32 and column n = 8*(r/4) + 4*(lane/32) + r%4 of the block.
+  const uint16_t* D = p.D ? p.D + batch * p.sD : nullptr;
+  uint16_t* C = p.C + batch * p.sC;
+  uint16_t* Ct = p.Ct ? p.Ct + batch * p.sCt : nullptr;
+  const bool c_vec = (p.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7) == 0);
+  const bool d_vec = D != nullptr && (p.ldd % 4 == 0) && ((reinterpret_cast<uintptr_t>(D) & 7) == 0);
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int64_t row = m0 + wm * Cfg::kWaveM + i * 32 + (lane & 31);
+    if (row >= p.M) continue;
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int64_t col = n0 + wn * Cfg::kWaveN + j * 32 + 8 * b + 4 * (lane >> 5);
+        if (col >= p.N) continue;
+        const bool full = col + 3 < p.N;
+        float dv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (D != nullptr) {
+          if (full && d_vec) {
+            const u32x2 raw = *reinterpret_cast<const u32x2*>(&D[row * p.ldd + col]);
+            dv[0] = u32_as_f32(raw.x << 16);
+            dv[1] = u32_as_f32(raw.x & 0xFFFF0000u);
+            dv[2] = u32_as_f32(raw.y << 16);
+            dv[3] = u32_as_f32(raw.y & 0xFFFF0000u);
+          } else {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+              if (col + t < p.N) dv[t] = bf16_bits_to_f32(D[row * p.ldd + col + t]);
+          }
+        }
+        uint32_t packed[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          float v = p.alpha * acc[i][j][4 * b + t];
+          if (D != nullptr) v += p.beta * dv[t];
+          packed[t] = f32_to_bf16_bits(v);
+        }
+        if (full && c_vec) {
+          *reinterpret_cast<u32x2*>(&C[row * p.ldc + col]) =
+              u32x2{packed[0] | (packed[1] << 16), packed[2] | (packed[3] << 16)};
+        } else {
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            if (col + t < p.N) C[row * p.ldc + col + t] = static_cast<uint16_t>(packed[t]);
+        }
+        if (Ct != nullptr) {
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            if (col + t < p.N) Ct[(col + t) * p.ldct + row] = static_cast<uint16_t>(packed[t]);
+        }
+      }
+  }
+}
+
+// Scheduling-group masks of __builtin_amdgcn_sched_group_barrier.
+constexpr int kSchedMfma = 0x008, kSchedVmemRead = 0x020, kSchedDsRead = 0x100, kSchedDsWrite = 0x200;
+
+// Interior fast path: M, N multiples of the block tile and K of BK, so there
+// are no predicates, addresses are one per-thread 32-bit offset plus uniform
+// terms, and the k loop is software pipelined by hand.  With 256 accumulators
+// a SIMD holds a single wave, so nothing else hides latency: the fragments of
+// k step s+1 are read from LDS while the MFMAs of step s issue, the next
+// tile's global loads are spread over the first k step, and their LDS writes
+// are interleaved with the MFMAs of the last one.
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::kThreads) void gemm_nt_interior_kernel(const GemmParams p) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, TM = Cfg::TM, TN = Cfg::TN;
+  constexpr int kLdsStride = Cfg::kLdsStride, KS = BK / 16, CPR = Cfg::kChunksPerRow;
+  constexpr int kRowsPerPass = Cfg::kThreads / CPR;  // tile rows covered by one chunk pass
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+  const int64_t batch = blockIdx.y;
+  const int tile = blockIdx.x;
+  const int tm = tile % p.tiles_m;
+  const int tn = tile / p.tiles_m;
+  const int64_t m0 = static_cast<int64_t>(tm) * BM;
+  const int64_t n0 = static_cast<int64_t>(tn) * BN;
+
+  // Uniform tile bases and one per-thread byte offset each for A and B.
+  const uint8_t* Ab = reinterpret_cast<const uint8_t*>(p.A + batch * p.sA + m0 * p.lda);
+  const uint8_t* Bb = reinterpret_cast<const uint8_t*>(p.B + batch * p.sB + n0 * p.ldb);
+  const int trow = tid / CPR, tkc = tid % CPR;
+  const uint32_t a_toff = static_cast<uint32_t>((trow * p.lda + tkc * 8) * 2);
+  const uint32_t b_toff = static_cast<uint32_t>((trow * p.ldb + tkc * 8) * 2);
+  const int64_t a_pass = static_cast<int64_t>(kRowsPerPass) * p.lda * 2;
+  const int64_t b_pass = static_cast<int64_t>(kRowsPerPass) * p.ldb * 2;
+  const int lds_toff = trow * kLdsStride + tkc * 8;  // elements
+
+  u32x4 ra[Cfg::kChunksA], rb[Cfg::kChunksB];
+  auto load_global = [&](int64_t kt) {
+    const int64_t koff = kt * BK * 2;
+#pragma unroll
+    for (int i = 0; i < Cfg::kChunksA; ++i)
+      ra[i] = *reinterpret_cast<const u32x4*>(Ab + (koff + i * a_pass) + a_toff);
+#pragma unroll
+    for (int i = 0; i < Cfg::kChunksB; ++i)
+      rb[i] = *reinterpret_cast<const u32x4*>(Bb + (koff + i * b_pass) + b_toff);
+  };
+  auto store_lds = [&](int buf) {
+    uint16_t* base = smem + buf * Cfg::kStageElems + lds_toff;
+#pragma unroll
+    for (int i = 0; i < Cfg::kChunksA; ++i)
+      *reinterpret_cast<u32x4*>(&base[i * kRowsPerPass * kLdsStride]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < Cfg::kChunksB; ++i)
+      *reinterpret_cast<u32x4*>(&base[(BM + i * kRowsPerPass) * kLdsStride]) = rb[i];
+  };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  const int a_frag = (wm * Cfg::kWaveM + (lane & 31)) * kLdsStride + (lane >> 5) * 8;
+  const int b_frag = (BM + wn * Cfg::kWaveN + (lane & 31)) * kLdsStride + (lane >> 5) * 8;
+  bf16x8 af[2][TM], bf[2][TN];
+  auto load_frags = [&](int set, const uint16_t* stage, int ks) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      af[set][i] = *reinterpret_cast<const bf16x8*>(&stage[a_frag + i * 32 * kLdsStride + ks * 16]);
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      bf[set][j] = *reinterpret_cast<const bf16x8*>(&stage[b_frag + j * 32 * kLdsStride + ks * 16]);
+  };
+  auto mfma_step = [&](int set) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[set][j], af[set][i], acc[i][j], 0, 0, 0);
+  };
+
+  const int64_t ktiles = p.K / BK;
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+  load_frags(0, smem, 0);
+
+  constexpr int kMfmaPerStep = TM * TN;
+  constexpr int kFragReads = TM + TN;
+  constexpr int kGlobalLoads = Cfg::kChunksA + Cfg::kChunksB;
+  // One k-tile.  `more` (a compile-time tag) says whether a next tile exists:
+  // the last tile is peeled so that each variant is straight-line code the
+  // scheduling hints can reorder freely.
+  auto k_tile = [&](int64_t kt, auto more_tag) {
+    constexpr bool more = decltype(more_tag)::value;
+    const int buf = static_cast<int>(kt & 1);
+    const uint16_t* stage = smem + buf * Cfg::kStageElems;
+    if (more) load_global(kt + 1);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks + 1 < KS) load_frags((ks + 1) & 1, stage, ks + 1);
+      if (ks == KS - 1 && more) store_lds(buf ^ 1);
+      mfma_step(ks & 1);
+      if (ks == 0 && more) {
+#pragma unroll
+        for (int g = 0; g < kGlobalLoads; ++g) {
+          __builtin_amdgcn_sched_group_barrier(kSchedVmemRead, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+          if (g < kFragReads) __builtin_amdgcn_sched_group_barrier(kSchedDsRead, 1, 0);
+        }
+      } else if (ks + 1 < KS) {
+#pragma unroll
+        for (int g = 0; g < kFragReads; ++g) {
+          __builtin_amdgcn_sched_group_barrier(kSchedDsRead, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(kSchedMfma, kMfmaPerStep / kFragReads, 0);
+        }
+      } else if (more) {
+#pragma unroll
+        for (int g = 0; g < kGlobalLoads; ++g) {
+          __builtin_amdgcn_sched_group_barrier(kSchedDsWrite, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+        }
+      }
+    }
+    __syncthreads();
+    if (more) load_frags(0, smem + (buf ^ 1) * Cfg::kStageElems, 0);
+  };
+  for (int64_t kt = 0; kt + 1 < ktiles; ++kt) k_tile(kt, std::true_type{});
+  k_tile(ktiles - 1, std::false_type{});
+
+  // Epilogue.  Accumulator r of block (i, j) belongs to output row
+  // m = lane%32 and column n = 8*(r/4) + 4*(lane/32) + r%4 of the block.
   const uint16_t* D = p.D ? p.D + batch * p.sD : nullptr;
   uint16_t* C = p.C + batch * p.sC;
   uint16_t* Ct = p.Ct ? p.Ct + batch * p.sCt : nullptr;
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TM; ++i) {
+    const int64_t row = m0 + wm * Cfg::kWaveM + i * 32 + (lane & 31);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int64_t col = n0 + wn * 64 + j * 32 + (lane & 31);
-      if (col >= p.N) continue;
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
-        const int64_t row_base = m0 + wm * 64 + i * 32 + 8 * b + 4 * (lane >> 5);
+        const int64_t col = n0 + wn * Cfg::kWaveN + j * 32 + 8 * b + 4 * (lane >> 5);
+        float dv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (D != nullptr) {
+          const u32x2 raw = *reinterpret_cast<const u32x2*>(&D[row * p.ldd + col]);
+          dv[0] = u32_as_f32(raw.x << 16);
+          dv[1] = u32_as_f32(raw.x & 0xFFFF0000u);
+          dv[2] = u32_as_f32(raw.y << 16);
+          dv[3] = u32_as_f32(raw.y & 0xFFFF0000u);
+        }
         uint32_t packed[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          const int64_t row = row_base + t;
           float v = p.alpha * acc[i][j][4 * b + t];
-          if (D != nullptr && row < p.M) v += p.beta * bf16_bits_to_f32(D[row * p.ldd + col]);
+          if (D != nullptr) v += p.beta * dv[t];
           packed[t] = f32_to_bf16_bits(v);
-          if (row < p.M) C[row * p.ldc + col] = static_cast<uint16_t>(packed[t]);
         }
+        *reinterpret_cast<u32x2*>(&C[row * p.ldc + col]) =
+            u32x2{packed[0] | (packed[1] << 16), packed[2] | (packed[3] << 16)};
         if (Ct != nullptr) {
-          if (row_base + 3 < p.M) {
-            *reinterpret_cast<u32x2*>(&Ct[col * p.ldct + row_base]) =
-                u32x2{packed[0] | (packed[1] << 16), packed[2] | (packed[3] << 16)};
-          } else {
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
-              if (row_base + t < p.M) Ct[col * p.ldct + row_base + t] = static_cast<uint16_t>(packed[t]);
-          }
+          for (int t = 0; t < 4; ++t) Ct[(col + t) * p.ldct + row] = static_cast<uint16_t>(packed[t]);
         }
       }
+  }
+}
+
+template <typename Kernel>
+int reserve_lds(Kernel kernel, int bytes) {
+  if (bytes <= 64 * 1024) return FSH_OK;
+  hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (err != hipSuccess) return fail(FSH_EHIP, "gemm: cannot reserve %d bytes of LDS: %s", bytes, hipGetErrorString(err));
+  return FSH_OK;
+}
+
+template <typename Cfg>
+int launch_gemm_cfg(GemmParams& p, int64_t batch, hipStream_t stream) {
+  p.tiles_m = static_cast<int32_t>(ceil_div(p.M, Cfg::BM));
+  p.tiles_n = static_cast<int32_t>(ceil_div(p.N, Cfg::BN));
+  const int64_t tiles = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
+  if (tiles > 0x7FFFFFFFLL) return fail(FSH_ENOTSUP, "gemm: too many tiles");
+  const dim3 grid(static_cast<uint32_t>(tiles), static_cast<uint32_t>(batch)), block(Cfg::kThreads);
+  // Interior path: whole tiles, 8-byte friendly epilogue, 32-bit tile spans.
+  const bool interior =
+      p.M % Cfg::BM == 0 && p.N % Cfg::BN == 0 && p.K % Cfg::BK == 0 && p.ldc % 4 == 0 &&
+      (reinterpret_cast<uintptr_t>(p.C) & 7) == 0 && p.sC % 4 == 0 &&
+      (p.D == nullptr || (p.ldd % 4 == 0 && (reinterpret_cast<uintptr_t>(p.D) & 7) == 0 && p.sD % 4 == 0)) &&
+      static_cast<int64_t>(Cfg::BM) * p.lda * 2 < (1LL << 31) && static_cast<int64_t>(Cfg::BN) * p.ldb * 2 < (1LL << 31);
+  if (interior) {
+    static bool reserved = false;  // the attribute is per device function and sticky
+    if (!reserved) {
+      if (int rc = reserve_lds(&gemm_nt_interior_kernel<Cfg>, Cfg::kLdsBytes)) return rc;
+      reserved = true;
     }
+    hipLaunchKernelGGL(gemm_nt_interior_kernel<Cfg>, grid, block, Cfg::kLdsBytes, stream, p);
+    return check_launch("gemm_nt_interior_kernel");
+  }
+  static bool reserved_edge = false;
+  if (!reserved_edge) {
+    if (int rc = reserve_lds(&gemm_nt_kernel<Cfg>, Cfg::kLdsBytes)) return rc;
+    reserved_edge = true;
+  }
+  hipLaunchKernelGGL(gemm_nt_kernel<Cfg>, grid, block, Cfg::kLdsBytes, stream, p);
+  return check_launch("gemm_nt_kernel");
 }
 
 int launch_gemm(const fsh_gemm_desc& d, hipStream_t stream) {
@@ -181,8 +449,6 @@ int launch_gemm(const fsh_gemm_desc& d, hipStream_t stream) {
     return fail(FSH_ENOTSUP, "gemm: k, lda, ldb and batch strides must be multiples of 8 and A, B 16-byte aligned");
   if (d.lda < d.k || d.ldb < d.k || d.ldc < d.n || (d.d_dev && d.ldd < d.n) || (d.ct_dev && d.ldct < d.m))
     return fail(FSH_EINVAL, "gemm: leading dimension smaller than the row length");
-  if (d.ct_dev && (d.ldct % 4 || d.stride_ct % 4 || !aligned(d.ct_dev, 8)))
-    return fail(FSH_ENOTSUP, "gemm: transposed output needs ldct %% 4 == 0 and an 8-byte aligned pointer");
   if (d.batch > 65535) return fail(FSH_ENOTSUP, "gemm: batch %lld exceeds 65535", (long long)d.batch);
   GemmParams p;
   p.A = static_cast<const uint16_t*>(d.a_dev);
@@ -194,13 +460,10 @@ int launch_gemm(const fsh_gemm_desc& d, hipStream_t stream) {
   p.lda = d.lda; p.ldb = d.ldb; p.ldd = d.ldd; p.ldc = d.ldc; p.ldct = d.ldct;
   p.sA = d.stride_a; p.sB = d.stride_b; p.sD = d.stride_d; p.sC = d.stride_c; p.sCt = d.stride_ct;
   p.alpha = d.alpha; p.beta = d.beta;
-  p.tiles_m = static_cast<int32_t>(ceil_div(d.m, BM));
-  p.tiles_n = static_cast<int32_t>(ceil_div(d.n, BN));
-  const int64_t tiles = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
-  if (tiles > 0x7FFFFFFFLL) return fail(FSH_ENOTSUP, "gemm: too many tiles");
-  hipLaunchKernelGGL(gemm_nt_kernel, dim3(static_cast<uint32_t>(tiles), static_cast<uint32_t>(d.batch)),
-                     dim3(kGemmThreads), 0, stream, p);
-  return check_launch("gemm_nt_kernel");
+  // The big tile pays off once it fills the chip at least once.
+  const int64_t big_tiles = ceil_div(d.m, BigCfg::BM) * ceil_div(d.n, BigCfg::BN) * d.batch;
+  if (big_tiles >= 192) return launch_gemm_cfg<BigCfg>(p, d.batch, stream);
+  return launch_gemm_cfg<SmallCfg>(p, d.batch, stream);
 }
 
 // ------------------------------------------------------- Frobenius normalize
