@@ -33,6 +33,13 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor figure
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
+# HBM bytes per launch of quantize_pack_kernel on the default workload, from
+# two counter runs (FETCH_SIZE, then WRITE_SIZE) of this script, each scaled by
+# the same counter's reading for the 256 MiB --calibrate-copy kernel:
+# 26 669.0 KiB x 1.9937 read + 26 932.2 KiB x 1.0 written.  Counters cannot be
+# read inside a timed run, so the figure is carried here and only reported
+# for the workload it was measured on.
+PROFILED_TRAFFIC_BYTES = {(27262976, 27531840): 82_024_000}
 
 
 def _factory(fp8_data, recip_scale, block_size, *, orig_dtype, requires_grad):
@@ -313,7 +320,7 @@ def main() -> None:
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": PROFILED_TRAFFIC_BYTES.get((q["elems"], q["payload_nbytes"])),
             "algorithmic_bytes_per_launch": q["algo_bytes"],
             "avg_launch_us": round(kernel_ms * 1e3, 2),
             "avg_launch_us_hot_cache": round(q["hot_event_ms"] / args.steps * 1e3, 2),
