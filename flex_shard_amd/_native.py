@@ -80,6 +80,8 @@ class GemmDesc(Structure):
         ("stride_ct", c_int64),
         ("alpha", c_float),
         ("beta", c_float),
+        ("symmetric", c_int32),
+        ("reserved", c_int32),
     ]
 
 

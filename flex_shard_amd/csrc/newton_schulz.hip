@@ -40,7 +40,51 @@ struct GemmParams {
   int64_t sA, sB, sD, sC, sCt;
   float alpha, beta;
   int32_t tiles_m, tiles_n;
+  int32_t symmetric;      // only tiles with tm <= tn are computed; the others are mirrored
+  int32_t tiles_per_matrix;
+  int64_t work_items;     // tiles_per_matrix * batch
+  int64_t items_per_xcd;  // ceil(work_items / 8); the grid has 8 * items_per_xcd workgroups
 };
+
+constexpr int kXcds = 8;         // accelerator dies, each with its own L2
+constexpr int kGroupTilesM = 4;  // tile rows walked together
+
+// Workgroup id -> (batch, tile row, tile column).  Workgroups are handed to
+// the 8 XCDs round-robin by id, and an XCD holds 32 of the large-tile
+// workgroups at a time (one per CU), so XCD x is given the contiguous run
+// [x, x+1) * items_per_xcd of an ordering in which 32 neighbours form a 4 x 8
+// patch of tiles of one matrix: its L2 then serves 12 distinct operand panels
+// per k-tile instead of 33.  Returns false for the padding ids at the end of
+// an XCD's run.
+__device__ inline bool tile_of_workgroup(const GemmParams& p, int64_t* batch, int* tm, int* tn) {
+  const int64_t id = blockIdx.x;
+  const int64_t slot = id / kXcds;
+  const int64_t item = (id % kXcds) * p.items_per_xcd + slot;
+  if (item >= p.work_items) return false;
+  const int tiles = p.tiles_per_matrix;
+  *batch = item / tiles;
+  int t = static_cast<int>(item % tiles);
+  if (p.symmetric) {
+    // Upper triangle row by row: row r holds columns r .. tiles_n-1.  One
+    // matrix's triangle (36 tiles of a 2048^2 result) is about what an XCD
+    // holds at a time, and it needs only the 8 row panels of the operand.
+    int r = 0;
+    for (int len = p.tiles_n; t >= len; --len) {
+      t -= len;
+      ++r;
+    }
+    *tm = r;
+    *tn = r + t;
+    return true;
+  }
+  const int group_span = kGroupTilesM * p.tiles_n;
+  const int first_m = (t / group_span) * kGroupTilesM;
+  const int rows = min(p.tiles_m - first_m, kGroupTilesM);
+  const int within = t % group_span;
+  *tm = first_m + within % rows;
+  *tn = within / rows;
+  return true;
+}
 
 // Tile configuration of one GEMM kernel instantiation.
 //   BM x BN block tile, BK k-tile, WM x WN wavefronts, each wave owns a
@@ -78,15 +122,9 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_nt_kernel(const GemmParams
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
-  const int64_t batch = blockIdx.y;
-
-  // Consecutive workgroup ids go round-robin to the 8 XCDs.  With tm the fast
-  // index and tiles_m a multiple of 8, every workgroup of one XCD works on
-  // A row-blocks {x, x+8, ...}: those stay in that XCD's L2 while the B
-  // row-blocks stream through.
-  const int tile = blockIdx.x;
-  const int tm = tile % p.tiles_m;
-  const int tn = tile / p.tiles_m;
+  int64_t batch;
+  int tm, tn;
+  if (!tile_of_workgroup(p, &batch, &tm, &tn)) return;  // whole workgroup, before any barrier
   const int64_t m0 = static_cast<int64_t>(tm) * BM;
   const int64_t n0 = static_cast<int64_t>(tn) * BN;
 
@@ -175,7 +213,10 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_nt_kernel(const GemmParams
   // m = lane%32 and column n = 8*(r/4) + 4*(lane/32) + r%4 of the block.
   const uint16_t* D = p.D ? p.D + batch * p.sD : nullptr;
   uint16_t* C = p.C + batch * p.sC;
-  uint16_t* Ct = p.Ct ? p.Ct + batch * p.sCt : nullptr;
+  // A symmetric product mirrors its off-diagonal tiles into the lower triangle.
+  const bool mirror = p.symmetric && tm != tn;
+  uint16_t* Ct = mirror ? C : (p.Ct ? p.Ct + batch * p.sCt : nullptr);
+  const int64_t ldct = mirror ? p.ldc : p.ldct;
   const bool c_vec = (p.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7) == 0);
   const bool d_vec = D != nullptr && (p.ldd % 4 == 0) && ((reinterpret_cast<uintptr_t>(D) & 7) == 0);
 #pragma unroll
@@ -221,7 +262,53 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_nt_kernel(const GemmParams
         if (Ct != nullptr) {
 #pragma unroll
           for (int t = 0; t < 4; ++t)
-            if (col + t < p.N) Ct[(col + t) * p.ldct + row] = static_cast<uint16_t>(packed[t]);
+            if (col + t < p.N) Ct[(col + t) * ldct + row] = static_cast<uint16_t>(packed[t]);
+        }
+      }
+  }
+}
+
+// Epilogue of the whole-tile kernels.  The accumulate is issued as
+// mfma(B, A), so accumulator r of block (i, j) belongs to output row
+// m = lane%32 and column n = 8*(r/4) + 4*(lane/32) + r%4 of the block: a lane
+// owns 4 consecutive columns and C leaves as 8-byte stores.
+template <typename Cfg>
+__device__ inline void store_whole_tile(const GemmParams& p, int64_t batch, int64_t m0, int64_t n0, int wm, int wn,
+                                        int lane, bool mirror, const f32x16 (&acc)[Cfg::TM][Cfg::TN]) {
+  constexpr int TM = Cfg::TM, TN = Cfg::TN;
+  const uint16_t* D = p.D ? p.D + batch * p.sD : nullptr;
+  uint16_t* C = p.C + batch * p.sC;
+  // A symmetric product mirrors its off-diagonal tiles into the lower triangle.
+  uint16_t* Ct = mirror ? C : (p.Ct ? p.Ct + batch * p.sCt : nullptr);
+  const int64_t ldct = mirror ? p.ldc : p.ldct;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int64_t row = m0 + wm * Cfg::kWaveM + i * 32 + (lane & 31);
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int64_t col = n0 + wn * Cfg::kWaveN + j * 32 + 8 * b + 4 * (lane >> 5);
+        float dv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (D != nullptr) {
+          const u32x2 raw = *reinterpret_cast<const u32x2*>(&D[row * p.ldd + col]);
+          dv[0] = u32_as_f32(raw.x << 16);
+          dv[1] = u32_as_f32(raw.x & 0xFFFF0000u);
+          dv[2] = u32_as_f32(raw.y << 16);
+          dv[3] = u32_as_f32(raw.y & 0xFFFF0000u);
+        }
+        uint32_t packed[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          float v = p.alpha * acc[i][j][4 * b + t];
+          if (D != nullptr) v += p.beta * dv[t];
+          packed[t] = f32_to_bf16_bits(v);
+        }
+        *reinterpret_cast<u32x2*>(&C[row * p.ldc + col]) =
+            u32x2{packed[0] | (packed[1] << 16), packed[2] | (packed[3] << 16)};
+        if (Ct != nullptr) {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) Ct[(col + t) * ldct + row] = static_cast<uint16_t>(packed[t]);
         }
       }
   }
@@ -248,10 +335,9 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_nt_interior_kernel(const G
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
-  const int64_t batch = blockIdx.y;
-  const int tile = blockIdx.x;
-  const int tm = tile % p.tiles_m;
-  const int tn = tile / p.tiles_m;
+  int64_t batch;
+  int tm, tn;
+  if (!tile_of_workgroup(p, &batch, &tm, &tn)) return;  // whole workgroup, before any barrier
   const int64_t m0 = static_cast<int64_t>(tm) * BM;
   const int64_t n0 = static_cast<int64_t>(tn) * BN;
 
@@ -361,42 +447,167 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_nt_interior_kernel(const G
   for (int64_t kt = 0; kt + 1 < ktiles; ++kt) k_tile(kt, std::true_type{});
   k_tile(ktiles - 1, std::false_type{});
 
-  // Epilogue.  Accumulator r of block (i, j) belongs to output row
-  // m = lane%32 and column n = 8*(r/4) + 4*(lane/32) + r%4 of the block.
-  const uint16_t* D = p.D ? p.D + batch * p.sD : nullptr;
-  uint16_t* C = p.C + batch * p.sC;
-  uint16_t* Ct = p.Ct ? p.Ct + batch * p.sCt : nullptr;
+  store_whole_tile<Cfg>(p, batch, m0, n0, wm, wn, lane, p.symmetric && tm != tn, acc);
+}
+
+// ---------------------------------------------------------------------------
+// Large whole-tile problems: 256x256x64 tiles with global->LDS loads.
+//
+// gfx950 can load 16 bytes per lane from global memory straight into LDS
+// (global_load_lds_dwordx4: lane l of a wave writes LDS bytes
+// [M0 + 16 l, M0 + 16 l + 16)), so a k-tile needs no staging registers and
+// no ds_write, and the loads of tile t+1 are waited for only at the end of
+// tile t.  A wave-level load fills 1 KB of LDS = 8 tile rows of 128 bytes
+// with no padding, so bank conflicts are avoided by an XOR swizzle instead:
+// the 16-byte chunk c of row r is stored in slot c ^ (r & 7) of its row, done
+// on the global side by letting the lane that fills slot s of row r fetch
+// chunk s ^ (r & 7).  Eight neighbouring lanes of a fragment read then hit
+// eight different slots.
+//
+// These loads and their waits are inline asm, which the compiler neither
+// reorders nor counts; everything else in the loop is compiler-visible and is
+// pinned around them with sched_barrier.
+//
+// The chip is power-limited in this kernel (the shader clock settles near
+// 1.2-1.4 GHz under sustained MFMA load), so what counts is data moved per
+// MFMA, not latency hiding: warming L2 with early touches of later k-tiles
+// was measured and bought nothing.
+struct DmaGemm {
+  static constexpr int BM = 256, BN = 256, BK = 64, WM = 2, WN = 2, TM = 4, TN = 4;
+  static constexpr int kThreads = 256, kWaveM = 128, kWaveN = 128, KS = BK / 16;
+  static constexpr int kRowBytes = BK * 2;                   // 128
+  static constexpr int kOperandBytes = BM * kRowBytes;       // 32 KB per operand and stage
+  static constexpr int kStageBytes = 2 * kOperandBytes;      // 64 KB
+  static constexpr int kLdsBytes = 2 * kStageBytes;
+  static constexpr int kLoadsPerOperand = BM / 8 / 4;        // wave-level 1 KB loads per wave: 8
+};
+
+__device__ inline void dma_load_16(uint32_t voffset, const uint8_t* base, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voffset), "s"(base), "s"(lds_addr) : "memory");
+}
+__device__ inline void wait_for_dma_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+__global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const GemmParams p) {
+  using Cfg = DmaGemm;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds_bytes[];
+  constexpr int TM = Cfg::TM, TN = Cfg::TN, KS = Cfg::KS;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+  int64_t batch;
+  int tm, tn;
+  if (!tile_of_workgroup(p, &batch, &tm, &tn)) return;  // whole workgroup, before any barrier
+  const int64_t m0 = static_cast<int64_t>(tm) * Cfg::BM;
+  const int64_t n0 = static_cast<int64_t>(tn) * Cfg::BN;
+  const uint8_t* Ab = reinterpret_cast<const uint8_t*>(p.A + batch * p.sA + m0 * p.lda);
+  const uint8_t* Bb = reinterpret_cast<const uint8_t*>(p.B + batch * p.sB + n0 * p.ldb);
+  const int64_t ktiles = p.K / Cfg::BK;
+
+  // Load side.  Wave-level load q (0..7) of this wave fills tile rows
+  // [32 q + 8 wave, +8); lane l fills slot l & 7 of row l >> 3 there.
+  const int fill_row = lane >> 3;
+  const int fill_chunk = (lane & 7) ^ fill_row;
+  uint32_t a_voff[Cfg::kLoadsPerOperand], b_voff[Cfg::kLoadsPerOperand];
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int64_t row = m0 + wm * Cfg::kWaveM + i * 32 + (lane & 31);
+  for (int q = 0; q < Cfg::kLoadsPerOperand; ++q) {
+    const int row = 32 * q + 8 * wave + fill_row;
+    a_voff[q] = static_cast<uint32_t>(row * p.lda * 2 + fill_chunk * 16);
+    b_voff[q] = static_cast<uint32_t>(row * p.ldb * 2 + fill_chunk * 16);
+  }
+  // M0 takes the LDS byte address relative to the workgroup's allocation.
+  typedef __attribute__((address_space(3))) uint8_t* lds_address;
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_address)lds_bytes));
+  const uint32_t fill_lds = lds_base + static_cast<uint32_t>(wave * 1024);  // + q * 4096 (+ operand, + stage)
+
+  // Fragment side.  Lane l reads row l & 31 of a 32-row block, k chunk
+  // 2 ks + (l >> 5); its slot is that chunk XOR (row & 7), i.e. the ks = 0
+  // address with bits 5..6 flipped by ks.
+  const int frag_row = lane & 31;
+  const uint32_t frag_base = static_cast<uint32_t>(frag_row * Cfg::kRowBytes + (((lane >> 5) ^ (frag_row & 7)) * 16));
+  uint32_t a_frag[KS], b_frag[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    a_frag[ks] = (frag_base ^ (ks * 32)) + wm * Cfg::kWaveM * Cfg::kRowBytes;
+    b_frag[ks] = (frag_base ^ (ks * 32)) + Cfg::kOperandBytes + wn * Cfg::kWaveN * Cfg::kRowBytes;
+  }
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const int64_t col = n0 + wn * Cfg::kWaveN + j * 32 + 8 * b + 4 * (lane >> 5);
-        float dv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (D != nullptr) {
-          const u32x2 raw = *reinterpret_cast<const u32x2*>(&D[row * p.ldd + col]);
-          dv[0] = u32_as_f32(raw.x << 16);
-          dv[1] = u32_as_f32(raw.x & 0xFFFF0000u);
-          dv[2] = u32_as_f32(raw.y << 16);
-          dv[3] = u32_as_f32(raw.y & 0xFFFF0000u);
-        }
-        uint32_t packed[4];
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  bf16x8 af[2][TM], bf[2][TN];
+  auto read_a = [&](int set, int stage_off, int ks, int i) {
+    af[set][i] = *reinterpret_cast<const bf16x8*>(lds_bytes + stage_off + a_frag[ks] + i * 32 * Cfg::kRowBytes);
+  };
+  auto read_b = [&](int set, int stage_off, int ks, int j) {
+    bf[set][j] = *reinterpret_cast<const bf16x8*>(lds_bytes + stage_off + b_frag[ks] + j * 32 * Cfg::kRowBytes);
+  };
+  auto read_frags = [&](int set, int stage_off, int ks) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          float v = p.alpha * acc[i][j][4 * b + t];
-          if (D != nullptr) v += p.beta * dv[t];
-          packed[t] = f32_to_bf16_bits(v);
-        }
-        *reinterpret_cast<u32x2*>(&C[row * p.ldc + col]) =
-            u32x2{packed[0] | (packed[1] << 16), packed[2] | (packed[3] << 16)};
-        if (Ct != nullptr) {
+    for (int i = 0; i < TM; ++i) read_a(set, stage_off, ks, i);
 #pragma unroll
-          for (int t = 0; t < 4; ++t) Ct[(col + t) * p.ldct + row] = static_cast<uint16_t>(packed[t]);
+    for (int j = 0; j < TN; ++j) read_b(set, stage_off, ks, j);
+  };
+  auto mfma = [&](int set, int i, int j) {
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[set][j], af[set][i], acc[i][j], 0, 0, 0);
+  };
+  auto issue_tile_load = [&](int64_t kt, int stage_off, int q_first, int q_last) {
+    const uint8_t* a_src = Ab + kt * Cfg::kRowBytes;
+    const uint8_t* b_src = Bb + kt * Cfg::kRowBytes;
+#pragma unroll
+    for (int q = q_first; q < q_last; ++q) {
+      dma_load_16(a_voff[q], a_src, stage_off + fill_lds + q * 4096);
+      dma_load_16(b_voff[q], b_src, stage_off + Cfg::kOperandBytes + fill_lds + q * 4096);
+    }
+  };
+
+  issue_tile_load(0, 0, 0, Cfg::kLoadsPerOperand);
+  wait_for_dma_loads();
+  __syncthreads();
+  read_frags(0, 0, 0);
+
+  auto k_tile = [&](int64_t kt, auto more_tag) {
+    constexpr bool more = decltype(more_tag)::value;
+    const int stage_off = static_cast<int>(kt & 1) * Cfg::kStageBytes;
+    const int next_off = stage_off ^ Cfg::kStageBytes;
+    // k step 0: one MFMA, one pair of loads of the next tile, one fragment
+    // read of k step 1 at a time.  The other stage is free: every wave passed
+    // the barrier that ended the previous tile after its last read of it.
+#pragma unroll
+    for (int g = 0; g < TM * TN; ++g) {
+      mfma(0, g / TN, g % TN);
+      if (more && g % 2 == 0) issue_tile_load(kt + 1, next_off, g / 2, g / 2 + 1);
+      if (g < TM) read_a(1, stage_off, 1, g);
+      else if (g < TM + TN) read_b(1, stage_off, 1, g - TM);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int ks = 1; ks < KS; ++ks) {
+      if (ks + 1 < KS) read_frags((ks + 1) & 1, stage_off, ks + 1);
+#pragma unroll
+      for (int g = 0; g < TM * TN; ++g) mfma(ks & 1, g / TN, g % TN);
+      if (ks + 1 < KS) {
+#pragma unroll
+        for (int g = 0; g < TM + TN; ++g) {
+          __builtin_amdgcn_sched_group_barrier(kSchedDsRead, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(kSchedMfma, TM * TN / (TM + TN), 0);
         }
       }
-  }
+    }
+    if (more) wait_for_dma_loads();  // this wave's part of the next tile has landed
+    __syncthreads();
+    if (more) read_frags(0, next_off, 0);
+  };
+  for (int64_t kt = 0; kt + 1 < ktiles; ++kt) k_tile(kt, std::true_type{});
+  k_tile(ktiles - 1, std::false_type{});
+
+  store_whole_tile<Cfg>(p, batch, m0, n0, wm, wn, lane, p.symmetric && tm != tn, acc);
 }
 
 template <typename Kernel>
@@ -412,17 +623,31 @@ template <typename Cfg>
 int launch_gemm_cfg(GemmParams& p, int64_t batch, hipStream_t stream) {
   p.tiles_m = static_cast<int32_t>(ceil_div(p.M, Cfg::BM));
   p.tiles_n = static_cast<int32_t>(ceil_div(p.N, Cfg::BN));
-  const int64_t tiles = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
-  if (tiles > 0x7FFFFFFFLL) return fail(FSH_ENOTSUP, "gemm: too many tiles");
-  const dim3 grid(static_cast<uint32_t>(tiles), static_cast<uint32_t>(batch)), block(Cfg::kThreads);
+  const int64_t tiles = p.symmetric ? static_cast<int64_t>(p.tiles_n) * (p.tiles_n + 1) / 2
+                                    : static_cast<int64_t>(p.tiles_m) * p.tiles_n;
+  p.tiles_per_matrix = static_cast<int32_t>(tiles);
+  p.work_items = tiles * batch;
+  p.items_per_xcd = ceil_div(p.work_items, static_cast<int64_t>(kXcds));
+  if (tiles > 0x3FFFFFFFLL || p.items_per_xcd * kXcds > 0x7FFFFFFFLL)
+    return fail(FSH_ENOTSUP, "gemm: too many tiles");
+  const dim3 grid(static_cast<uint32_t>(p.items_per_xcd * kXcds)), block(Cfg::kThreads);
   // Interior path: whole tiles, 8-byte friendly epilogue, 32-bit tile spans.
   const bool interior =
       p.M % Cfg::BM == 0 && p.N % Cfg::BN == 0 && p.K % Cfg::BK == 0 && p.ldc % 4 == 0 &&
       (reinterpret_cast<uintptr_t>(p.C) & 7) == 0 && p.sC % 4 == 0 &&
       (p.D == nullptr || (p.ldd % 4 == 0 && (reinterpret_cast<uintptr_t>(p.D) & 7) == 0 && p.sD % 4 == 0)) &&
       static_cast<int64_t>(Cfg::BM) * p.lda * 2 < (1LL << 31) && static_cast<int64_t>(Cfg::BN) * p.ldb * 2 < (1LL << 31);
+  if (interior && std::is_same<Cfg, BigCfg>::value) {
+    static bool reserved_dma = false;  // the attribute is per device function and sticky
+    if (!reserved_dma) {
+      if (int rc = reserve_lds(&gemm_nt_dma_kernel, DmaGemm::kLdsBytes)) return rc;
+      reserved_dma = true;
+    }
+    hipLaunchKernelGGL(gemm_nt_dma_kernel, grid, block, DmaGemm::kLdsBytes, stream, p);
+    return check_launch("gemm_nt_dma_kernel");
+  }
   if (interior) {
-    static bool reserved = false;  // the attribute is per device function and sticky
+    static bool reserved = false;
     if (!reserved) {
       if (int rc = reserve_lds(&gemm_nt_interior_kernel<Cfg>, Cfg::kLdsBytes)) return rc;
       reserved = true;
@@ -449,8 +674,10 @@ int launch_gemm(const fsh_gemm_desc& d, hipStream_t stream) {
     return fail(FSH_ENOTSUP, "gemm: k, lda, ldb and batch strides must be multiples of 8 and A, B 16-byte aligned");
   if (d.lda < d.k || d.ldb < d.k || d.ldc < d.n || (d.d_dev && d.ldd < d.n) || (d.ct_dev && d.ldct < d.m))
     return fail(FSH_EINVAL, "gemm: leading dimension smaller than the row length");
-  if (d.batch > 65535) return fail(FSH_ENOTSUP, "gemm: batch %lld exceeds 65535", (long long)d.batch);
+  if (d.symmetric && (d.m != d.n || d.ct_dev != nullptr))
+    return fail(FSH_EINVAL, "gemm: a symmetric product needs m == n and no transposed output");
   GemmParams p;
+  p.symmetric = d.symmetric ? 1 : 0;
   p.A = static_cast<const uint16_t*>(d.a_dev);
   p.B = static_cast<const uint16_t*>(d.b_dev);
   p.D = static_cast<const uint16_t*>(d.d_dev);
@@ -461,7 +688,8 @@ int launch_gemm(const fsh_gemm_desc& d, hipStream_t stream) {
   p.sA = d.stride_a; p.sB = d.stride_b; p.sD = d.stride_d; p.sC = d.stride_c; p.sCt = d.stride_ct;
   p.alpha = d.alpha; p.beta = d.beta;
   // The big tile pays off once it fills the chip at least once.
-  const int64_t big_tiles = ceil_div(d.m, BigCfg::BM) * ceil_div(d.n, BigCfg::BN) * d.batch;
+  const int64_t big_n = ceil_div(d.n, BigCfg::BN);
+  const int64_t big_tiles = (d.symmetric ? big_n * (big_n + 1) / 2 : ceil_div(d.m, BigCfg::BM) * big_n) * d.batch;
   if (big_tiles >= 192) return launch_gemm_cfg<BigCfg>(p, d.batch, stream);
   return launch_gemm_cfg<SmallCfg>(p, d.batch, stream);
 }
@@ -622,14 +850,16 @@ FSH_API int fsh_newton_schulz(void* x_dev, int64_t batch, int64_t rows, int64_t 
     g.m = s; g.n = s; g.k = l; g.lda = l; g.ldb = l; g.ldc = s;
     g.stride_a = sl; g.stride_b = sl; g.stride_c = ss;
     g.alpha = 1.0f; g.beta = 0.0f;
+    g.symmetric = 1;
     if (int rc = launch_gemm(g, stream)) return rc;
-    // P = b G + c G G
+    // P = b G + c G G, symmetric because G is
     g.a_dev = G; g.b_dev = G; g.d_dev = G; g.c_dev = P;
     g.m = s; g.n = s; g.k = s; g.lda = s; g.ldb = s; g.ldd = s; g.ldc = s;
     g.stride_a = ss; g.stride_b = ss; g.stride_d = ss; g.stride_c = ss;
     g.alpha = c; g.beta = b;
     if (int rc = launch_gemm(g, stream)) return rc;
     // X' = a X + P X, also written transposed into the other X^T buffer
+    g.symmetric = 0;
     g.a_dev = P; g.b_dev = XT[cur]; g.d_dev = X; g.c_dev = X; g.ct_dev = XT[cur ^ 1];
     g.m = s; g.n = l; g.k = s; g.lda = s; g.ldb = s; g.ldd = l; g.ldc = l; g.ldct = s;
     g.stride_a = ss; g.stride_b = sl; g.stride_d = sl; g.stride_c = sl; g.stride_ct = sl;

@@ -313,10 +313,12 @@ def newton_schulz(
 
 def gemm_nt(
     a: torch.Tensor, b: torch.Tensor, *, d: torch.Tensor | None = None, alpha: float = 1.0, beta: float = 0.0,
-    out: torch.Tensor | None = None, out_t: torch.Tensor | None = None,
+    out: torch.Tensor | None = None, out_t: torch.Tensor | None = None, symmetric: bool = False,
 ) -> torch.Tensor:
     """``bf16(alpha * a @ b^T + beta * d)`` for contiguous bf16 [batch, m, k] /
-    [batch, n, k] (or 2-D) operands; optionally also the transpose."""
+    [batch, n, k] (or 2-D) operands; optionally also the transpose.  With
+    ``symmetric`` the caller guarantees a symmetric result (m == n); only the
+    upper triangle of tiles is computed and mirrored."""
     _require_gpu(a, b)
     if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16 or not a.is_contiguous() or not b.is_contiguous():
         raise ValueError("a and b must be contiguous bf16")
@@ -345,6 +347,7 @@ def gemm_nt(
     desc.stride_a, desc.stride_b = m * k, n * k
     desc.stride_d = desc.stride_c = desc.stride_ct = m * n
     desc.alpha, desc.beta = alpha, beta
+    desc.symmetric = 1 if symmetric else 0
     status = _native.lib().fsh_gemm_bf16_nt(ctypes.byref(desc), stream_ptr(a.device))
     _native.check(status, "fsh_gemm_bf16_nt")
     return out

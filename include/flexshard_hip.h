@@ -205,6 +205,10 @@ typedef struct fsh_gemm_desc {
   int64_t batch;
   int64_t stride_a, stride_b, stride_d, stride_c, stride_ct;
   float alpha, beta;
+  int32_t symmetric; /* nonzero: the caller guarantees a symmetric result (m == n, e.g. b == a
+                        and d symmetric); only the tiles on or above the diagonal are
+                        computed and the rest is mirrored.  ct_dev must be null. */
+  int32_t reserved;  /* 0 */
 } fsh_gemm_desc;
 int fsh_gemm_bf16_nt(const fsh_gemm_desc* desc, void* stream);
 

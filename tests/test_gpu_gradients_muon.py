@@ -358,6 +358,59 @@ def test_gemm_building_block(device):
     assert torch.allclose(big.double(), want, rtol=2.0**-7, atol=0.5)
 
 
+def _gemm_reference(a, b, d=None, alpha=1.0, beta=0.0):
+    ref = alpha * (a.cpu().double() @ b.cpu().double().transpose(-1, -2))
+    return ref + beta * d.cpu().double() if d is not None else ref
+
+
+@pytest.mark.parametrize(
+    "batch,m,n,k",
+    [
+        (6, 1536, 1536, 192),  # 256x256x64 whole-tile kernel, 3 k-tiles
+        (7, 1536, 1280, 64),  # same kernel, single k-tile, padding workgroups in the grid
+        (1, 512, 384, 96),  # 128x128x32 whole-tile kernel
+        (9, 1544, 1288, 72),  # 256x256 predicated kernel
+    ],
+)
+def test_gemm_tile_paths(device, batch, m, n, k):
+    gen = torch.Generator().manual_seed(batch * 1000 + k)
+    a = torch.randn(batch, m, k, generator=gen).bfloat16().to(device)
+    b = torch.randn(batch, n, k, generator=gen).bfloat16().to(device)
+    d = torch.randn(batch, m, n, generator=gen).bfloat16().to(device)
+    # guard bands around both outputs: a tile path must not write outside them
+    pad = 2048
+    c_buf = torch.full((batch * m * n + 2 * pad,), 7.0, dtype=torch.bfloat16, device=device)
+    t_buf = torch.full((batch * m * n + 2 * pad,), 7.0, dtype=torch.bfloat16, device=device)
+    c = c_buf[pad:-pad].view(batch, m, n)
+    ct = t_buf[pad:-pad].view(batch, n, m)
+    hip_ops.gemm_nt(a, b, d=d, alpha=0.5, beta=2.0, out=c, out_t=ct)
+    ref = _gemm_reference(a, b, d, 0.5, 2.0)
+    assert torch.allclose(c.cpu().double(), ref, rtol=2.0**-8, atol=2e-2)  # one bf16 rounding of the fp32 result
+    assert torch.equal(ct, c.transpose(1, 2).contiguous())
+    for buf in (c_buf, t_buf):
+        assert (buf[:pad] == 7).all() and (buf[-pad:] == 7).all()
+
+
+@pytest.mark.parametrize("batch,n,k", [(6, 1536, 192), (1, 512, 96), (9, 1544, 72), (40, 520, 64)])
+def test_gemm_symmetric_mode_mirrors_the_upper_triangle(device, batch, n, k):
+    gen = torch.Generator().manual_seed(n + k)
+    a = torch.randn(batch, n, k, generator=gen).bfloat16().to(device)
+    full = hip_ops.gemm_nt(a, a)
+    sym = hip_ops.gemm_nt(a, a, symmetric=True)
+    assert torch.equal(sym, sym.transpose(1, 2))
+    assert torch.equal(torch.triu(sym), torch.triu(full))  # the computed tiles are the same work
+    assert torch.allclose(sym.float(), full.float(), rtol=2.0**-7, atol=1e-2)
+    # with a symmetric addend, as in P = b G + c G G
+    p_full = hip_ops.gemm_nt(sym, sym, d=sym, alpha=-0.05, beta=0.3)
+    p_sym = hip_ops.gemm_nt(sym, sym, d=sym, alpha=-0.05, beta=0.3, symmetric=True)
+    assert torch.equal(p_sym, p_sym.transpose(1, 2))
+    assert torch.equal(torch.triu(p_sym), torch.triu(p_full))
+    ref = _gemm_reference(sym, sym, sym, -0.05, 0.3)
+    assert torch.allclose(p_sym.cpu().double(), ref, rtol=2.0**-7, atol=2e-2 * ref.abs().max().item() / 8)
+    with pytest.raises(RuntimeError, match="symmetric"):
+        hip_ops.gemm_nt(a, a[:, : n - 8].contiguous(), symmetric=True)
+
+
 def test_newton_schulz_full_size_invariants(device):
     """Config 5 shapes: [7168, 2048] (tall, iterated as its transpose) and
     [2048, 2048].  Singular values of the result lie in the quintic's band and
