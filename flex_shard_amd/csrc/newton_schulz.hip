@@ -268,50 +268,114 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_nt_kernel(const GemmParams
   }
 }
 
-// Epilogue of the whole-tile kernels.  The accumulate is issued as
-// mfma(B, A), so accumulator r of block (i, j) belongs to output row
-// m = lane%32 and column n = 8*(r/4) + 4*(lane/32) + r%4 of the block: a lane
-// owns 4 consecutive columns and C leaves as 8-byte stores.
+// Epilogue of the whole-tile kernels, staged through LDS (free once the last
+// k-tile's barrier has passed; every wave uses a private region, but the
+// phases are still separated by workgroup barriers).
+//
+// The accumulate is issued as mfma(B, A), so accumulator r of block (i, j)
+// belongs to output row m = lane%32 and column n = 8*(r/4) + 4*(lane/32) + r%4
+// of the block.  In that layout a store instruction would touch 32 rows with
+// 16 bytes each, and the transposed output would leave as 2-byte stores.
+// Instead:
+//   1. finals = bf16(alpha*acc + beta*D) are computed in registers (D is read
+//      in accumulator layout, 16 loads in flight per 32-row block) and written
+//      to LDS as [row][col];
+//   2. the wave reads its region back row-wise and stores C as 16 bytes per
+//      lane, 256 contiguous bytes per row;
+//   3. for a transposed (or mirrored) output the finals are written again as
+//      [col][row] and leave the same way.
+// The LDS row pitch is the row plus 8 bytes: 8-byte writes of 16 lanes then
+// cover all 32 banks, and so do the row-wise 8-byte reads of a half-wave.
+template <typename Cfg>
+struct WholeTileEpilogue {
+  static constexpr int kPitch = Cfg::kWaveN * 2 + 8;   // bytes, [row][col] staging
+  static constexpr int kPitchT = Cfg::kWaveM * 2 + 8;  // bytes, [col][row] staging
+  static constexpr int kRegion =
+      (Cfg::kWaveM * kPitch > Cfg::kWaveN * kPitchT) ? Cfg::kWaveM * kPitch : Cfg::kWaveN * kPitchT;
+  static constexpr int kLdsBytes = Cfg::WM * Cfg::WN * kRegion;
+};
+
+// Stores a [rows][row_bytes] bf16 image held in LDS (pitch bytes apart) to
+// global rows `ld` elements apart, 16 bytes per lane.
+template <int kRows, int kRowBytes, int kPitch>
+__device__ inline void store_staged_rows(const uint8_t* region, uint16_t* dst, int64_t ld, int lane) {
+  constexpr int kLanesPerRow = kRowBytes / 16;
+  constexpr int kRowsPerPass = 64 / kLanesPerRow;
+  static_assert(kRowBytes % 16 == 0 && 64 % kLanesPerRow == 0 && kRows % kRowsPerPass == 0, "staged store shape");
+  const int r0 = lane / kLanesPerRow, chunk = lane % kLanesPerRow;
+#pragma unroll
+  for (int pass = 0; pass < kRows / kRowsPerPass; ++pass) {
+    const int r = pass * kRowsPerPass + r0;
+    const uint8_t* src = region + r * kPitch + chunk * 16;
+    const u32x2 lo = *reinterpret_cast<const u32x2*>(src);
+    const u32x2 hi = *reinterpret_cast<const u32x2*>(src + 8);
+    *reinterpret_cast<u32x4*>(dst + r * ld + chunk * 8) = u32x4{lo.x, lo.y, hi.x, hi.y};
+  }
+}
+
 template <typename Cfg>
 __device__ inline void store_whole_tile(const GemmParams& p, int64_t batch, int64_t m0, int64_t n0, int wm, int wn,
-                                        int lane, bool mirror, const f32x16 (&acc)[Cfg::TM][Cfg::TN]) {
+                                        int lane, bool mirror, const f32x16 (&acc)[Cfg::TM][Cfg::TN],
+                                        uint8_t* lds) {
+  using Epi = WholeTileEpilogue<Cfg>;
   constexpr int TM = Cfg::TM, TN = Cfg::TN;
   const uint16_t* D = p.D ? p.D + batch * p.sD : nullptr;
   uint16_t* C = p.C + batch * p.sC;
   // A symmetric product mirrors its off-diagonal tiles into the lower triangle.
   uint16_t* Ct = mirror ? C : (p.Ct ? p.Ct + batch * p.sCt : nullptr);
   const int64_t ldct = mirror ? p.ldc : p.ldct;
+  const int64_t wave_row = m0 + wm * Cfg::kWaveM, wave_col = n0 + wn * Cfg::kWaveN;
+  uint8_t* region = lds + (wm * Cfg::WN + wn) * Epi::kRegion;
+  const int r_lane = lane & 31, h = lane >> 5;
+
+  uint32_t fin[TM][TN][4][2];  // packed bf16 pairs of the finals, accumulator layout
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int64_t row = m0 + wm * Cfg::kWaveM + i * 32 + (lane & 31);
+    u32x2 draw[TN][4];
+    if (D != nullptr) {
+      const uint16_t* drow = D + (wave_row + i * 32 + r_lane) * p.ldd + wave_col + 4 * h;
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) draw[j][b] = *reinterpret_cast<const u32x2*>(drow + j * 32 + 8 * b);
+    }
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
-        const int64_t col = n0 + wn * Cfg::kWaveN + j * 32 + 8 * b + 4 * (lane >> 5);
-        float dv[4] = {0.f, 0.f, 0.f, 0.f};
+        float v[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) v[t] = p.alpha * acc[i][j][4 * b + t];
         if (D != nullptr) {
-          const u32x2 raw = *reinterpret_cast<const u32x2*>(&D[row * p.ldd + col]);
-          dv[0] = u32_as_f32(raw.x << 16);
-          dv[1] = u32_as_f32(raw.x & 0xFFFF0000u);
-          dv[2] = u32_as_f32(raw.y << 16);
-          dv[3] = u32_as_f32(raw.y & 0xFFFF0000u);
+          v[0] += p.beta * u32_as_f32(draw[j][b].x << 16);
+          v[1] += p.beta * u32_as_f32(draw[j][b].x & 0xFFFF0000u);
+          v[2] += p.beta * u32_as_f32(draw[j][b].y << 16);
+          v[3] += p.beta * u32_as_f32(draw[j][b].y & 0xFFFF0000u);
         }
-        uint32_t packed[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          float v = p.alpha * acc[i][j][4 * b + t];
-          if (D != nullptr) v += p.beta * dv[t];
-          packed[t] = f32_to_bf16_bits(v);
-        }
-        *reinterpret_cast<u32x2*>(&C[row * p.ldc + col]) =
-            u32x2{packed[0] | (packed[1] << 16), packed[2] | (packed[3] << 16)};
-        if (Ct != nullptr) {
-#pragma unroll
-          for (int t = 0; t < 4; ++t) Ct[(col + t) * ldct + row] = static_cast<uint16_t>(packed[t]);
-        }
+        fin[i][j][b][0] = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
+        fin[i][j][b][1] = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
+        *reinterpret_cast<u32x2*>(region + (i * 32 + r_lane) * Epi::kPitch + (j * 32 + 8 * b + 4 * h) * 2) =
+            u32x2{fin[i][j][b][0], fin[i][j][b][1]};
       }
   }
+  __syncthreads();
+  store_staged_rows<Cfg::kWaveM, Cfg::kWaveN * 2, Epi::kPitch>(region, C + wave_row * p.ldc + wave_col, p.ldc, lane);
+  if (Ct == nullptr) return;  // uniform over the workgroup
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const uint32_t pair = fin[i][j][b][t >> 1];
+          *reinterpret_cast<uint16_t*>(region + (j * 32 + 8 * b + 4 * h + t) * Epi::kPitchT + (i * 32 + r_lane) * 2) =
+              static_cast<uint16_t>((t & 1) ? (pair >> 16) : pair);
+        }
+  __syncthreads();
+  store_staged_rows<Cfg::kWaveN, Cfg::kWaveM * 2, Epi::kPitchT>(region, Ct + wave_col * ldct + wave_row, ldct, lane);
 }
 
 // Scheduling-group masks of __builtin_amdgcn_sched_group_barrier.
@@ -447,7 +511,8 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_nt_interior_kernel(const G
   for (int64_t kt = 0; kt + 1 < ktiles; ++kt) k_tile(kt, std::true_type{});
   k_tile(ktiles - 1, std::false_type{});
 
-  store_whole_tile<Cfg>(p, batch, m0, n0, wm, wn, lane, p.symmetric && tm != tn, acc);
+  store_whole_tile<Cfg>(p, batch, m0, n0, wm, wn, lane, p.symmetric && tm != tn, acc,
+                        reinterpret_cast<uint8_t*>(smem));
 }
 
 // ---------------------------------------------------------------------------
@@ -478,7 +543,7 @@ struct DmaGemm {
   static constexpr int kRowBytes = BK * 2;                   // 128
   static constexpr int kOperandBytes = BM * kRowBytes;       // 32 KB per operand and stage
   static constexpr int kStageBytes = 2 * kOperandBytes;      // 64 KB
-  static constexpr int kLdsBytes = 2 * kStageBytes;
+  static constexpr int kLoopLdsBytes = 2 * kStageBytes;
   static constexpr int kLoadsPerOperand = BM / 8 / 4;        // wave-level 1 KB loads per wave: 8
 };
 
@@ -607,8 +672,10 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   for (int64_t kt = 0; kt + 1 < ktiles; ++kt) k_tile(kt, std::true_type{});
   k_tile(ktiles - 1, std::false_type{});
 
-  store_whole_tile<Cfg>(p, batch, m0, n0, wm, wn, lane, p.symmetric && tm != tn, acc);
+  store_whole_tile<Cfg>(p, batch, m0, n0, wm, wn, lane, p.symmetric && tm != tn, acc, lds_bytes);
 }
+
+constexpr int max_int(int a, int b) { return a > b ? a : b; }
 
 template <typename Kernel>
 int reserve_lds(Kernel kernel, int bytes) {
@@ -631,28 +698,31 @@ int launch_gemm_cfg(GemmParams& p, int64_t batch, hipStream_t stream) {
   if (tiles > 0x3FFFFFFFLL || p.items_per_xcd * kXcds > 0x7FFFFFFFLL)
     return fail(FSH_ENOTSUP, "gemm: too many tiles");
   const dim3 grid(static_cast<uint32_t>(p.items_per_xcd * kXcds)), block(Cfg::kThreads);
-  // Interior path: whole tiles, 8-byte friendly epilogue, 32-bit tile spans.
+  // Interior path: whole tiles, 16-byte stores in the epilogue, 32-bit tile spans.
   const bool interior =
-      p.M % Cfg::BM == 0 && p.N % Cfg::BN == 0 && p.K % Cfg::BK == 0 && p.ldc % 4 == 0 &&
-      (reinterpret_cast<uintptr_t>(p.C) & 7) == 0 && p.sC % 4 == 0 &&
+      p.M % Cfg::BM == 0 && p.N % Cfg::BN == 0 && p.K % Cfg::BK == 0 && p.ldc % 8 == 0 &&
+      (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 && p.sC % 8 == 0 &&
+      (p.Ct == nullptr || (p.ldct % 8 == 0 && (reinterpret_cast<uintptr_t>(p.Ct) & 15) == 0 && p.sCt % 8 == 0)) &&
       (p.D == nullptr || (p.ldd % 4 == 0 && (reinterpret_cast<uintptr_t>(p.D) & 7) == 0 && p.sD % 4 == 0)) &&
       static_cast<int64_t>(Cfg::BM) * p.lda * 2 < (1LL << 31) && static_cast<int64_t>(Cfg::BN) * p.ldb * 2 < (1LL << 31);
   if (interior && std::is_same<Cfg, BigCfg>::value) {
+    constexpr int kDmaLds = max_int(DmaGemm::kLoopLdsBytes, WholeTileEpilogue<DmaGemm>::kLdsBytes);
     static bool reserved_dma = false;  // the attribute is per device function and sticky
     if (!reserved_dma) {
-      if (int rc = reserve_lds(&gemm_nt_dma_kernel, DmaGemm::kLdsBytes)) return rc;
+      if (int rc = reserve_lds(&gemm_nt_dma_kernel, kDmaLds)) return rc;
       reserved_dma = true;
     }
-    hipLaunchKernelGGL(gemm_nt_dma_kernel, grid, block, DmaGemm::kLdsBytes, stream, p);
+    hipLaunchKernelGGL(gemm_nt_dma_kernel, grid, block, kDmaLds, stream, p);
     return check_launch("gemm_nt_dma_kernel");
   }
   if (interior) {
+    constexpr int kInteriorLds = max_int(Cfg::kLdsBytes, WholeTileEpilogue<Cfg>::kLdsBytes);
     static bool reserved = false;
     if (!reserved) {
-      if (int rc = reserve_lds(&gemm_nt_interior_kernel<Cfg>, Cfg::kLdsBytes)) return rc;
+      if (int rc = reserve_lds(&gemm_nt_interior_kernel<Cfg>, kInteriorLds)) return rc;
       reserved = true;
     }
-    hipLaunchKernelGGL(gemm_nt_interior_kernel<Cfg>, grid, block, Cfg::kLdsBytes, stream, p);
+    hipLaunchKernelGGL(gemm_nt_interior_kernel<Cfg>, grid, block, kInteriorLds, stream, p);
     return check_launch("gemm_nt_interior_kernel");
   }
   static bool reserved_edge = false;
