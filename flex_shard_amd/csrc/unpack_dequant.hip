@@ -3,10 +3,10 @@
 // the FP8 bytes.
 //
 // A workgroup owns one block x block tile of one (rank, parameter) chunk.  For
-// block = 128 and 16-byte friendly addresses each thread moves 16 FP8 bytes
-// per row pass: one 16-byte load, one 16-byte store into the compact buffer,
-// eight v_cvt_pk_f32_fp8 + multiplies by the tile's reciprocal scale, and two
-// 16-byte bf16 stores.  Any other block size or alignment (rank rows at odd
+// block = 128 and 16-byte friendly addresses each thread moves 8 FP8 bytes
+// per row pass: one 8-byte load, one 8-byte store into the compact buffer,
+// four v_cvt_pk_f32_fp8 + multiplies by the tile's reciprocal scale, and one
+// 16-byte bf16 store.  Any other block size or alignment (rank rows at odd
 // byte offsets inside a mixed bucket) takes an element-wise path.
 #include "common.hpp"
 
@@ -52,14 +52,24 @@ __global__ __launch_bounds__(kThreads) void unpack_dequant_kernel(
     const int64_t* __restrict__ tile_starts, int nchunks, uint8_t* __restrict__ compact,
     uint8_t* __restrict__ dequant, int block) {
   const int64_t bid = blockIdx.x;
-  // Largest c with tile_starts[c] <= bid.
-  int lo = 0, hi = nchunks - 1;
-  while (lo < hi) {
-    const int mid = (lo + hi + 1) >> 1;
-    if (tile_starts[mid] <= bid)
-      lo = mid;
-    else
-      hi = mid - 1;
+  // Largest c with tile_starts[c] <= bid.  Up to 64 chunks are resolved in one
+  // memory round trip (a lane per chunk and a ballot) instead of a dependent
+  // chain of binary-search probes; tile_starts is ascending, so the count of
+  // entries <= bid is the index plus one.
+  int lo = 0;
+  if (nchunks <= 64) {
+    const int l = threadIdx.x & 63;
+    const bool below = l < nchunks && tile_starts[l] <= bid;
+    lo = __builtin_popcountll(__ballot(below)) - 1;
+  } else {
+    int hi = nchunks - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (tile_starts[mid] <= bid)
+        lo = mid;
+      else
+        hi = mid - 1;
+    }
   }
   const fsh_unpack_chunk ch = chunks[lo];
   const int64_t tiles_c = (ch.in_dim + block - 1) / block;
@@ -80,37 +90,42 @@ __global__ __launch_bounds__(kThreads) void unpack_dequant_kernel(
   const bool fast = block == 128 && (ch.in_dim & 15) == 0 && (addr_bits & 15) == 0;
 
   if (fast) {
-    const int g = tid & 7, r0 = tid >> 3;
-    const int64_t col = tc * 128 + g * 16;
+    // 16 threads per tile row, 8 FP8 bytes each: every load and store
+    // instruction of a wave then covers whole contiguous row segments (128 B
+    // of FP8, 256 B of bf16), which the memory pipeline needs for full-width
+    // requests.  16 rows per pass, 8 passes, all loads issued up front; rows
+    // past the chunk's end are clamped for the load and skipped for the stores.
+    const int g = tid & 15, r0 = tid >> 4;
+    const int64_t col = tc * 128 + g * 8;
     if (col >= ch.in_dim) return;
+    u32x2 vin[8];
+    int64_t idxs[8];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int64_t row = tr * 128 + r0 + 32 * k;
-      if (row >= ch.rows) break;
-      const int64_t idx = row * ch.in_dim + col;
-      const u32x4 v = load_stream_u32x4(src + idx);
-      if (cq) store_stream_u32x4(cq + idx, v);
+    for (int k = 0; k < 8; ++k) {
+      const int64_t row = tr * 128 + r0 + 16 * k;
+      idxs[k] = (row < ch.rows ? row : ch.rows - 1) * ch.in_dim + col;
+      vin[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(src + idxs[k]));
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      if (tr * 128 + r0 + 16 * k >= ch.rows) break;
+      const int64_t idx = idxs[k];
+      const u32x2 v = vin[k];
+      if (cq) store_stream_u32x2(cq + idx, v.x, v.y);
       if (dq) {
-        float f[16];
+        float f[8];
         dequant4(v.x, scale, f);
         dequant4(v.y, scale, f + 4);
-        dequant4(v.z, scale, f + 8);
-        dequant4(v.w, scale, f + 12);
         if (DQ == FSH_DT_BF16) {
-          u32x4 o0, o1;
-          o0.x = f32_to_bf16_bits(f[0]) | (f32_to_bf16_bits(f[1]) << 16);
-          o0.y = f32_to_bf16_bits(f[2]) | (f32_to_bf16_bits(f[3]) << 16);
-          o0.z = f32_to_bf16_bits(f[4]) | (f32_to_bf16_bits(f[5]) << 16);
-          o0.w = f32_to_bf16_bits(f[6]) | (f32_to_bf16_bits(f[7]) << 16);
-          o1.x = f32_to_bf16_bits(f[8]) | (f32_to_bf16_bits(f[9]) << 16);
-          o1.y = f32_to_bf16_bits(f[10]) | (f32_to_bf16_bits(f[11]) << 16);
-          o1.z = f32_to_bf16_bits(f[12]) | (f32_to_bf16_bits(f[13]) << 16);
-          o1.w = f32_to_bf16_bits(f[14]) | (f32_to_bf16_bits(f[15]) << 16);
-          store_stream_u32x4(dq + idx * 2, o0);
-          store_stream_u32x4(dq + idx * 2 + 16, o1);
+          u32x4 o;
+          o.x = f32_to_bf16_bits(f[0]) | (f32_to_bf16_bits(f[1]) << 16);
+          o.y = f32_to_bf16_bits(f[2]) | (f32_to_bf16_bits(f[3]) << 16);
+          o.z = f32_to_bf16_bits(f[4]) | (f32_to_bf16_bits(f[5]) << 16);
+          o.w = f32_to_bf16_bits(f[6]) | (f32_to_bf16_bits(f[7]) << 16);
+          store_stream_u32x4(dq + idx * 2, o);
         } else {
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
+          for (int j = 0; j < 2; ++j) {
             u32x4 o = {f32_as_u32(f[4 * j]), f32_as_u32(f[4 * j + 1]), f32_as_u32(f[4 * j + 2]),
                        f32_as_u32(f[4 * j + 3])};
             store_stream_u32x4(dq + idx * 4 + 16 * j, o);
