@@ -120,34 +120,89 @@ __device__ __forceinline__ float lerp_f32(float start, float end, float w) {
   return w < 0.5f ? start + w * diff : end - diff * (1.0f - w);
 }
 
+// Eight bf16 values of a 16-byte vector as floats, and back.
+__device__ __forceinline__ void unpack8(const u32x4 v, float* f) {
+  const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    f[2 * j] = u32_as_f32(d[j] << 16);
+    f[2 * j + 1] = u32_as_f32(d[j] & 0xFFFF0000u);
+  }
+}
+__device__ __forceinline__ u32x4 pack8(const uint32_t* bits) {
+  return u32x4{bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16), bits[4] | (bits[5] << 16),
+               bits[6] | (bits[7] << 16)};
+}
+
+__device__ __forceinline__ void muon_prepare_one(float m, float g, float one_minus_mu, float mu, int nesterov,
+                                                 uint32_t* m_bits, uint32_t* out_bits) {
+  *m_bits = f32_to_bf16_bits(lerp_f32(m, g, one_minus_mu));
+  *out_bits = nesterov ? f32_to_bf16_bits(lerp_f32(g, bf16_bits_to_f32(*m_bits), mu)) : *m_bits;
+}
+
 // m = bf16(lerp(m, g, 1-mu)); out = nesterov ? bf16(lerp(g, m, mu)) : m.
+// 8 elements (16 bytes) per thread and iteration when the three pointers are
+// 16-byte aligned, then a scalar tail; scalar throughout otherwise.
 __global__ __launch_bounds__(kThreads) void muon_prepare_kernel(uint16_t* __restrict__ mom,
                                                                const uint16_t* __restrict__ grad,
                                                                uint16_t* __restrict__ out, int64_t n,
-                                                               float one_minus_mu, float mu, int nesterov) {
+                                                               float one_minus_mu, float mu, int nesterov,
+                                                               int vec_ok) {
   const int64_t tid = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   const int64_t nthreads = static_cast<int64_t>(gridDim.x) * kThreads;
-  for (int64_t i = tid; i < n; i += nthreads) {
-    const float g = bf16_bits_to_f32(grad[i]);
-    const uint32_t mb = f32_to_bf16_bits(lerp_f32(bf16_bits_to_f32(mom[i]), g, one_minus_mu));
-    mom[i] = static_cast<uint16_t>(mb);
-    out[i] = nesterov ? static_cast<uint16_t>(f32_to_bf16_bits(lerp_f32(g, bf16_bits_to_f32(mb), mu)))
-                      : static_cast<uint16_t>(mb);
+  int64_t done = 0;
+  if (vec_ok) {
+    const int64_t groups = n / 8;
+    for (int64_t gi = tid; gi < groups; gi += nthreads) {
+      float m[8], g[8];
+      unpack8(load_stream_u32x4(mom + gi * 8), m);
+      unpack8(load_stream_u32x4(grad + gi * 8), g);
+      uint32_t mb[8], ob[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) muon_prepare_one(m[j], g[j], one_minus_mu, mu, nesterov, &mb[j], &ob[j]);
+      store_stream_u32x4(mom + gi * 8, pack8(mb));
+      store_stream_u32x4(out + gi * 8, pack8(ob));
+    }
+    done = groups * 8;
   }
+  for (int64_t i = done + tid; i < n; i += nthreads) {
+    uint32_t mb, ob;
+    muon_prepare_one(bf16_bits_to_f32(mom[i]), bf16_bits_to_f32(grad[i]), one_minus_mu, mu, nesterov, &mb, &ob);
+    mom[i] = static_cast<uint16_t>(mb);
+    out[i] = static_cast<uint16_t>(ob);
+  }
+}
+
+__device__ __forceinline__ uint32_t muon_apply_one(float p, float d, float decay, float neg_lr, float dir_scale) {
+  if (dir_scale != 1.0f) d = bf16_bits_to_f32(f32_to_bf16_bits(d * dir_scale));
+  p = bf16_bits_to_f32(f32_to_bf16_bits(p * decay));
+  return f32_to_bf16_bits(p + neg_lr * d);
 }
 
 // p = bf16(p * decay); p = bf16(p + neg_lr * d'), d' = scale == 1 ? d : bf16(d * scale).
 __global__ __launch_bounds__(kThreads) void muon_apply_kernel(uint16_t* __restrict__ param,
                                                              const uint16_t* __restrict__ dir, int64_t n,
-                                                             float decay, float neg_lr, float dir_scale) {
+                                                             float decay, float neg_lr, float dir_scale,
+                                                             int vec_ok) {
   const int64_t tid = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   const int64_t nthreads = static_cast<int64_t>(gridDim.x) * kThreads;
-  for (int64_t i = tid; i < n; i += nthreads) {
-    float d = bf16_bits_to_f32(dir[i]);
-    if (dir_scale != 1.0f) d = bf16_bits_to_f32(f32_to_bf16_bits(d * dir_scale));
-    const float p = bf16_bits_to_f32(f32_to_bf16_bits(bf16_bits_to_f32(param[i]) * decay));
-    param[i] = static_cast<uint16_t>(f32_to_bf16_bits(p + neg_lr * d));
+  int64_t done = 0;
+  if (vec_ok) {
+    const int64_t groups = n / 8;
+    for (int64_t gi = tid; gi < groups; gi += nthreads) {
+      float pv[8], dv[8];
+      unpack8(load_stream_u32x4(param + gi * 8), pv);
+      unpack8(load_stream_u32x4(dir + gi * 8), dv);
+      uint32_t pb[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) pb[j] = muon_apply_one(pv[j], dv[j], decay, neg_lr, dir_scale);
+      store_stream_u32x4(param + gi * 8, pack8(pb));
+    }
+    done = groups * 8;
   }
+  for (int64_t i = done + tid; i < n; i += nthreads)
+    param[i] = static_cast<uint16_t>(
+        muon_apply_one(bf16_bits_to_f32(param[i]), bf16_bits_to_f32(dir[i]), decay, neg_lr, dir_scale));
 }
 
 }  // namespace
@@ -219,10 +274,13 @@ FSH_API int fsh_muon_prepare(void* momentum_dev, const void* grad_dev, void* out
   if (numel < 0) return fail(FSH_EINVAL, "fsh_muon_prepare: negative numel");
   if (numel == 0) return FSH_OK;
   if (!momentum_dev || !grad_dev || !out_dev) return fail(FSH_EINVAL, "fsh_muon_prepare: null pointer");
-  hipLaunchKernelGGL(muon_prepare_kernel, dim3(grid_for(numel)), dim3(kThreads), 0,
+  if (!aligned(momentum_dev, 2) || !aligned(grad_dev, 2) || !aligned(out_dev, 2))
+    return fail(FSH_EINVAL, "fsh_muon_prepare: pointers misaligned for bf16");
+  const int vec_ok = aligned(momentum_dev, 16) && aligned(grad_dev, 16) && aligned(out_dev, 16);
+  hipLaunchKernelGGL(muon_prepare_kernel, dim3(grid_for(ceil_div(numel, 8))), dim3(kThreads), 0,
                      static_cast<hipStream_t>(stream), static_cast<uint16_t*>(momentum_dev),
                      static_cast<const uint16_t*>(grad_dev), static_cast<uint16_t*>(out_dev), numel,
-                     lerp_weight, nesterov_weight, nesterov);
+                     lerp_weight, nesterov_weight, nesterov, vec_ok);
   return check_launch("fsh_muon_prepare");
 }
 
@@ -232,9 +290,12 @@ FSH_API int fsh_muon_apply(void* param_dev, const void* direction_dev, int64_t n
   if (numel < 0) return fail(FSH_EINVAL, "fsh_muon_apply: negative numel");
   if (numel == 0) return FSH_OK;
   if (!param_dev || !direction_dev) return fail(FSH_EINVAL, "fsh_muon_apply: null pointer");
-  hipLaunchKernelGGL(muon_apply_kernel, dim3(grid_for(numel)), dim3(kThreads), 0,
+  if (!aligned(param_dev, 2) || !aligned(direction_dev, 2))
+    return fail(FSH_EINVAL, "fsh_muon_apply: pointers misaligned for bf16");
+  const int vec_ok = aligned(param_dev, 16) && aligned(direction_dev, 16);
+  hipLaunchKernelGGL(muon_apply_kernel, dim3(grid_for(ceil_div(numel, 8))), dim3(kThreads), 0,
                      static_cast<hipStream_t>(stream), static_cast<uint16_t*>(param_dev),
                      static_cast<const uint16_t*>(direction_dev), numel, decay_factor, neg_adjusted_lr,
-                     direction_scale);
+                     direction_scale, vec_ok);
   return check_launch("fsh_muon_apply");
 }

@@ -768,19 +768,29 @@ int launch_gemm(const fsh_gemm_desc& d, hipStream_t stream) {
 constexpr int kNormThreads = 256;
 constexpr int kNormBlocksPerMatrix = 64;
 
-// partial[b][j] = sum of squares of a slice of matrix b (fp32, fixed order).
+// partial[b][j] = sum of squares of slice j of matrix b in fp32.  The order
+// is fixed: a thread walks its 8-element groups front to back, lanes are
+// folded by the wave reduction, waves left to right.  numel is a multiple of
+// 8 and every matrix starts 16-byte aligned.
 __global__ __launch_bounds__(kNormThreads) void sumsq_partial_kernel(const uint16_t* __restrict__ x,
                                                                     int64_t numel, float* __restrict__ partial) {
   __shared__ float lds[kNormThreads / 64];
   const int64_t b = blockIdx.y;
   const uint16_t* m = x + b * numel;
-  const int64_t per = ceil_div(ceil_div(numel, (int64_t)kNormBlocksPerMatrix), 8) * 8;
+  const int64_t groups = numel / 8;
+  const int64_t per = ceil_div(groups, (int64_t)kNormBlocksPerMatrix);
   const int64_t begin = blockIdx.x * per;
-  const int64_t end = (begin + per) < numel ? (begin + per) : numel;
+  const int64_t end = (begin + per) < groups ? (begin + per) : groups;
   float s = 0.0f;
-  for (int64_t i = begin + threadIdx.x; i < end; i += kNormThreads) {
-    const float v = bf16_bits_to_f32(m[i]);
-    s += v * v;
+  for (int64_t g = begin + threadIdx.x; g < end; g += kNormThreads) {
+    const u32x4 v = load_stream_u32x4(m + g * 8);
+    const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float lo = u32_as_f32(d[j] << 16), hi = u32_as_f32(d[j] & 0xFFFF0000u);
+      s += lo * lo;
+      s += hi * hi;
+    }
   }
   s = wave_sum_f32(s);
   if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = s;
@@ -791,37 +801,60 @@ __global__ __launch_bounds__(kNormThreads) void sumsq_partial_kernel(const uint1
 // Reads matrix b of `in` ([rows, cols]), divides by max(||.||_F, eps) as bf16
 // tensor ops would (norm rounded to bf16, fp32 division, bf16 result), and
 // writes the result to `out_same` ([rows, cols]) and `out_t` ([cols, rows]).
-// 32x32 tiles go through LDS so both writes are row-contiguous.
+// A workgroup owns a 64x64 tile: 16-byte loads and stores of 8 elements along
+// the rows, and for the transposed copy the tile goes through LDS and leaves
+// as 16-byte stores of 8 elements along the columns.  rows and cols are
+// multiples of 8, so an 8-element group is either whole or absent.
+constexpr int kNormTile = 64;
+constexpr int kNormPitch = kNormTile + 2;  // u16 per LDS row
 __global__ __launch_bounds__(kNormThreads) void normalize_dual_kernel(const uint16_t* __restrict__ in,
                                                                      uint16_t* __restrict__ out_same,
                                                                      uint16_t* __restrict__ out_t, int64_t rows,
                                                                      int64_t cols, const float* __restrict__ partial,
                                                                      float eps_bf16) {
-  __shared__ uint16_t tile[32][33];
+  __shared__ uint16_t tile[kNormTile * kNormPitch];
   const int64_t b = blockIdx.z;
   float total = 0.0f;
   for (int j = 0; j < kNormBlocksPerMatrix; ++j) total += partial[b * kNormBlocksPerMatrix + j];
   float norm = bf16_bits_to_f32(f32_to_bf16_bits(sqrtf(total)));
   norm = norm < eps_bf16 ? eps_bf16 : norm;
-  const int64_t r0 = static_cast<int64_t>(blockIdx.y) * 32, c0 = static_cast<int64_t>(blockIdx.x) * 32;
+  const int64_t r0 = static_cast<int64_t>(blockIdx.y) * kNormTile, c0 = static_cast<int64_t>(blockIdx.x) * kNormTile;
   const uint16_t* m = in + b * rows * cols;
   uint16_t* o = out_same + b * rows * cols;
   uint16_t* ot = out_t + b * rows * cols;
-  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+  const int q = threadIdx.x & 7, line = threadIdx.x >> 3;  // 8 groups of 8 elements per line, 32 lines per pass
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const int64_t r = r0 + ty + 8 * k, c = c0 + tx;
+  for (int pass = 0; pass < 2; ++pass) {
+    const int lr = line + 32 * pass;
+    const int64_t r = r0 + lr, c = c0 + 8 * q;
     if (r < rows && c < cols) {
-      const uint16_t v = static_cast<uint16_t>(f32_to_bf16_bits(bf16_bits_to_f32(m[r * cols + c]) / norm));
-      o[r * cols + c] = v;
-      tile[ty + 8 * k][tx] = v;
+      const u32x4 v = load_stream_u32x4(m + r * cols + c);
+      const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+      uint32_t bits[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        bits[2 * j] = f32_to_bf16_bits(u32_as_f32(d[j] << 16) / norm);
+        bits[2 * j + 1] = f32_to_bf16_bits(u32_as_f32(d[j] & 0xFFFF0000u) / norm);
+      }
+      store_stream_u32x4(o + r * cols + c, u32x4{bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16),
+                                                   bits[4] | (bits[5] << 16), bits[6] | (bits[7] << 16)});
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        *reinterpret_cast<uint32_t*>(&tile[lr * kNormPitch + 8 * q + 2 * j]) = bits[2 * j] | (bits[2 * j + 1] << 16);
     }
   }
   __syncthreads();
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const int64_t c = c0 + ty + 8 * k, r = r0 + tx;
-    if (r < rows && c < cols) ot[c * rows + r] = tile[tx][ty + 8 * k];
+  for (int pass = 0; pass < 2; ++pass) {
+    const int lc = line + 32 * pass;  // tile column = row of the transposed output
+    const int64_t c = c0 + lc, r = r0 + 8 * q;
+    if (c < cols && r < rows) {
+      uint32_t bits[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) bits[j] = tile[(8 * q + j) * kNormPitch + lc];
+      store_stream_u32x4(ot + c * rows + r, u32x4{bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16),
+                                                    bits[4] | (bits[5] << 16), bits[6] | (bits[7] << 16)});
+    }
   }
 }
 
@@ -903,9 +936,9 @@ FSH_API int fsh_newton_schulz(void* x_dev, int64_t batch, int64_t rows, int64_t 
     // and X^T for a tall one.
     uint16_t* same = tall ? XT[cur] : X;
     uint16_t* transposed = tall ? X : XT[cur];
-    const dim3 grid(static_cast<uint32_t>(ceil_div(cols, 32)), static_cast<uint32_t>(ceil_div(rows, 32)),
-                    static_cast<uint32_t>(batch));
-    if (grid.y > 65535) return fail(FSH_ENOTSUP, "fsh_newton_schulz: more than %d row tiles", 65535 * 32);
+    const dim3 grid(static_cast<uint32_t>(ceil_div(cols, (int64_t)kNormTile)),
+                    static_cast<uint32_t>(ceil_div(rows, (int64_t)kNormTile)), static_cast<uint32_t>(batch));
+    if (grid.y > 65535) return fail(FSH_ENOTSUP, "fsh_newton_schulz: more than %d row tiles", 65535 * kNormTile);
     hipLaunchKernelGGL(normalize_dual_kernel, grid, dim3(kNormThreads), 0, stream, x, same, transposed, rows,
                        cols, partial, bf16_round_host(eps));
     if (int rc = check_launch("normalize_dual_kernel")) return rc;
