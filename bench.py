@@ -62,8 +62,8 @@ def _event_ms(fn, steps: int, warmup: int) -> tuple[float, float]:
     return wall, start.elapsed_time(stop)
 
 
-def build_quant_workload(device, layers: int):
-    """Per layer: rank 0's local shards as views of one flat bf16 storage (the
+def build_quant_workload(device, layers: int, rank: int = 0, spec=None, std: float = 0.02):
+    """Per layer: one rank's local shards as views of one flat bf16 storage (the
     sharded bucket storage layout), their ParamInfos, and a reusable payload."""
     import torch.nn as nn
 
@@ -71,13 +71,14 @@ def build_quant_workload(device, layers: int):
     from flex_shard_amd.testing import LLAMA3_8B_LAYER, FakeMesh, make_param_infos, seeded_normal
 
     placement = Fp8BucketedBlockShard(world_size=8, weight_factory=_factory)
-    mesh = FakeMesh(8, 0)
-    meta = [(n, nn.Parameter(torch.empty(s, device="meta", dtype=torch.bfloat16))) for n, s in LLAMA3_8B_LAYER]
+    mesh = FakeMesh(8, rank)
+    meta = [(n, nn.Parameter(torch.empty(s, device="meta", dtype=torch.bfloat16)))
+            for n, s in (spec or LLAMA3_8B_LAYER)]
     infos = make_param_infos(meta, placement, mesh)
     local_numel = infos[0].bucket_layout.local_numel
     work = []
     for layer in range(layers):
-        storage = seeded_normal((local_numel,), 0.02, 1000 + layer, device)
+        storage = seeded_normal((local_numel,), std, 1000 + layer, device)
         shards = [
             storage[i.byte_offset // 2 : i.byte_offset // 2 + i.local_numel].view(i.local_shape) for i in infos
         ]
@@ -85,10 +86,10 @@ def build_quant_workload(device, layers: int):
     return placement, mesh, infos, work
 
 
-def bench_quant_pack(device, steps, warmup, layers):
-    placement, mesh, infos, work = build_quant_workload(device, layers)
+def bench_quant_pack(device, steps, warmup, layers, rank: int = 0, spec=None, std: float = 0.02):
+    placement, mesh, infos, work = build_quant_workload(device, layers, rank, spec, std)
     metadata = placement._quant_metadata_from_infos(infos)
-    plan = metadata.rank_pack_plans[0]
+    plan = metadata.rank_pack_plans[rank]
     elems = plan.qdata_numel
     scales = sum(sum(c.scale_numels) for c in plan.chunks)
     algo_bytes = 3 * elems + 4 * scales  # 2 B read + 1 B write per element, 4 B per tile scale
@@ -98,7 +99,7 @@ def bench_quant_pack(device, steps, warmup, layers):
         _, shards = work[i % len(work)]
         # The placement's own entry point; the payload buffer is recycled the
         # way the caching allocator recycles it in a training loop.
-        payloads[i % len(work)] = placement._pack_local_quantized_chunks(shards, infos, 0, metadata)
+        payloads[i % len(work)] = placement._pack_local_quantized_chunks(shards, infos, rank, metadata)
 
     wall_ms, event_ms = _event_ms(step, steps, warmup)
     # Hot-cache variant (one layer over and over) for the record.
@@ -113,6 +114,27 @@ def bench_quant_pack(device, steps, warmup, layers):
         "chunks": len(plan.chunks),
         "work": (placement, infos, work, metadata, payloads),
     }
+
+
+def bench_other_shares(device):
+    """The same launch on two other shares: the
+    largest rank share of the Llama bucket (rank 6: rows of `down`, in_dim
+    14336) and rank 0 of the DeepSeek-V3 expert bucket (stacked w1 rows)."""
+    from flex_shard_amd.testing import DEEPSEEK_V3_EXPERTS
+
+    out = {}
+    for name, kwargs, steps in (
+        ("llama3_8b_rank6", dict(layers=8, rank=6), 200),
+        ("deepseek_v3_experts_rank0", dict(layers=2, rank=0, spec=DEEPSEEK_V3_EXPERTS, std=0.006), 40),
+    ):
+        q = bench_quant_pack(device, steps, 10, **kwargs)
+        q.pop("work")
+        us = q["event_ms"] / steps * 1e3
+        out[name] = {"elems": q["elems"], "chunks": q["chunks"], "algorithmic_bytes": q["algo_bytes"],
+                     "us_per_launch": us, "GBps": q["algo_bytes"] / us / 1e3,
+                     "frac_of_hbm_peak": q["algo_bytes"] / us / 1e3 / HBM_PEAK_GBPS}
+        torch.cuda.empty_cache()
+    return out
 
 
 def check_against_oracle(placement, infos, work, metadata, payloads):
@@ -340,6 +362,11 @@ def main() -> None:
     torch.cuda.empty_cache()
     if not args.skip_secondary:
         secondary = {}
+        secondary["quantize_pack_other_shares"] = {
+            name: {k: (round(v, 4) if isinstance(v, float) else v) for k, v in d.items()}
+            for name, d in bench_other_shares(device).items()
+        }
+        torch.cuda.empty_cache()
         secondary["unpack_gathered_layout"] = {k: round(v, 3) if isinstance(v, float) else v
                                                for k, v in bench_unpack(device, placement, infos).items()}
         torch.cuda.empty_cache()
