@@ -19,72 +19,10 @@
 // whose dimensions are multiples of the tile.  Global->register->LDS double
 // buffering with one barrier per k-tile; LDS rows padded by 16 bytes so the
 // 64 lanes of a ds_read_b128 hit distinct banks.
-#include "common.hpp"
-
-#include <type_traits>
+#include "mfma_tiles.hpp"
 
 namespace fsh {
 namespace {
-
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-
-struct GemmParams {
-  const uint16_t* A;
-  const uint16_t* B;
-  const uint16_t* D;
-  uint16_t* C;
-  uint16_t* Ct;
-  int64_t M, N, K;
-  int64_t lda, ldb, ldd, ldc, ldct;
-  int64_t sA, sB, sD, sC, sCt;
-  float alpha, beta;
-  int32_t tiles_m, tiles_n;
-  int32_t symmetric;      // only tiles with tm <= tn are computed; the others are mirrored
-  int32_t tiles_per_matrix;
-  int64_t work_items;     // tiles_per_matrix * batch
-  int64_t items_per_xcd;  // ceil(work_items / 8); the grid has 8 * items_per_xcd workgroups
-};
-
-constexpr int kXcds = 8;         // accelerator dies, each with its own L2
-constexpr int kGroupTilesM = 4;  // tile rows walked together
-
-// Workgroup id -> (batch, tile row, tile column).  Workgroups are handed to
-// the 8 XCDs round-robin by id, and an XCD holds 32 of the large-tile
-// workgroups at a time (one per CU), so XCD x is given the contiguous run
-// [x, x+1) * items_per_xcd of an ordering in which 32 neighbours form a 4 x 8
-// patch of tiles of one matrix: its L2 then serves 12 distinct operand panels
-// per k-tile instead of 33.  Returns false for the padding ids at the end of
-// an XCD's run.
-__device__ inline bool tile_of_workgroup(const GemmParams& p, int64_t* batch, int* tm, int* tn) {
-  const int64_t id = blockIdx.x;
-  const int64_t slot = id / kXcds;
-  const int64_t item = (id % kXcds) * p.items_per_xcd + slot;
-  if (item >= p.work_items) return false;
-  const int tiles = p.tiles_per_matrix;
-  *batch = item / tiles;
-  int t = static_cast<int>(item % tiles);
-  if (p.symmetric) {
-    // Upper triangle row by row: row r holds columns r .. tiles_n-1.  One
-    // matrix's triangle (36 tiles of a 2048^2 result) is about what an XCD
-    // holds at a time, and it needs only the 8 row panels of the operand.
-    int r = 0;
-    for (int len = p.tiles_n; t >= len; --len) {
-      t -= len;
-      ++r;
-    }
-    *tm = r;
-    *tn = r + t;
-    return true;
-  }
-  const int group_span = kGroupTilesM * p.tiles_n;
-  const int first_m = (t / group_span) * kGroupTilesM;
-  const int rows = min(p.tiles_m - first_m, kGroupTilesM);
-  const int within = t % group_span;
-  *tm = first_m + within % rows;
-  *tn = within / rows;
-  return true;
-}
 
 // Tile configuration of one GEMM kernel instantiation.
 //   BM x BN block tile, BK k-tile, WM x WN wavefronts, each wave owns a
@@ -268,118 +206,6 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_nt_kernel(const GemmParams
   }
 }
 
-// Epilogue of the whole-tile kernels, staged through LDS (free once the last
-// k-tile's barrier has passed; every wave uses a private region, but the
-// phases are still separated by workgroup barriers).
-//
-// The accumulate is issued as mfma(B, A), so accumulator r of block (i, j)
-// belongs to output row m = lane%32 and column n = 8*(r/4) + 4*(lane/32) + r%4
-// of the block.  In that layout a store instruction would touch 32 rows with
-// 16 bytes each, and the transposed output would leave as 2-byte stores.
-// Instead:
-//   1. finals = bf16(alpha*acc + beta*D) are computed in registers (D is read
-//      in accumulator layout, 16 loads in flight per 32-row block) and written
-//      to LDS as [row][col];
-//   2. the wave reads its region back row-wise and stores C as 16 bytes per
-//      lane, 256 contiguous bytes per row;
-//   3. for a transposed (or mirrored) output the finals are written again as
-//      [col][row] and leave the same way.
-// The LDS row pitch is the row plus 8 bytes: 8-byte writes of 16 lanes then
-// cover all 32 banks, and so do the row-wise 8-byte reads of a half-wave.
-template <typename Cfg>
-struct WholeTileEpilogue {
-  static constexpr int kPitch = Cfg::kWaveN * 2 + 8;   // bytes, [row][col] staging
-  static constexpr int kPitchT = Cfg::kWaveM * 2 + 8;  // bytes, [col][row] staging
-  static constexpr int kRegion =
-      (Cfg::kWaveM * kPitch > Cfg::kWaveN * kPitchT) ? Cfg::kWaveM * kPitch : Cfg::kWaveN * kPitchT;
-  static constexpr int kLdsBytes = Cfg::WM * Cfg::WN * kRegion;
-};
-
-// Stores a [rows][row_bytes] bf16 image held in LDS (pitch bytes apart) to
-// global rows `ld` elements apart, 16 bytes per lane.
-template <int kRows, int kRowBytes, int kPitch>
-__device__ inline void store_staged_rows(const uint8_t* region, uint16_t* dst, int64_t ld, int lane) {
-  constexpr int kLanesPerRow = kRowBytes / 16;
-  constexpr int kRowsPerPass = 64 / kLanesPerRow;
-  static_assert(kRowBytes % 16 == 0 && 64 % kLanesPerRow == 0 && kRows % kRowsPerPass == 0, "staged store shape");
-  const int r0 = lane / kLanesPerRow, chunk = lane % kLanesPerRow;
-#pragma unroll
-  for (int pass = 0; pass < kRows / kRowsPerPass; ++pass) {
-    const int r = pass * kRowsPerPass + r0;
-    const uint8_t* src = region + r * kPitch + chunk * 16;
-    const u32x2 lo = *reinterpret_cast<const u32x2*>(src);
-    const u32x2 hi = *reinterpret_cast<const u32x2*>(src + 8);
-    *reinterpret_cast<u32x4*>(dst + r * ld + chunk * 8) = u32x4{lo.x, lo.y, hi.x, hi.y};
-  }
-}
-
-template <typename Cfg>
-__device__ inline void store_whole_tile(const GemmParams& p, int64_t batch, int64_t m0, int64_t n0, int wm, int wn,
-                                        int lane, bool mirror, const f32x16 (&acc)[Cfg::TM][Cfg::TN],
-                                        uint8_t* lds) {
-  using Epi = WholeTileEpilogue<Cfg>;
-  constexpr int TM = Cfg::TM, TN = Cfg::TN;
-  const uint16_t* D = p.D ? p.D + batch * p.sD : nullptr;
-  uint16_t* C = p.C + batch * p.sC;
-  // A symmetric product mirrors its off-diagonal tiles into the lower triangle.
-  uint16_t* Ct = mirror ? C : (p.Ct ? p.Ct + batch * p.sCt : nullptr);
-  const int64_t ldct = mirror ? p.ldc : p.ldct;
-  const int64_t wave_row = m0 + wm * Cfg::kWaveM, wave_col = n0 + wn * Cfg::kWaveN;
-  uint8_t* region = lds + (wm * Cfg::WN + wn) * Epi::kRegion;
-  const int r_lane = lane & 31, h = lane >> 5;
-
-  uint32_t fin[TM][TN][4][2];  // packed bf16 pairs of the finals, accumulator layout
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    u32x2 draw[TN][4];
-    if (D != nullptr) {
-      const uint16_t* drow = D + (wave_row + i * 32 + r_lane) * p.ldd + wave_col + 4 * h;
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int b = 0; b < 4; ++b) draw[j][b] = *reinterpret_cast<const u32x2*>(drow + j * 32 + 8 * b);
-    }
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        float v[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) v[t] = p.alpha * acc[i][j][4 * b + t];
-        if (D != nullptr) {
-          v[0] += p.beta * u32_as_f32(draw[j][b].x << 16);
-          v[1] += p.beta * u32_as_f32(draw[j][b].x & 0xFFFF0000u);
-          v[2] += p.beta * u32_as_f32(draw[j][b].y << 16);
-          v[3] += p.beta * u32_as_f32(draw[j][b].y & 0xFFFF0000u);
-        }
-        fin[i][j][b][0] = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
-        fin[i][j][b][1] = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
-        *reinterpret_cast<u32x2*>(region + (i * 32 + r_lane) * Epi::kPitch + (j * 32 + 8 * b + 4 * h) * 2) =
-            u32x2{fin[i][j][b][0], fin[i][j][b][1]};
-      }
-  }
-  __syncthreads();
-  store_staged_rows<Cfg::kWaveM, Cfg::kWaveN * 2, Epi::kPitch>(region, C + wave_row * p.ldc + wave_col, p.ldc, lane);
-  if (Ct == nullptr) return;  // uniform over the workgroup
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int b = 0; b < 4; ++b)
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const uint32_t pair = fin[i][j][b][t >> 1];
-          *reinterpret_cast<uint16_t*>(region + (j * 32 + 8 * b + 4 * h + t) * Epi::kPitchT + (i * 32 + r_lane) * 2) =
-              static_cast<uint16_t>((t & 1) ? (pair >> 16) : pair);
-        }
-  __syncthreads();
-  store_staged_rows<Cfg::kWaveN, Cfg::kWaveM * 2, Epi::kPitchT>(region, Ct + wave_col * ldct + wave_row, ldct, lane);
-}
-
-// Scheduling-group masks of __builtin_amdgcn_sched_group_barrier.
-constexpr int kSchedMfma = 0x008, kSchedVmemRead = 0x020, kSchedDsRead = 0x100, kSchedDsWrite = 0x200;
 
 // Interior fast path: M, N multiples of the block tile and K of BK, so there
 // are no predicates, addresses are one per-thread 32-bit offset plus uniform
@@ -547,11 +373,6 @@ struct DmaGemm {
   static constexpr int kLoadsPerOperand = BM / 8 / 4;        // wave-level 1 KB loads per wave: 8
 };
 
-__device__ inline void dma_load_16(uint32_t voffset, const uint8_t* base, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voffset), "s"(base), "s"(lds_addr) : "memory");
-}
-__device__ inline void wait_for_dma_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
 __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const GemmParams p) {
   using Cfg = DmaGemm;
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds_bytes[];
@@ -673,17 +494,6 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   k_tile(ktiles - 1, std::false_type{});
 
   store_whole_tile<Cfg>(p, batch, m0, n0, wm, wn, lane, p.symmetric && tm != tn, acc, lds_bytes);
-}
-
-constexpr int max_int(int a, int b) { return a > b ? a : b; }
-
-template <typename Kernel>
-int reserve_lds(Kernel kernel, int bytes) {
-  if (bytes <= 64 * 1024) return FSH_OK;
-  hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-  if (err != hipSuccess) return fail(FSH_EHIP, "gemm: cannot reserve %d bytes of LDS: %s", bytes, hipGetErrorString(err));
-  return FSH_OK;
 }
 
 template <typename Cfg>
