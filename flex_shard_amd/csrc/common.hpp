@@ -85,6 +85,28 @@ __device__ __forceinline__ float wave_sum_f32(float v) {
   return v;
 }
 
+// ------------------------------------------------- FP8 quantizer arithmetic
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+  u16x2 va = __builtin_bit_cast(u16x2, a);
+  u16x2 vb = __builtin_bit_cast(u16x2, b);
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(va, vb));
+}
+
+// Two floats -> two E4M3FN bytes in the low (hi=false) or high half of `old`.
+__device__ __forceinline__ uint32_t cvt2_fp8(float a, float b, uint32_t old, bool hi) {
+  return hi ? static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, static_cast<int>(old), true))
+            : static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, static_cast<int>(old), false));
+}
+
+// Scale pair of a tile from its amax; identical on every lane.
+__device__ __forceinline__ void tile_scale(float amax, float eps, float& scale, float& recip) {
+  const float floored = (amax < eps) ? eps : amax;  // NaN fails the test and stays
+  scale = static_cast<float>(448.0 / static_cast<double>(floored));
+  recip = 1.0f / scale;
+}
+
 // ------------------------------------------------- cooperative byte movers
 // All threads of the workgroup call these with identical arguments.  The
 // widest vector the relative alignment of src and dst allows is used for the
