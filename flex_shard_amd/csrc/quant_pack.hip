@@ -226,28 +226,28 @@ __device__ void quant_tile_scalar(const QuantChunkDev& ch, int64_t tr, int64_t t
   }
 }
 
-// ALL_BF16_FAST: every chunk is a bf16 shard on the vector path.  That
-// instantiation carries only the 32-dword tile, stays under 64 VGPRs and so
-// keeps 8 workgroups resident per compute unit: the ~1700 tiles of a
-// Llama-sized rank share are then all in flight at once instead of running in
-// two uneven rounds.
-template <bool ALL_BF16_FAST>
+// Zeroes this pad workgroup's 64 KiB slice of the two pad ranges laid end to end.
+__device__ __forceinline__ void zero_pad_slice(uint8_t* payload, const int64_t (&zero_begin)[2],
+                                               const int64_t (&zero_len)[2], int64_t slice) {
+  const int64_t begin = slice * kZeroChunk;
+  const int64_t end = begin + kZeroChunk;
+  int64_t base = 0;
+#pragma unroll
+  for (int z = 0; z < 2; ++z) {
+    const int64_t lo = begin > base ? begin : base;
+    const int64_t limit = base + zero_len[z];
+    const int64_t hi = end < limit ? end : limit;
+    if (lo < hi) zero_bytes(payload + zero_begin[z] + (lo - base), hi - lo, threadIdx.x, kThreads);
+    base = limit;
+  }
+}
+
+// General kernel: any mix of source kinds, block sizes and alignments.
 __global__ __launch_bounds__(kThreads) void quantize_pack_kernel(const QuantParams prm) {
   __shared__ uint32_t lds[4];
   const int64_t bid = blockIdx.x;
   if (bid >= prm.total_tiles) {
-    // Pad workgroups: zero a slice of the two pad ranges laid end to end.
-    const int64_t begin = (bid - prm.total_tiles) * kZeroChunk;
-    const int64_t end = begin + kZeroChunk;
-    int64_t base = 0;
-#pragma unroll
-    for (int z = 0; z < 2; ++z) {
-      const int64_t lo = begin > base ? begin : base;
-      const int64_t limit = base + prm.zero_len[z];
-      const int64_t hi = end < limit ? end : limit;
-      if (lo < hi) zero_bytes(prm.payload + prm.zero_begin[z] + (lo - base), hi - lo, threadIdx.x, kThreads);
-      base = limit;
-    }
+    zero_pad_slice(prm.payload, prm.zero_begin, prm.zero_len, bid - prm.total_tiles);
     return;
   }
   int c = 0;
@@ -256,10 +256,6 @@ __global__ __launch_bounds__(kThreads) void quantize_pack_kernel(const QuantPara
   const int64_t t = bid - ch.tile_begin;
   const int64_t tr = t / ch.tiles_c;
   const int64_t tc = t - tr * ch.tiles_c;
-  if (ALL_BF16_FAST) {
-    quant_tile128_bf16<FSH_SRC_BF16>(ch, tr, tc, prm.payload, prm.eps[FSH_SRC_BF16], lds);
-    return;
-  }
   const float eps = prm.eps[ch.src_kind];
   if (ch.fast) {
     if (ch.src_kind == FSH_SRC_BF16)
@@ -271,6 +267,156 @@ __global__ __launch_bounds__(kThreads) void quantize_pack_kernel(const QuantPara
   } else {
     quant_tile_scalar(ch, tr, tc, prm.block, prm.payload, eps, lds);
   }
+}
+
+// ------------------------------------------------ bf16 kernel (the hot one)
+// Every chunk is a 16-byte-friendly bf16 shard with 128x128 tiles.  All of a
+// rank share's ~1700 workgroups are resident at once and each runs exactly
+// once, so whatever precedes a workgroup's first load is added to the whole
+// launch: the chunk is found with independent scalar loads (one compare per
+// table entry, no dependent chain), its descriptor arrives in one more round
+// trip with pointers already resolved, tile indices are 32-bit, and interior
+// tiles skip every bounds test.  The tile itself is 32 dwords per thread
+// (under 64 VGPRs, 8 workgroups per compute unit).
+struct FastChunk {
+  const uint8_t* src;     // first element of the chunk
+  uint8_t* qdst;          // payload + qdata_offset
+  float* scales;          // payload + scale_offset
+  int64_t src_row_bytes;
+  int32_t rows;
+  int32_t in_dim;
+  int32_t tiles_c;
+  int32_t tile_begin;
+};
+
+// Entry `nchunks` of both tables stands for the pad workgroups that follow
+// the tiles: its first "tile" is the total tile count.  N is 8 for the usual
+// rank share (a handful of parameters: the whole lookup header is then one
+// 32-byte scalar load) and FSH_MAX_QUANT_CHUNKS otherwise.
+template <int N>
+struct QuantFastParams {
+  int32_t next_begin[N];  // first tile of chunk i + 1; INT32_MAX past the pad entry
+  int32_t nchunks;
+  float eps;
+  FastChunk chunks[N + 1];
+  uint8_t* payload;
+  int64_t zero_begin[2];
+  int64_t zero_len[2];
+};
+
+template <bool FULL>
+__device__ __forceinline__ void quant_tile128_fast(const FastChunk& ch, uint32_t tr, uint32_t tc, float eps,
+                                                   uint32_t* lds) {
+  const uint32_t tid = threadIdx.x;
+  const uint32_t g = tid & 15;
+  const uint32_t row0 = tr * 128u + (tid >> 4);
+  const uint32_t col = tc * 128u + g * 8u;
+  const bool col_ok = FULL || col < static_cast<uint32_t>(ch.in_dim);
+  const uint32_t rows = static_cast<uint32_t>(ch.rows);
+  const int64_t src_row_bytes = ch.src_row_bytes;
+  const int64_t dst_row_bytes = ch.in_dim;
+  const uint8_t* sp = ch.src + static_cast<int64_t>(row0) * src_row_bytes + static_cast<int64_t>(col) * 2;
+  uint8_t* dp = ch.qdst + static_cast<int64_t>(row0) * dst_row_bytes + col;
+  float* scale_slot = ch.scales + static_cast<int64_t>(tr) * ch.tiles_c + tc;
+
+  u32x4 v[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    if (FULL) {
+      v[k] = load_stream_u32x4(sp + 16 * k * src_row_bytes);
+    } else {
+      v[k] = u32x4{0, 0, 0, 0};
+      if (col_ok && row0 + 16u * k < rows) v[k] = load_stream_u32x4(sp + 16 * k * src_row_bytes);
+    }
+  }
+
+  // |x| as raw 15-bit magnitudes: integer order equals float order, and any
+  // NaN pattern exceeds infinity, so a NaN in the tile surfaces as a NaN amax.
+  uint32_t m = 0;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    m = pk_max_u16(m, v[k].x & 0x7FFF7FFFu);
+    m = pk_max_u16(m, v[k].y & 0x7FFF7FFFu);
+    m = pk_max_u16(m, v[k].z & 0x7FFF7FFFu);
+    m = pk_max_u16(m, v[k].w & 0x7FFF7FFFu);
+  }
+  const uint32_t lo = m & 0xFFFFu, hi = m >> 16;
+  m = block_max_u32(lo > hi ? lo : hi, lds);
+
+  float scale, recip;
+  tile_scale(bf16_bits_to_f32(m), eps, scale, recip);
+  if (tid == 0) *scale_slot = recip;
+
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    if (FULL || (col_ok && row0 + 16u * k < rows)) {
+      const uint32_t d[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+      uint32_t w[2] = {0, 0};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float e0 = u32_as_f32(d[j] << 16) * scale;
+        const float e1 = u32_as_f32(d[j] & 0xFFFF0000u) * scale;
+        w[j >> 1] = cvt2_fp8(e0, e1, w[j >> 1], (j & 1) != 0);
+      }
+      store_stream_u32x2(dp + 16 * k * dst_row_bytes, w[0], w[1]);
+    }
+  }
+}
+
+template <int N>
+__global__ __launch_bounds__(kThreads) void quantize_pack_bf16_kernel(const QuantFastParams<N> prm) {
+  __shared__ uint32_t lds[4];
+  const int32_t bid = static_cast<int32_t>(blockIdx.x);
+  int c = 0;
+#pragma unroll
+  for (int i = 0; i < N; ++i) c += bid >= prm.next_begin[i] ? 1 : 0;
+  if (c >= prm.nchunks) {
+    zero_pad_slice(prm.payload, prm.zero_begin, prm.zero_len, bid - prm.chunks[c].tile_begin);
+    return;
+  }
+  const FastChunk ch = prm.chunks[c];
+  const uint32_t t = static_cast<uint32_t>(bid - ch.tile_begin);
+  const uint32_t tr = t / static_cast<uint32_t>(ch.tiles_c);
+  const uint32_t tc = t - tr * static_cast<uint32_t>(ch.tiles_c);
+  const bool full = (tr + 1) * 128u <= static_cast<uint32_t>(ch.rows) &&
+                    (tc + 1) * 128u <= static_cast<uint32_t>(ch.in_dim);
+  if (full)
+    quant_tile128_fast<true>(ch, tr, tc, prm.eps, lds);
+  else
+    quant_tile128_fast<false>(ch, tr, tc, prm.eps, lds);
+}
+
+template <int N>
+void launch_bf16_kernel(const QuantParams& prm, int64_t tiles, int64_t grid, hipStream_t stream) {
+  QuantFastParams<N> fast;
+  memset(&fast, 0, sizeof(fast));
+  const int nchunks = prm.nchunks;
+  for (int i = 0; i < N; ++i) fast.next_begin[i] = INT32_MAX;
+  for (int i = 0; i < nchunks; ++i) {
+    const QuantChunkDev& in = prm.chunks[i];
+    FastChunk& out = fast.chunks[i];
+    out.src = in.src;
+    out.qdst = prm.payload + in.qdata_offset;
+    out.scales = reinterpret_cast<float*>(prm.payload + in.scale_offset);
+    out.src_row_bytes = in.src_row_stride * 2;
+    out.rows = static_cast<int32_t>(in.rows);
+    out.in_dim = static_cast<int32_t>(in.in_dim);
+    out.tiles_c = in.tiles_c;
+    out.tile_begin = static_cast<int32_t>(in.tile_begin);
+    if (i > 0) fast.next_begin[i - 1] = out.tile_begin;
+  }
+  fast.chunks[nchunks].tile_begin = static_cast<int32_t>(tiles);
+  fast.chunks[nchunks].tiles_c = 1;
+  if (nchunks > 0) fast.next_begin[nchunks - 1] = static_cast<int32_t>(tiles);
+  fast.payload = prm.payload;
+  for (int z = 0; z < 2; ++z) {
+    fast.zero_begin[z] = prm.zero_begin[z];
+    fast.zero_len[z] = prm.zero_len[z];
+  }
+  fast.eps = prm.eps[FSH_SRC_BF16];
+  fast.nchunks = nchunks;
+  hipLaunchKernelGGL(quantize_pack_bf16_kernel<N>, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), 0, stream,
+                     fast);
 }
 
 float bf16_round_host(float f) {
@@ -346,7 +492,8 @@ FSH_API int fsh_quantize_pack(const fsh_quant_chunk* chunks, int32_t nchunks, vo
     out.src_kind = in.src_kind;
     out.fast = block == 128 && aligned(in.src_dev, 16) && (in.src_row_stride * elem) % 16 == 0 &&
                in.in_dim % 8 == 0 && in.qdata_offset % 8 == 0;
-    all_bf16_fast = all_bf16_fast && out.fast && in.src_kind == FSH_SRC_BF16;
+    all_bf16_fast = all_bf16_fast && out.fast && in.src_kind == FSH_SRC_BF16 && in.rows < (1LL << 30) &&
+                    in.in_dim < (1LL << 30);
     tiles += tiles_r * tiles_c;
   }
   prm.total_tiles = tiles;
@@ -359,11 +506,14 @@ FSH_API int fsh_quantize_pack(const fsh_quant_chunk* chunks, int32_t nchunks, vo
   const int64_t grid = tiles + ceil_div(zero_total, kZeroChunk);
   if (grid == 0) return FSH_OK;
   if (grid > 0x7FFFFFFFLL) return fail(FSH_ENOTSUP, "fsh_quantize_pack: %lld workgroups exceed the grid limit", (long long)grid);
-  if (all_bf16_fast)
-    hipLaunchKernelGGL(quantize_pack_kernel<true>, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), 0,
+  if (all_bf16_fast) {
+    if (nchunks < 8)
+      launch_bf16_kernel<8>(prm, tiles, grid, static_cast<hipStream_t>(stream));
+    else
+      launch_bf16_kernel<FSH_MAX_QUANT_CHUNKS>(prm, tiles, grid, static_cast<hipStream_t>(stream));
+  } else {
+    hipLaunchKernelGGL(quantize_pack_kernel, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), 0,
                        static_cast<hipStream_t>(stream), prm);
-  else
-    hipLaunchKernelGGL(quantize_pack_kernel<false>, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), 0,
-                       static_cast<hipStream_t>(stream), prm);
+  }
   return check_launch("fsh_quantize_pack");
 }
