@@ -85,6 +85,22 @@ class GemmDesc(Structure):
     ]
 
 
+class NsProblem(Structure):
+    """``fsh_ns_problem``."""
+
+    _fields_ = [
+        ("x_dev", c_void_p),
+        ("batch", c_int64),
+        ("rows", c_int64),
+        ("cols", c_int64),
+        ("workspace_dev", c_void_p),
+        ("workspace_nbytes", c_int64),
+    ]
+
+
+MAX_NS_PROBLEMS = 16
+
+
 # name -> (restype, argtypes); every symbol include/flexshard_hip.h declares.
 SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "fsh_version": (c_int32, []),
@@ -110,7 +126,11 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         c_int,
         [c_void_p, c_int64, c_int64, c_int64, c_float, c_float, c_float, c_int32, c_float, c_void_p, c_int64, c_void_p],
     ),
+    "fsh_newton_schulz_multi": (
+        c_int, [POINTER(NsProblem), c_int32, c_float, c_float, c_float, c_int32, c_float, c_void_p],
+    ),
     "fsh_gemm_bf16_nt": (c_int, [POINTER(GemmDesc), c_void_p]),
+    "fsh_gemm_bf16_nt_group": (c_int, [POINTER(GemmDesc), c_int32, c_void_p]),
     "fsh_muon_prepare": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_float, c_float, c_int32, c_void_p]),
     "fsh_muon_apply": (c_int, [c_void_p, c_void_p, c_int64, c_float, c_float, c_float, c_void_p]),
 }

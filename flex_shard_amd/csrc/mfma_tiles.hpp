@@ -27,6 +27,25 @@ struct GemmParams {
   int32_t tiles_per_matrix;
   int64_t work_items;     // tiles_per_matrix * batch
   int64_t items_per_xcd;  // ceil(work_items / 8); the grid has 8 * items_per_xcd workgroups
+#ifdef FSH_TRACE
+  uint64_t* trace;
+#endif
+};
+#ifdef FSH_TRACE
+#define FSH_STAMP(slot) do { if (p.trace && threadIdx.x == 0) p.trace[blockIdx.x * 16 + (slot)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define FSH_STAMP(slot) do {} while (0)
+#endif
+
+// Several problems served by one launch of the large-tile kernel: problem i
+// owns the workgroup ids [first_workgroup[i], first_workgroup[i+1]), each run
+// a multiple of 8 long so that the id -> XCD mapping is the same for all.
+// Workgroups are dispatched in id order, so the host lists the problem with
+// the longest tiles first and the short ones fill the tail of the long ones.
+constexpr int kMaxGemmProblems = 4;
+struct GemmLaunch {
+  GemmParams problem[kMaxGemmProblems];
+  int32_t first_workgroup[kMaxGemmProblems];  // INT32_MAX past the last problem
 };
 
 constexpr int kXcds = 8;         // accelerator dies, each with its own L2
@@ -39,8 +58,7 @@ constexpr int kGroupTilesM = 4;  // tile rows walked together
 // patch of tiles of one matrix: its L2 then serves 12 distinct operand panels
 // per k-tile instead of 33.  Returns false for the padding ids at the end of
 // an XCD's run.
-__device__ inline bool tile_of_workgroup(const GemmParams& p, int64_t* batch, int* tm, int* tn) {
-  const int64_t id = blockIdx.x;
+__device__ inline bool tile_of_workgroup(const GemmParams& p, int64_t id, int64_t* batch, int* tm, int* tn) {
   const int64_t slot = id / kXcds;
   const int64_t item = (id % kXcds) * p.items_per_xcd + slot;
   if (item >= p.work_items) return false;
@@ -78,13 +96,13 @@ __device__ inline bool tile_of_workgroup(const GemmParams& p, int64_t* batch, in
 // of the block.  In that layout a store instruction would touch 32 rows with
 // 16 bytes each, and the transposed output would leave as 2-byte stores.
 // Instead:
-//   1. finals = bf16(alpha*acc + beta*D) are computed in registers (D is read
-//      in accumulator layout, 16 loads in flight per 32-row block) and written
-//      to LDS as [row][col];
+//   1. D is loaded row-wise (16 bytes per lane) into the staging region; the
+//      finals = bf16(alpha*acc + beta*D) are computed in registers and written
+//      to LDS as [row][col], each over the D value it used;
 //   2. the wave reads its region back row-wise and stores C as 16 bytes per
 //      lane, 256 contiguous bytes per row;
-//   3. for a transposed (or mirrored) output the finals are written again as
-//      [col][row] and leave the same way.
+//   3. for a transposed (or mirrored) output the finals are read back in
+//      accumulator layout, written again as [col][row] and leave the same way.
 // The LDS row pitch is the row plus 8 bytes: 8-byte writes of 16 lanes then
 // cover all 32 banks, and so do the row-wise 8-byte reads of a half-wave.
 template <typename Cfg>
@@ -114,13 +132,61 @@ __device__ inline void store_staged_rows(const uint8_t* region, uint16_t* dst, i
   }
 }
 
+// Two floats -> packed bf16 pair (low half = first), round to nearest even:
+// one v_cvt_pk_bf16_f32 on gfx950.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
+// Half of a wave's D tile (its upper or lower kWaveM/2 rows), loaded the way
+// C leaves: 16 bytes per lane, 256 contiguous bytes per row (in accumulator
+// layout a load instruction would touch 32 rows with 16 bytes each).  Both
+// halves are requested when the epilogue starts; the lower one lands while
+// the upper one is being used.  (Requesting a half before the last k-tile
+// was tried: with 256 accumulators live the extra 64 registers spill.)
+template <typename Cfg>
+struct DRows {
+  static constexpr int kLanesPerRow = Cfg::kWaveN * 2 / 16, kRowsPerPass = 64 / kLanesPerRow;
+  static constexpr int kPasses = Cfg::kWaveM / 2 / kRowsPerPass;
+  u32x4 t[kPasses];
+};
+
+template <typename Cfg>
+__device__ __forceinline__ void load_d_rows(const GemmParams& p, int64_t batch, int64_t m0, int64_t n0, int wm, int wn,
+                                            int lane, int half, DRows<Cfg>& rows) {
+  using R = DRows<Cfg>;
+  const int r0 = half * (Cfg::kWaveM / 2) + lane / R::kLanesPerRow, chunk = lane % R::kLanesPerRow;
+  const uint16_t* dsrc =
+      p.D + batch * p.sD + (m0 + wm * Cfg::kWaveM + r0) * p.ldd + n0 + wn * Cfg::kWaveN + chunk * 8;
+#pragma unroll
+  for (int q = 0; q < R::kPasses; ++q)
+    rows.t[q] = *reinterpret_cast<const u32x4*>(dsrc + static_cast<int64_t>(q) * R::kRowsPerPass * p.ldd);
+}
+
+template <typename Cfg, int kPitch>
+__device__ __forceinline__ void stage_d_rows(uint8_t* region, int lane, int half, const DRows<Cfg>& rows) {
+  using R = DRows<Cfg>;
+  const int r0 = half * (Cfg::kWaveM / 2) + lane / R::kLanesPerRow, chunk = lane % R::kLanesPerRow;
+  uint8_t* ddst = region + r0 * kPitch + chunk * 16;
+#pragma unroll
+  for (int q = 0; q < R::kPasses; ++q) {
+    uint8_t* d = ddst + q * R::kRowsPerPass * kPitch;
+    *reinterpret_cast<u32x2*>(d) = u32x2{rows.t[q].x, rows.t[q].y};
+    *reinterpret_cast<u32x2*>(d + 8) = u32x2{rows.t[q].z, rows.t[q].w};
+  }
+}
+
 template <typename Cfg>
 __device__ inline void store_whole_tile(const GemmParams& p, int64_t batch, int64_t m0, int64_t n0, int wm, int wn,
                                         int lane, bool mirror, const f32x16 (&acc)[Cfg::TM][Cfg::TN],
                                         uint8_t* lds) {
   using Epi = WholeTileEpilogue<Cfg>;
   constexpr int TM = Cfg::TM, TN = Cfg::TN;
-  const uint16_t* D = p.D ? p.D + batch * p.sD : nullptr;
+  static_assert(TM % 2 == 0, "the D tile is handled in two halves of TM/2 blocks");
+  const bool has_d = p.D != nullptr;
   uint16_t* C = p.C + batch * p.sC;
   // A symmetric product mirrors its off-diagonal tiles into the lower triangle.
   uint16_t* Ct = mirror ? C : (p.Ct ? p.Ct + batch * p.sCt : nullptr);
@@ -129,16 +195,32 @@ __device__ inline void store_whole_tile(const GemmParams& p, int64_t batch, int6
   uint8_t* region = lds + (wm * Cfg::WN + wn) * Epi::kRegion;
   const int r_lane = lane & 31, h = lane >> 5;
 
-  uint32_t fin[TM][TN][4][2];  // packed bf16 pairs of the finals, accumulator layout
+  // D goes to the wave's staging region row-wise and is read back in
+  // accumulator layout; each final then replaces the D value it used.
+  DRows<Cfg> upper, lower;
+  if (has_d) {
+    load_d_rows<Cfg>(p, batch, m0, n0, wm, wn, lane, 0, upper);
+    load_d_rows<Cfg>(p, batch, m0, n0, wm, wn, lane, 1, lower);
+    stage_d_rows<Cfg, Epi::kPitch>(region, lane, 0, upper);
+  }
+  FSH_STAMP(8);
+
+  // finals = bf16(fma(beta, D, alpha*acc)): one rounding of the scaled
+  // accumulator, one of the sum, as a BLAS epilogue does.
+  const bool unit_alpha = p.alpha == 1.0f;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    u32x2 draw[TN][4];
-    if (D != nullptr) {
-      const uint16_t* drow = D + (wave_row + i * 32 + r_lane) * p.ldd + wave_col + 4 * h;
+    if (has_d && i == TM / 2) stage_d_rows<Cfg, Epi::kPitch>(region, lane, 1, lower);
+    // All of a 32-row block's D reads are issued before its first write: the
+    // compiler cannot move a read above a write to the same region.
+    u32x2 dv[TN][4];
+    if (has_d) {
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int b = 0; b < 4; ++b) draw[j][b] = *reinterpret_cast<const u32x2*>(drow + j * 32 + 8 * b);
+        for (int b = 0; b < 4; ++b)
+          dv[j][b] = *reinterpret_cast<const u32x2*>(region + (i * 32 + r_lane) * Epi::kPitch +
+                                                     (j * 32 + 8 * b + 4 * h) * 2);
     }
 #pragma unroll
     for (int j = 0; j < TN; ++j)
@@ -146,23 +228,36 @@ __device__ inline void store_whole_tile(const GemmParams& p, int64_t batch, int6
       for (int b = 0; b < 4; ++b) {
         float v[4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) v[t] = p.alpha * acc[i][j][4 * b + t];
-        if (D != nullptr) {
-          v[0] += p.beta * u32_as_f32(draw[j][b].x << 16);
-          v[1] += p.beta * u32_as_f32(draw[j][b].x & 0xFFFF0000u);
-          v[2] += p.beta * u32_as_f32(draw[j][b].y << 16);
-          v[3] += p.beta * u32_as_f32(draw[j][b].y & 0xFFFF0000u);
+        for (int t = 0; t < 4; ++t) v[t] = unit_alpha ? acc[i][j][4 * b + t] : p.alpha * acc[i][j][4 * b + t];
+        if (has_d) {
+          v[0] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].x << 16), v[0]);
+          v[1] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].x & 0xFFFF0000u), v[1]);
+          v[2] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].y << 16), v[2]);
+          v[3] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].y & 0xFFFF0000u), v[3]);
         }
-        fin[i][j][b][0] = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
-        fin[i][j][b][1] = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
         *reinterpret_cast<u32x2*>(region + (i * 32 + r_lane) * Epi::kPitch + (j * 32 + 8 * b + 4 * h) * 2) =
-            u32x2{fin[i][j][b][0], fin[i][j][b][1]};
+            u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
       }
   }
+  FSH_STAMP(9);
   __syncthreads();
   store_staged_rows<Cfg::kWaveM, Cfg::kWaveN * 2, Epi::kPitch>(region, C + wave_row * p.ldc + wave_col, p.ldc, lane);
+  FSH_STAMP(10);
   if (Ct == nullptr) return;  // uniform over the workgroup
   __syncthreads();
+  FSH_STAMP(11);
+  // The finals come back from the [row][col] image in accumulator layout
+  // (all reads before the first write: the transposed image reuses the
+  // region) and are written again as [col][row].
+  u32x2 fin[TM][TN][4];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+        fin[i][j][b] = *reinterpret_cast<const u32x2*>(region + (i * 32 + r_lane) * Epi::kPitch +
+                                                       (j * 32 + 8 * b + 4 * h) * 2);
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -171,10 +266,11 @@ __device__ inline void store_whole_tile(const GemmParams& p, int64_t batch, int6
       for (int b = 0; b < 4; ++b)
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          const uint32_t pair = fin[i][j][b][t >> 1];
+          const uint32_t pair = (t >> 1) ? fin[i][j][b].y : fin[i][j][b].x;
           *reinterpret_cast<uint16_t*>(region + (j * 32 + 8 * b + 4 * h + t) * Epi::kPitchT + (i * 32 + r_lane) * 2) =
               static_cast<uint16_t>((t & 1) ? (pair >> 16) : pair);
         }
+  FSH_STAMP(12);
   __syncthreads();
   store_staged_rows<Cfg::kWaveN, Cfg::kWaveM * 2, Epi::kPitchT>(region, Ct + wave_col * ldct + wave_row, ldct, lane);
 }

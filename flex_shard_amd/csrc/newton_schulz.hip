@@ -62,7 +62,7 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_nt_kernel(const GemmParams
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
   int64_t batch;
   int tm, tn;
-  if (!tile_of_workgroup(p, &batch, &tm, &tn)) return;  // whole workgroup, before any barrier
+  if (!tile_of_workgroup(p, blockIdx.x, &batch, &tm, &tn)) return;  // whole workgroup, before any barrier
   const int64_t m0 = static_cast<int64_t>(tm) * BM;
   const int64_t n0 = static_cast<int64_t>(tn) * BN;
 
@@ -227,7 +227,7 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_nt_interior_kernel(const G
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
   int64_t batch;
   int tm, tn;
-  if (!tile_of_workgroup(p, &batch, &tm, &tn)) return;  // whole workgroup, before any barrier
+  if (!tile_of_workgroup(p, blockIdx.x, &batch, &tm, &tn)) return;  // whole workgroup, before any barrier
   const int64_t m0 = static_cast<int64_t>(tm) * BM;
   const int64_t n0 = static_cast<int64_t>(tn) * BN;
 
@@ -373,8 +373,14 @@ struct DmaGemm {
   static constexpr int kLoadsPerOperand = BM / 8 / 4;        // wave-level 1 KB loads per wave: 8
 };
 
-__global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const GemmParams p) {
+__global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const GemmLaunch launch) {
   using Cfg = DmaGemm;
+  int which = 0;
+#pragma unroll
+  for (int i = 1; i < kMaxGemmProblems; ++i) which += static_cast<int>(blockIdx.x) >= launch.first_workgroup[i] ? 1 : 0;
+  const GemmParams& p = launch.problem[which];
+  const int64_t local_id = static_cast<int64_t>(blockIdx.x) - launch.first_workgroup[which];
+  FSH_STAMP(0);
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds_bytes[];
   constexpr int TM = Cfg::TM, TN = Cfg::TN, KS = Cfg::KS;
 
@@ -384,7 +390,7 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
   int64_t batch;
   int tm, tn;
-  if (!tile_of_workgroup(p, &batch, &tm, &tn)) return;  // whole workgroup, before any barrier
+  if (!tile_of_workgroup(p, local_id, &batch, &tm, &tn)) return;  // whole workgroup, before any barrier
   const int64_t m0 = static_cast<int64_t>(tm) * Cfg::BM;
   const int64_t n0 = static_cast<int64_t>(tn) * Cfg::BN;
   const uint8_t* Ab = reinterpret_cast<const uint8_t*>(p.A + batch * p.sA + m0 * p.lda);
@@ -453,10 +459,12 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
     }
   };
 
+  FSH_STAMP(1);
   issue_tile_load(0, 0, 0, Cfg::kLoadsPerOperand);
   wait_for_dma_loads();
   __syncthreads();
   read_frags(0, 0, 0);
+  FSH_STAMP(2);
 
   auto k_tile = [&](int64_t kt, auto more_tag) {
     constexpr bool more = decltype(more_tag)::value;
@@ -492,12 +500,34 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   };
   for (int64_t kt = 0; kt + 1 < ktiles; ++kt) k_tile(kt, std::true_type{});
   k_tile(ktiles - 1, std::false_type{});
+  FSH_STAMP(3);
 
   store_whole_tile<Cfg>(p, batch, m0, n0, wm, wn, lane, p.symmetric && tm != tn, acc, lds_bytes);
+  FSH_STAMP(4);
+#ifdef FSH_TRACE
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  FSH_STAMP(5);
+  if (p.trace && threadIdx.x == 0) {
+    uint32_t hwid;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+    uint32_t xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    p.trace[blockIdx.x * 16 + 6] = (static_cast<uint64_t>(xcc) << 32) | hwid;
+  }
+#endif
 }
 
+// A validated problem with its kernel chosen and its tile schedule filled in.
+enum GemmKernelKind { kKernelDma, kKernelInteriorBig, kKernelInteriorSmall, kKernelEdgeBig, kKernelEdgeSmall };
+struct PlannedGemm {
+  GemmParams p;
+  GemmKernelKind kind;
+  int64_t workgroups;
+};
+
 template <typename Cfg>
-int launch_gemm_cfg(GemmParams& p, int64_t batch, hipStream_t stream) {
+int plan_gemm_cfg(PlannedGemm* plan, int64_t batch) {
+  GemmParams& p = plan->p;
   p.tiles_m = static_cast<int32_t>(ceil_div(p.M, Cfg::BM));
   p.tiles_n = static_cast<int32_t>(ceil_div(p.N, Cfg::BN));
   const int64_t tiles = p.symmetric ? static_cast<int64_t>(p.tiles_n) * (p.tiles_n + 1) / 2
@@ -505,46 +535,25 @@ int launch_gemm_cfg(GemmParams& p, int64_t batch, hipStream_t stream) {
   p.tiles_per_matrix = static_cast<int32_t>(tiles);
   p.work_items = tiles * batch;
   p.items_per_xcd = ceil_div(p.work_items, static_cast<int64_t>(kXcds));
-  if (tiles > 0x3FFFFFFFLL || p.items_per_xcd * kXcds > 0x7FFFFFFFLL)
+  if (tiles > 0x3FFFFFFFLL || p.items_per_xcd * kXcds > 0x3FFFFFFFLL)
     return fail(FSH_ENOTSUP, "gemm: too many tiles");
-  const dim3 grid(static_cast<uint32_t>(p.items_per_xcd * kXcds)), block(Cfg::kThreads);
-  // Interior path: whole tiles, 16-byte stores in the epilogue, 32-bit tile spans.
+  plan->workgroups = p.items_per_xcd * kXcds;
+  constexpr bool big = std::is_same<Cfg, BigCfg>::value;
+  // Interior path: whole tiles, 16-byte accesses in the epilogue, 32-bit tile spans.
   const bool interior =
       p.M % Cfg::BM == 0 && p.N % Cfg::BN == 0 && p.K % Cfg::BK == 0 && p.ldc % 8 == 0 &&
       (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 && p.sC % 8 == 0 &&
       (p.Ct == nullptr || (p.ldct % 8 == 0 && (reinterpret_cast<uintptr_t>(p.Ct) & 15) == 0 && p.sCt % 8 == 0)) &&
-      (p.D == nullptr || (p.ldd % 4 == 0 && (reinterpret_cast<uintptr_t>(p.D) & 7) == 0 && p.sD % 4 == 0)) &&
+      (p.D == nullptr || (p.ldd % 8 == 0 && (reinterpret_cast<uintptr_t>(p.D) & 15) == 0 && p.sD % 8 == 0)) &&
       static_cast<int64_t>(Cfg::BM) * p.lda * 2 < (1LL << 31) && static_cast<int64_t>(Cfg::BN) * p.ldb * 2 < (1LL << 31);
-  if (interior && std::is_same<Cfg, BigCfg>::value) {
-    constexpr int kDmaLds = max_int(DmaGemm::kLoopLdsBytes, WholeTileEpilogue<DmaGemm>::kLdsBytes);
-    static bool reserved_dma = false;  // the attribute is per device function and sticky
-    if (!reserved_dma) {
-      if (int rc = reserve_lds(&gemm_nt_dma_kernel, kDmaLds)) return rc;
-      reserved_dma = true;
-    }
-    hipLaunchKernelGGL(gemm_nt_dma_kernel, grid, block, kDmaLds, stream, p);
-    return check_launch("gemm_nt_dma_kernel");
-  }
-  if (interior) {
-    constexpr int kInteriorLds = max_int(Cfg::kLdsBytes, WholeTileEpilogue<Cfg>::kLdsBytes);
-    static bool reserved = false;
-    if (!reserved) {
-      if (int rc = reserve_lds(&gemm_nt_interior_kernel<Cfg>, kInteriorLds)) return rc;
-      reserved = true;
-    }
-    hipLaunchKernelGGL(gemm_nt_interior_kernel<Cfg>, grid, block, kInteriorLds, stream, p);
-    return check_launch("gemm_nt_interior_kernel");
-  }
-  static bool reserved_edge = false;
-  if (!reserved_edge) {
-    if (int rc = reserve_lds(&gemm_nt_kernel<Cfg>, Cfg::kLdsBytes)) return rc;
-    reserved_edge = true;
-  }
-  hipLaunchKernelGGL(gemm_nt_kernel<Cfg>, grid, block, Cfg::kLdsBytes, stream, p);
-  return check_launch("gemm_nt_kernel");
+  if (interior)
+    plan->kind = big ? kKernelDma : kKernelInteriorSmall;
+  else
+    plan->kind = big ? kKernelEdgeBig : kKernelEdgeSmall;
+  return FSH_OK;
 }
 
-int launch_gemm(const fsh_gemm_desc& d, hipStream_t stream) {
+int plan_gemm(const fsh_gemm_desc& d, PlannedGemm* plan) {
   if (d.m <= 0 || d.n <= 0 || d.k <= 0 || d.batch <= 0)
     return fail(FSH_EINVAL, "gemm: non-positive size (m %lld, n %lld, k %lld, batch %lld)", (long long)d.m,
                 (long long)d.n, (long long)d.k, (long long)d.batch);
@@ -556,7 +565,8 @@ int launch_gemm(const fsh_gemm_desc& d, hipStream_t stream) {
     return fail(FSH_EINVAL, "gemm: leading dimension smaller than the row length");
   if (d.symmetric && (d.m != d.n || d.ct_dev != nullptr))
     return fail(FSH_EINVAL, "gemm: a symmetric product needs m == n and no transposed output");
-  GemmParams p;
+  GemmParams& p = plan->p;
+  memset(&p, 0, sizeof(p));
   p.symmetric = d.symmetric ? 1 : 0;
   p.A = static_cast<const uint16_t*>(d.a_dev);
   p.B = static_cast<const uint16_t*>(d.b_dev);
@@ -567,11 +577,98 @@ int launch_gemm(const fsh_gemm_desc& d, hipStream_t stream) {
   p.lda = d.lda; p.ldb = d.ldb; p.ldd = d.ldd; p.ldc = d.ldc; p.ldct = d.ldct;
   p.sA = d.stride_a; p.sB = d.stride_b; p.sD = d.stride_d; p.sC = d.stride_c; p.sCt = d.stride_ct;
   p.alpha = d.alpha; p.beta = d.beta;
+#ifdef FSH_TRACE
+  if (const char* e = getenv("FSH_GEMM_TRACE")) p.trace = reinterpret_cast<uint64_t*>(strtoull(e, nullptr, 0));
+#endif
   // The big tile pays off once it fills the chip at least once.
   const int64_t big_n = ceil_div(d.n, BigCfg::BN);
   const int64_t big_tiles = (d.symmetric ? big_n * (big_n + 1) / 2 : ceil_div(d.m, BigCfg::BM) * big_n) * d.batch;
-  if (big_tiles >= 192) return launch_gemm_cfg<BigCfg>(p, d.batch, stream);
-  return launch_gemm_cfg<SmallCfg>(p, d.batch, stream);
+  if (big_tiles >= 192) return plan_gemm_cfg<BigCfg>(plan, d.batch);
+  return plan_gemm_cfg<SmallCfg>(plan, d.batch);
+}
+
+template <typename Kernel>
+int launch_single(Kernel kernel, bool* reserved, int lds_bytes, int threads, const PlannedGemm& plan,
+                  hipStream_t stream, const char* name) {
+  if (!*reserved) {  // the attribute is per device function and sticky
+    if (int rc = reserve_lds(kernel, lds_bytes)) return rc;
+    *reserved = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(plan.workgroups)), dim3(threads), lds_bytes, stream, plan.p);
+  return check_launch(name);
+}
+
+// Launches the planned problems in order.  Runs of problems that take the
+// large-tile kernel share launches (up to kMaxGemmProblems each, longest k
+// first): the short tiles of one problem then fill the partly empty last
+// round of another instead of each launch paying its own tail.  The problems
+// of one call must not depend on each other.
+int launch_planned(PlannedGemm* plans, int count, hipStream_t stream) {
+  static bool reserved_dma = false, reserved_small = false, reserved_edge_big = false, reserved_edge_small = false;
+  constexpr int kDmaLds = max_int(DmaGemm::kLoopLdsBytes, WholeTileEpilogue<DmaGemm>::kLdsBytes);
+  int i = 0;
+  while (i < count) {
+    if (plans[i].kind != kKernelDma) {
+      int rc;
+      if (plans[i].kind == kKernelInteriorSmall)
+        rc = launch_single(&gemm_nt_interior_kernel<SmallCfg>, &reserved_small,
+                           max_int(SmallCfg::kLdsBytes, WholeTileEpilogue<SmallCfg>::kLdsBytes), SmallCfg::kThreads,
+                           plans[i], stream, "gemm_nt_interior_kernel");
+      else if (plans[i].kind == kKernelEdgeBig)
+        rc = launch_single(&gemm_nt_kernel<BigCfg>, &reserved_edge_big, BigCfg::kLdsBytes, BigCfg::kThreads, plans[i],
+                           stream, "gemm_nt_kernel");
+      else
+        rc = launch_single(&gemm_nt_kernel<SmallCfg>, &reserved_edge_small, SmallCfg::kLdsBytes, SmallCfg::kThreads,
+                           plans[i], stream, "gemm_nt_kernel");
+      if (rc) return rc;
+      ++i;
+      continue;
+    }
+    int order[kMaxGemmProblems];
+    int n = 0;
+    int64_t total = 0;
+    while (i < count && n < kMaxGemmProblems && plans[i].kind == kKernelDma &&
+           total + plans[i].workgroups <= 0x3FFFFFFFLL) {
+      total += plans[i].workgroups;
+      order[n++] = i++;
+    }
+    for (int a = 1; a < n; ++a)  // insertion sort, longest k first, stable
+      for (int b = a; b > 0 && plans[order[b]].p.K > plans[order[b - 1]].p.K; --b) {
+        const int t = order[b];
+        order[b] = order[b - 1];
+        order[b - 1] = t;
+      }
+    GemmLaunch launch;
+    memset(&launch, 0, sizeof(launch));
+    int64_t first = 0;
+    for (int k = 0; k < kMaxGemmProblems; ++k) {
+      launch.first_workgroup[k] = k < n ? static_cast<int32_t>(first) : INT32_MAX;
+      if (k < n) {
+        launch.problem[k] = plans[order[k]].p;
+        first += plans[order[k]].workgroups;
+      }
+    }
+    if (!reserved_dma) {
+      if (int rc = reserve_lds(&gemm_nt_dma_kernel, kDmaLds)) return rc;
+      reserved_dma = true;
+    }
+    hipLaunchKernelGGL(gemm_nt_dma_kernel, dim3(static_cast<uint32_t>(total)), dim3(DmaGemm::kThreads), kDmaLds,
+                       stream, launch);
+    if (int rc = check_launch("gemm_nt_dma_kernel")) return rc;
+  }
+  return FSH_OK;
+}
+
+int launch_gemms(const fsh_gemm_desc* descs, int count, hipStream_t stream) {
+  constexpr int kChunk = 16;
+  PlannedGemm plans[kChunk];
+  for (int begin = 0; begin < count; begin += kChunk) {
+    const int n = count - begin < kChunk ? count - begin : kChunk;
+    for (int i = 0; i < n; ++i)
+      if (int rc = plan_gemm(descs[begin + i], &plans[i])) return rc;
+    if (int rc = launch_planned(plans, n, stream)) return rc;
+  }
+  return FSH_OK;
 }
 
 // ------------------------------------------------------- Frobenius normalize
@@ -683,7 +780,13 @@ int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
 
 FSH_API int fsh_gemm_bf16_nt(const fsh_gemm_desc* desc, void* stream) {
   if (desc == nullptr) return fsh::fail(FSH_EINVAL, "fsh_gemm_bf16_nt: null descriptor");
-  return fsh::launch_gemm(*desc, static_cast<hipStream_t>(stream));
+  return fsh::launch_gemms(desc, 1, static_cast<hipStream_t>(stream));
+}
+
+FSH_API int fsh_gemm_bf16_nt_group(const fsh_gemm_desc* descs, int32_t count, void* stream) {
+  if (count < 0 || (count > 0 && descs == nullptr))
+    return fsh::fail(FSH_EINVAL, "fsh_gemm_bf16_nt_group: bad descriptor list");
+  return fsh::launch_gemms(descs, count, static_cast<hipStream_t>(stream));
 }
 
 // Workspace layout (bytes, each region 256-aligned):
@@ -700,87 +803,138 @@ FSH_API int64_t fsh_newton_schulz_workspace_bytes(int64_t batch, int64_t rows, i
          align256(batch * kNormBlocksPerMatrix * 4);
 }
 
-FSH_API int fsh_newton_schulz(void* x_dev, int64_t batch, int64_t rows, int64_t cols, float a, float b,
-                              float c, int32_t steps, float eps, void* workspace_dev,
-                              int64_t workspace_nbytes, void* stream_) {
-  using namespace fsh;
-  if (batch <= 0 || rows <= 0 || cols <= 0 || steps < 0)
-    return fail(FSH_EINVAL, "fsh_newton_schulz: bad sizes (batch %lld, rows %lld, cols %lld, steps %d)",
-                (long long)batch, (long long)rows, (long long)cols, steps);
-  if (!x_dev || !workspace_dev) return fail(FSH_EINVAL, "fsh_newton_schulz: null pointer");
-  if (rows % 8 || cols % 8)
-    return fail(FSH_ENOTSUP, "fsh_newton_schulz: rows and cols must be multiples of 8, got %lld x %lld",
+namespace fsh {
+namespace {
+
+// One batch of equally shaped matrices on its way through the iteration.
+// X is [s, l]; XT[0], XT[1] are the two [l, s] buffers.  The caller's buffer
+// is X when the input is wide and XT[0] when it is tall.  The first X^T goes
+// to XT[steps % 2] so that the last step leaves X^T in XT[0].
+struct NsState {
+  int64_t batch, s, l;
+  uint16_t* X;
+  uint16_t* XT[2];
+  uint16_t* G;
+  uint16_t* P;
+  int cur;
+};
+
+int ns_begin(const fsh_ns_problem& q, int32_t steps, float eps, hipStream_t stream, NsState* st) {
+  const int64_t batch = q.batch, rows = q.rows, cols = q.cols;
+  if (batch <= 0 || rows <= 0 || cols <= 0)
+    return fail(FSH_EINVAL, "newton_schulz: bad sizes (batch %lld, rows %lld, cols %lld)", (long long)batch,
                 (long long)rows, (long long)cols);
-  if (!aligned(x_dev, 16) || !aligned(workspace_dev, 256))
-    return fail(FSH_EINVAL, "fsh_newton_schulz: x must be 16-byte and workspace 256-byte aligned");
-  if (batch > 65535) return fail(FSH_ENOTSUP, "fsh_newton_schulz: batch %lld exceeds 65535", (long long)batch);
+  if (!q.x_dev || !q.workspace_dev) return fail(FSH_EINVAL, "newton_schulz: null pointer");
+  if (rows % 8 || cols % 8)
+    return fail(FSH_ENOTSUP, "newton_schulz: rows and cols must be multiples of 8, got %lld x %lld", (long long)rows,
+                (long long)cols);
+  if (!aligned(q.x_dev, 16) || !aligned(q.workspace_dev, 256))
+    return fail(FSH_EINVAL, "newton_schulz: x must be 16-byte and workspace 256-byte aligned");
+  if (batch > 65535) return fail(FSH_ENOTSUP, "newton_schulz: batch %lld exceeds 65535", (long long)batch);
   const int64_t need = fsh_newton_schulz_workspace_bytes(batch, rows, cols);
-  if (workspace_nbytes < need)
-    return fail(FSH_EINVAL, "fsh_newton_schulz: workspace of %lld bytes, need %lld", (long long)workspace_nbytes,
+  if (q.workspace_nbytes < need)
+    return fail(FSH_EINVAL, "newton_schulz: workspace of %lld bytes, need %lld", (long long)q.workspace_nbytes,
                 (long long)need);
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
   const bool tall = rows > cols;
   const int64_t s = tall ? cols : rows, l = tall ? rows : cols;
   const int64_t sl = s * l, ss = s * s;
-
-  uint8_t* ws = static_cast<uint8_t*>(workspace_dev);
+  uint8_t* ws = static_cast<uint8_t*>(q.workspace_dev);
   uint16_t* w0 = reinterpret_cast<uint16_t*>(ws);
   uint16_t* w1 = reinterpret_cast<uint16_t*>(ws + align256(batch * sl * 2));
-  uint16_t* G = reinterpret_cast<uint16_t*>(ws + 2 * align256(batch * sl * 2));
-  uint16_t* P = reinterpret_cast<uint16_t*>(ws + 2 * align256(batch * sl * 2) + align256(batch * ss * 2));
+  uint16_t* x = static_cast<uint16_t*>(q.x_dev);
+  st->batch = batch;
+  st->s = s;
+  st->l = l;
+  st->G = reinterpret_cast<uint16_t*>(ws + 2 * align256(batch * sl * 2));
+  st->P = reinterpret_cast<uint16_t*>(ws + 2 * align256(batch * sl * 2) + align256(batch * ss * 2));
   float* partial = reinterpret_cast<float*>(ws + 2 * align256(batch * sl * 2) + 2 * align256(batch * ss * 2));
-  uint16_t* x = static_cast<uint16_t*>(x_dev);
-
-  // X is [s, l]; XT[0], XT[1] are the two [l, s] buffers.  The caller's
-  // buffer is X when the input is wide and XT[0] when it is tall.  The first
-  // X^T goes to XT[steps % 2] so that the last step leaves X^T in XT[0].
-  uint16_t* X = tall ? w0 : x;
-  uint16_t* XT[2] = {tall ? x : w0, w1};
-  int cur = steps & 1;
+  st->X = tall ? w0 : x;
+  st->XT[0] = tall ? x : w0;
+  st->XT[1] = w1;
+  st->cur = steps & 1;
 
   hipLaunchKernelGGL(sumsq_partial_kernel, dim3(kNormBlocksPerMatrix, static_cast<uint32_t>(batch)),
                      dim3(kNormThreads), 0, stream, x, rows * cols, partial);
   if (int rc = check_launch("sumsq_partial_kernel")) return rc;
-  {
-    // Input is [rows, cols]; "same orientation" output is X for a wide input
-    // and X^T for a tall one.
-    uint16_t* same = tall ? XT[cur] : X;
-    uint16_t* transposed = tall ? X : XT[cur];
-    const dim3 grid(static_cast<uint32_t>(ceil_div(cols, (int64_t)kNormTile)),
-                    static_cast<uint32_t>(ceil_div(rows, (int64_t)kNormTile)), static_cast<uint32_t>(batch));
-    if (grid.y > 65535) return fail(FSH_ENOTSUP, "fsh_newton_schulz: more than %d row tiles", 65535 * kNormTile);
-    hipLaunchKernelGGL(normalize_dual_kernel, grid, dim3(kNormThreads), 0, stream, x, same, transposed, rows,
-                       cols, partial, bf16_round_host(eps));
-    if (int rc = check_launch("normalize_dual_kernel")) return rc;
-  }
+  // Input is [rows, cols]; "same orientation" output is X for a wide input
+  // and X^T for a tall one.
+  uint16_t* same = tall ? st->XT[st->cur] : st->X;
+  uint16_t* transposed = tall ? st->X : st->XT[st->cur];
+  const dim3 grid(static_cast<uint32_t>(ceil_div(cols, (int64_t)kNormTile)),
+                  static_cast<uint32_t>(ceil_div(rows, (int64_t)kNormTile)), static_cast<uint32_t>(batch));
+  if (grid.y > 65535) return fail(FSH_ENOTSUP, "newton_schulz: more than %d row tiles", 65535 * kNormTile);
+  hipLaunchKernelGGL(normalize_dual_kernel, grid, dim3(kNormThreads), 0, stream, x, same, transposed, rows, cols,
+                     partial, bf16_round_host(eps));
+  return check_launch("normalize_dual_kernel");
+}
 
-  for (int step = 0; step < steps; ++step) {
-    fsh_gemm_desc g;
-    memset(&g, 0, sizeof(g));
-    g.batch = batch;
-    // G = X X^T
-    g.a_dev = X; g.b_dev = X; g.d_dev = nullptr; g.c_dev = G; g.ct_dev = nullptr;
+// The three products of one iteration; `which` = 0: G = X X^T, 1: P = b G +
+// c G G (symmetric because G is), 2: X' = a X + P X, also written transposed
+// into the other X^T buffer.
+fsh_gemm_desc ns_product(const NsState& st, int which, float a, float b, float c) {
+  const int64_t s = st.s, l = st.l, sl = s * l, ss = s * s;
+  fsh_gemm_desc g;
+  memset(&g, 0, sizeof(g));
+  g.batch = st.batch;
+  if (which == 0) {
+    g.a_dev = st.X; g.b_dev = st.X; g.c_dev = st.G;
     g.m = s; g.n = s; g.k = l; g.lda = l; g.ldb = l; g.ldc = s;
     g.stride_a = sl; g.stride_b = sl; g.stride_c = ss;
     g.alpha = 1.0f; g.beta = 0.0f;
     g.symmetric = 1;
-    if (int rc = launch_gemm(g, stream)) return rc;
-    // P = b G + c G G, symmetric because G is
-    g.a_dev = G; g.b_dev = G; g.d_dev = G; g.c_dev = P;
+  } else if (which == 1) {
+    g.a_dev = st.G; g.b_dev = st.G; g.d_dev = st.G; g.c_dev = st.P;
     g.m = s; g.n = s; g.k = s; g.lda = s; g.ldb = s; g.ldd = s; g.ldc = s;
     g.stride_a = ss; g.stride_b = ss; g.stride_d = ss; g.stride_c = ss;
     g.alpha = c; g.beta = b;
-    if (int rc = launch_gemm(g, stream)) return rc;
-    // X' = a X + P X, also written transposed into the other X^T buffer
-    g.symmetric = 0;
-    g.a_dev = P; g.b_dev = XT[cur]; g.d_dev = X; g.c_dev = X; g.ct_dev = XT[cur ^ 1];
+    g.symmetric = 1;
+  } else {
+    g.a_dev = st.P; g.b_dev = st.XT[st.cur]; g.d_dev = st.X; g.c_dev = st.X; g.ct_dev = st.XT[st.cur ^ 1];
     g.m = s; g.n = l; g.k = s; g.lda = s; g.ldb = s; g.ldd = l; g.ldc = l; g.ldct = s;
     g.stride_a = ss; g.stride_b = sl; g.stride_d = sl; g.stride_c = sl; g.stride_ct = sl;
     g.alpha = 1.0f; g.beta = a;
-    if (int rc = launch_gemm(g, stream)) return rc;
-    cur ^= 1;
+  }
+  return g;
+}
+
+}  // namespace
+}  // namespace fsh
+
+FSH_API int fsh_newton_schulz_multi(const fsh_ns_problem* problems, int32_t count, float a, float b, float c,
+                                    int32_t steps, float eps, void* stream_) {
+  using namespace fsh;
+  if (count < 0 || count > FSH_MAX_NS_PROBLEMS || (count > 0 && problems == nullptr))
+    return fail(FSH_EINVAL, "fsh_newton_schulz_multi: count %d outside [0, %d] or null list", count,
+                FSH_MAX_NS_PROBLEMS);
+  if (steps < 0) return fail(FSH_EINVAL, "fsh_newton_schulz_multi: negative step count %d", steps);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  NsState st[FSH_MAX_NS_PROBLEMS];
+  for (int i = 0; i < count; ++i)
+    if (int rc = ns_begin(problems[i], steps, eps, stream, &st[i])) return rc;
+  fsh_gemm_desc descs[FSH_MAX_NS_PROBLEMS];
+  for (int step = 0; step < steps; ++step) {
+    // The same product of every problem goes out together: problems are
+    // independent of each other, the three products of one are not.
+    for (int which = 0; which < 3; ++which) {
+      for (int i = 0; i < count; ++i) descs[i] = ns_product(st[i], which, a, b, c);
+      if (int rc = launch_gemms(descs, count, stream)) return rc;
+    }
+    for (int i = 0; i < count; ++i) st[i].cur ^= 1;
   }
   // cur == 0 here: for a tall input the result X^T is in the caller's buffer;
   // for a wide input X was updated in place.
   return FSH_OK;
+}
+
+FSH_API int fsh_newton_schulz(void* x_dev, int64_t batch, int64_t rows, int64_t cols, float a, float b,
+                              float c, int32_t steps, float eps, void* workspace_dev,
+                              int64_t workspace_nbytes, void* stream_) {
+  fsh_ns_problem q;
+  q.x_dev = x_dev;
+  q.batch = batch;
+  q.rows = rows;
+  q.cols = cols;
+  q.workspace_dev = workspace_dev;
+  q.workspace_nbytes = workspace_nbytes;
+  return fsh_newton_schulz_multi(&q, 1, a, b, c, steps, eps, stream_);
 }

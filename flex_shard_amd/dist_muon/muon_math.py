@@ -194,6 +194,9 @@ class OwnedMuon:
             if g.shape != p.shape:
                 raise ValueError(f"gradient shape {tuple(g.shape)} does not match parameter {tuple(p.shape)}")
         _require_bf16_gpu(*grads)
+        # Momentum for every matrix first, then one Newton-Schulz call over all
+        # shape groups (each product of the iteration is issued for all groups
+        # together), then the updates.
         for shape, members in self._groups.items():
             batch = self._batch[shape]
             for slot, index in enumerate(members):
@@ -201,10 +204,12 @@ class OwnedMuon:
                     grads[index], self.momentum_buffers[index], momentum=self.momentum, nesterov=self.nesterov,
                     out=batch[slot],
                 )
-            _compute_muon_direction(
-                batch, ns_coefficients=self.ns_coefficients, ns_steps=self.ns_steps, eps=self.eps,
-                workspace=self._workspace[shape],
-            )
+        hip_ops.newton_schulz_multi(
+            [(self._batch[shape], self._workspace[shape]) for shape in self._groups],
+            self.ns_coefficients, self.ns_steps, self.eps,
+        )
+        for shape, members in self._groups.items():
+            batch = self._batch[shape]
             for slot, index in enumerate(members):
                 _apply_muon_update(
                     self.params[index], batch[slot], lr=self.lr, weight_decay=self.weight_decay,

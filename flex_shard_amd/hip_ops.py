@@ -311,14 +311,50 @@ def newton_schulz(
     return x
 
 
-def gemm_nt(
-    a: torch.Tensor, b: torch.Tensor, *, d: torch.Tensor | None = None, alpha: float = 1.0, beta: float = 0.0,
-    out: torch.Tensor | None = None, out_t: torch.Tensor | None = None, symmetric: bool = False,
-) -> torch.Tensor:
-    """``bf16(alpha * a @ b^T + beta * d)`` for contiguous bf16 [batch, m, k] /
-    [batch, n, k] (or 2-D) operands; optionally also the transpose.  With
-    ``symmetric`` the caller guarantees a symmetric result (m == n); only the
-    upper triangle of tiles is computed and mirrored."""
+def newton_schulz_multi(
+    problems: Sequence[tuple[torch.Tensor, torch.Tensor | None]],
+    coefficients: tuple[float, float, float],
+    steps: int,
+    eps: float,
+) -> None:
+    """In-place Newton-Schulz of several contiguous bf16 [batch, rows, cols]
+    tensors of different shapes, each with its workspace (allocated when
+    ``None``).  Same results as one ``newton_schulz`` call per tensor."""
+    if not problems:
+        return
+    if len(problems) > _native.MAX_NS_PROBLEMS:
+        for begin in range(0, len(problems), _native.MAX_NS_PROBLEMS):
+            newton_schulz_multi(problems[begin : begin + _native.MAX_NS_PROBLEMS], coefficients, steps, eps)
+        return
+    table = (_native.NsProblem * len(problems))()
+    keep = []
+    device = problems[0][0].device
+    for i, (x, workspace) in enumerate(problems):
+        _require_gpu(x)
+        if x.device != device:
+            raise ValueError("all problems of a call must live on one device")
+        if x.dtype != torch.bfloat16 or not x.is_contiguous() or x.ndim not in (2, 3):
+            raise ValueError("x must be a contiguous bf16 matrix or batch of matrices")
+        batch = 1 if x.ndim == 2 else x.shape[0]
+        rows, cols = x.shape[-2:]
+        need = newton_schulz_workspace_bytes(batch, rows, cols)
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+        _require_gpu(x, workspace)
+        if workspace.dtype != torch.uint8 or not workspace.is_contiguous() or workspace.numel() < need:
+            raise ValueError(f"workspace must be contiguous uint8 with at least {need} bytes")
+        keep.append(workspace)
+        table[i].x_dev, table[i].batch, table[i].rows, table[i].cols = x.data_ptr(), batch, rows, cols
+        table[i].workspace_dev, table[i].workspace_nbytes = workspace.data_ptr(), workspace.numel()
+    a, b, c = coefficients
+    status = _native.lib().fsh_newton_schulz_multi(table, len(problems), a, b, c, steps, eps, stream_ptr(device))
+    _native.check(status, "fsh_newton_schulz_multi")
+
+
+def _gemm_desc(
+    a: torch.Tensor, b: torch.Tensor, d: torch.Tensor | None, alpha: float, beta: float,
+    out: torch.Tensor | None, out_t: torch.Tensor | None, symmetric: bool,
+) -> tuple["_native.GemmDesc", torch.Tensor]:
     _require_gpu(a, b)
     if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16 or not a.is_contiguous() or not b.is_contiguous():
         raise ValueError("a and b must be contiguous bf16")
@@ -348,9 +384,42 @@ def gemm_nt(
     desc.stride_d = desc.stride_c = desc.stride_ct = m * n
     desc.alpha, desc.beta = alpha, beta
     desc.symmetric = 1 if symmetric else 0
+    return desc, out
+
+
+def gemm_nt(
+    a: torch.Tensor, b: torch.Tensor, *, d: torch.Tensor | None = None, alpha: float = 1.0, beta: float = 0.0,
+    out: torch.Tensor | None = None, out_t: torch.Tensor | None = None, symmetric: bool = False,
+) -> torch.Tensor:
+    """``bf16(alpha * a @ b^T + beta * d)`` for contiguous bf16 [batch, m, k] /
+    [batch, n, k] (or 2-D) operands; optionally also the transpose.  With
+    ``symmetric`` the caller guarantees a symmetric result (m == n); only the
+    upper triangle of tiles is computed and mirrored."""
+    desc, out = _gemm_desc(a, b, d, alpha, beta, out, out_t, symmetric)
     status = _native.lib().fsh_gemm_bf16_nt(ctypes.byref(desc), stream_ptr(a.device))
     _native.check(status, "fsh_gemm_bf16_nt")
     return out
+
+
+def gemm_nt_group(problems: Sequence[dict]) -> list[torch.Tensor]:
+    """Independent ``gemm_nt`` problems (dicts of its arguments) issued in one
+    call; the ones that take the large-tile kernel share launches."""
+    if not problems:
+        return []
+    descs = (_native.GemmDesc * len(problems))()
+    outs = []
+    for i, q in enumerate(problems):
+        desc, out = _gemm_desc(
+            q["a"], q["b"], q.get("d"), q.get("alpha", 1.0), q.get("beta", 0.0), q.get("out"), q.get("out_t"),
+            q.get("symmetric", False),
+        )
+        descs[i] = desc
+        outs.append(out)
+        if out.device != outs[0].device:
+            raise ValueError("all problems of a group must live on one device")
+    status = _native.lib().fsh_gemm_bf16_nt_group(descs, len(problems), stream_ptr(outs[0].device))
+    _native.check(status, "fsh_gemm_bf16_nt_group")
+    return outs
 
 
 def muon_prepare(

@@ -186,6 +186,22 @@ int fsh_newton_schulz(void* x_dev, int64_t batch, int64_t rows, int64_t cols, fl
                       float c, int32_t steps, float eps, void* workspace_dev,
                       int64_t workspace_nbytes, void* stream);
 
+/* Several batches of different shapes in one call (the per-shape groups of
+ * the owned matrices of dist_muon/optimizer.py, which the reference runs one
+ * after the other through :2120-2151).  Results are identical to calling
+ * fsh_newton_schulz once per problem; the same product of all problems is
+ * issued together so that the short tiles of one shape fill the last,
+ * partly empty round of workgroups of another.  Problems must not overlap. */
+typedef struct fsh_ns_problem {
+  void* x_dev;             /* [batch, rows, cols] bf16, overwritten            */
+  int64_t batch, rows, cols;
+  void* workspace_dev;     /* >= fsh_newton_schulz_workspace_bytes(batch, rows, cols) */
+  int64_t workspace_nbytes;
+} fsh_ns_problem;
+#define FSH_MAX_NS_PROBLEMS 16
+int fsh_newton_schulz_multi(const fsh_ns_problem* problems, int32_t count, float a, float b, float c,
+                            int32_t steps, float eps, void* stream);
+
 /* Batched bf16 "NT" GEMM, the building block of (6), exported for tests:
  *   C[b] = bf16(alpha * A[b] . B[b]^T + beta * D[b])      fp32 accumulation
  * A is [m, k] with row stride lda, B is [n, k] with row stride ldb (both
@@ -211,6 +227,9 @@ typedef struct fsh_gemm_desc {
   int32_t reserved;  /* 0 */
 } fsh_gemm_desc;
 int fsh_gemm_bf16_nt(const fsh_gemm_desc* desc, void* stream);
+/* `count` independent products; those that qualify for the large-tile kernel
+ * share launches.  Same results as `count` calls of fsh_gemm_bf16_nt. */
+int fsh_gemm_bf16_nt_group(const fsh_gemm_desc* descs, int32_t count, void* stream);
 
 /* ------------------------------------------------------------------------
  * 7. Muon elementwise steps in bf16 (fp32 math, one rounding per reference

@@ -411,6 +411,71 @@ def test_gemm_symmetric_mode_mirrors_the_upper_triangle(device, batch, n, k):
         hip_ops.gemm_nt(a, a[:, : n - 8].contiguous(), symmetric=True)
 
 
+def test_gemm_group_equals_separate_calls(device):
+    """Problems of different shapes and kernels in one call: the ones on the
+    large-tile kernel share a launch (longest k first), every result is bit
+    for bit what a call of its own gives, and nothing outside the outputs is
+    written."""
+    gen = torch.Generator().manual_seed(21)
+    specs = [
+        # (batch, m, n, k, symmetric, with d, with out_t)
+        (10, 1536, 1536, 128, True, False, False),  # large tile, short k
+        (7, 1536, 1280, 320, False, True, True),  # large tile, long k, all outputs
+        (1, 512, 384, 96, False, True, False),  # 128x128 whole-tile kernel
+        (10, 1536, 1536, 192, True, True, False),  # large tile, symmetric with addend
+        (2, 264, 136, 72, False, False, True),  # predicated kernel
+        (8, 1280, 1280, 64, False, False, False),  # large tile, one k-tile
+    ]
+    pad = 1024
+    problems, buffers = [], []
+    for batch, m, n, k, symmetric, with_d, with_t in specs:
+        a = torch.randn(batch, m, k, generator=gen).bfloat16().to(device)
+        b = a if symmetric else torch.randn(batch, n, k, generator=gen).bfloat16().to(device)
+        d = None
+        if with_d:
+            d = torch.randn(batch, m, n, generator=gen).bfloat16().to(device)
+            if symmetric:
+                d = torch.triu(d) + torch.triu(d, 1).transpose(1, 2)
+        c_buf = torch.full((batch * m * n + 2 * pad,), 7.0, dtype=torch.bfloat16, device=device)
+        t_buf = torch.full((batch * m * n + 2 * pad,), 7.0, dtype=torch.bfloat16, device=device) if with_t else None
+        buffers += [c_buf] + ([t_buf] if with_t else [])
+        problems.append(dict(
+            a=a, b=b, d=d, alpha=0.75, beta=-1.5, symmetric=symmetric, out=c_buf[pad:-pad].view(batch, m, n),
+            out_t=t_buf[pad:-pad].view(batch, n, m) if with_t else None,
+        ))
+    outs = hip_ops.gemm_nt_group(problems)
+    for q, out in zip(problems, outs):
+        alone = hip_ops.gemm_nt(q["a"], q["b"], d=q["d"], alpha=q["alpha"], beta=q["beta"], symmetric=q["symmetric"])
+        assert torch.equal(out, alone)
+        if q["out_t"] is not None:
+            assert torch.equal(q["out_t"], out.transpose(1, 2).contiguous())
+        ref = _gemm_reference(q["a"], q["b"], q["d"], q["alpha"], q["beta"])
+        assert torch.allclose(out.cpu().double(), ref, rtol=2.0**-7, atol=0.25)
+    for buf in buffers:
+        assert (buf[:pad] == 7).all() and (buf[-pad:] == 7).all()
+    assert hip_ops.gemm_nt_group([]) == []
+
+
+def test_newton_schulz_multi_equals_one_call_per_shape(device):
+    """Shape groups iterated together (each product issued for all groups at
+    once) against one call per group: identical bits, tall, wide and square,
+    large-tile and small-tile kernels mixed."""
+    shapes = [(40, 1024, 768), (48, 768, 768), (5, 256, 1024), (1, 64, 96)]  # the first two fill the large tile
+    inputs = [seeded_normal(shape, 1.0, 30 + i, device) for i, shape in enumerate(shapes)]
+    together = [x.clone() for x in inputs]
+    hip_ops.newton_schulz_multi([(x, None) for x in together], COEFFS, 5, 1e-7)
+    for x, y in zip(inputs, together):
+        alone = hip_ops.newton_schulz(x.clone(), COEFFS, 5, 1e-7)
+        assert torch.equal(alone, y)
+    from torch.optim._muon import _zeropower_via_newtonschulz as torch_ns
+
+    want = torch_ns(inputs[0][0].cpu(), COEFFS, 5, 1e-7)
+    assert (together[0][0].cpu().float() - want.float()).abs().max().item() <= 2e-2
+    hip_ops.newton_schulz_multi([], COEFFS, 5, 1e-7)
+    with pytest.raises(RuntimeError, match="multiples of 8"):
+        hip_ops.newton_schulz_multi([(together[0], None), (torch.zeros(2, 12, 20, device=device, dtype=torch.bfloat16), None)], COEFFS, 5, 1e-7)
+
+
 def test_newton_schulz_full_size_invariants(device):
     """Config 5 shapes: [7168, 2048] (tall, iterated as its transpose) and
     [2048, 2048].  Singular values of the result lie in the quintic's band and
