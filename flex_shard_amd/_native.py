@@ -81,7 +81,7 @@ class GemmDesc(Structure):
         ("alpha", c_float),
         ("beta", c_float),
         ("symmetric", c_int32),
-        ("reserved", c_int32),
+        ("diag_add", c_float),
     ]
 
 

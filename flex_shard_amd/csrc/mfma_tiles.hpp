@@ -22,6 +22,7 @@ struct GemmParams {
   int64_t lda, ldb, ldd, ldc, ldct;
   int64_t sA, sB, sD, sC, sCt;
   float alpha, beta;
+  float diag_add;         // added to C[i][i] before the rounding
   int32_t tiles_m, tiles_n;
   int32_t symmetric;      // only tiles with tm <= tn are computed; the others are mirrored
   int32_t tiles_per_matrix;
@@ -46,6 +47,7 @@ constexpr int kMaxGemmProblems = 4;
 struct GemmLaunch {
   GemmParams problem[kMaxGemmProblems];
   int32_t first_workgroup[kMaxGemmProblems];  // INT32_MAX past the last problem
+  int32_t total_workgroups;
 };
 
 constexpr int kXcds = 8;         // accelerator dies, each with its own L2
@@ -114,21 +116,39 @@ struct WholeTileEpilogue {
   static constexpr int kLdsBytes = Cfg::WM * Cfg::WN * kRegion;
 };
 
+// Values that are the same in every lane but that the compiler cannot prove
+// so: moved to scalar registers.
+__device__ __forceinline__ int uniform_i32(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ int64_t uniform_i64(int64_t v) {
+  const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(v & 0xFFFFFFFFLL)));
+  const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(v >> 32)));
+  return static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+template <typename T>
+__device__ __forceinline__ T* uniform_ptr(T* ptr) {
+  return reinterpret_cast<T*>(uniform_i64(reinterpret_cast<int64_t>(ptr)));
+}
+
 // Stores a [rows][row_bytes] bf16 image held in LDS (pitch bytes apart) to
-// global rows `ld` elements apart, 16 bytes per lane.
+// global rows `ld` elements apart, 16 bytes per lane.  `dst` is the same in
+// every lane: each store is a scalar base (advanced per pass) plus one 32-bit
+// lane offset, so the passes share a single address register.
 template <int kRows, int kRowBytes, int kPitch>
 __device__ inline void store_staged_rows(const uint8_t* region, uint16_t* dst, int64_t ld, int lane) {
   constexpr int kLanesPerRow = kRowBytes / 16;
   constexpr int kRowsPerPass = 64 / kLanesPerRow;
   static_assert(kRowBytes % 16 == 0 && 64 % kLanesPerRow == 0 && kRows % kRowsPerPass == 0, "staged store shape");
   const int r0 = lane / kLanesPerRow, chunk = lane % kLanesPerRow;
+  const uint32_t lane_off = static_cast<uint32_t>(r0) * static_cast<uint32_t>(ld * 2) + chunk * 16;
+  uint8_t* base = uniform_ptr(reinterpret_cast<uint8_t*>(dst));
+  const int64_t pass_bytes = uniform_i64(static_cast<int64_t>(kRowsPerPass) * ld * 2);
 #pragma unroll
   for (int pass = 0; pass < kRows / kRowsPerPass; ++pass) {
     const int r = pass * kRowsPerPass + r0;
     const uint8_t* src = region + r * kPitch + chunk * 16;
     const u32x2 lo = *reinterpret_cast<const u32x2*>(src);
     const u32x2 hi = *reinterpret_cast<const u32x2*>(src + 8);
-    *reinterpret_cast<u32x4*>(dst + r * ld + chunk * 8) = u32x4{lo.x, lo.y, hi.x, hi.y};
+    *reinterpret_cast<u32x4*>(base + pass * pass_bytes + lane_off) = u32x4{lo.x, lo.y, hi.x, hi.y};
   }
 }
 
@@ -158,12 +178,13 @@ template <typename Cfg>
 __device__ __forceinline__ void load_d_rows(const GemmParams& p, int64_t batch, int64_t m0, int64_t n0, int wm, int wn,
                                             int lane, int half, DRows<Cfg>& rows) {
   using R = DRows<Cfg>;
-  const int r0 = half * (Cfg::kWaveM / 2) + lane / R::kLanesPerRow, chunk = lane % R::kLanesPerRow;
-  const uint16_t* dsrc =
-      p.D + batch * p.sD + (m0 + wm * Cfg::kWaveM + r0) * p.ldd + n0 + wn * Cfg::kWaveN + chunk * 8;
+  const int r0 = lane / R::kLanesPerRow, chunk = lane % R::kLanesPerRow;
+  const uint32_t lane_off = static_cast<uint32_t>(r0) * static_cast<uint32_t>(p.ldd * 2) + chunk * 16;
+  const uint8_t* base = uniform_ptr(reinterpret_cast<const uint8_t*>(
+      p.D + batch * p.sD + (m0 + wm * Cfg::kWaveM + half * (Cfg::kWaveM / 2)) * p.ldd + n0 + wn * Cfg::kWaveN));
+  const int64_t pass_bytes = uniform_i64(static_cast<int64_t>(R::kRowsPerPass) * p.ldd * 2);
 #pragma unroll
-  for (int q = 0; q < R::kPasses; ++q)
-    rows.t[q] = *reinterpret_cast<const u32x4*>(dsrc + static_cast<int64_t>(q) * R::kRowsPerPass * p.ldd);
+  for (int q = 0; q < R::kPasses; ++q) rows.t[q] = *reinterpret_cast<const u32x4*>(base + q * pass_bytes + lane_off);
 }
 
 template <typename Cfg, int kPitch>
@@ -208,6 +229,9 @@ __device__ inline void store_whole_tile(const GemmParams& p, int64_t batch, int6
   // finals = bf16(fma(beta, D, alpha*acc)): one rounding of the scaled
   // accumulator, one of the sum, as a BLAS epilogue does.
   const bool unit_alpha = p.alpha == 1.0f;
+  // Block tiles and wave sub-tiles are square, so C's diagonal runs through
+  // the (i, i) blocks of the diagonal sub-tiles of the diagonal tiles.
+  const bool on_diagonal = p.diag_add != 0.0f && m0 == n0 && wm == wn;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     if (has_d && i == TM / 2) stage_d_rows<Cfg, Epi::kPitch>(region, lane, 1, lower);
@@ -234,6 +258,11 @@ __device__ inline void store_whole_tile(const GemmParams& p, int64_t batch, int6
           v[1] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].x & 0xFFFF0000u), v[1]);
           v[2] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].y << 16), v[2]);
           v[3] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].y & 0xFFFF0000u), v[3]);
+        }
+        if (on_diagonal && i == j) {
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            if (r_lane == 8 * b + 4 * h + t) v[t] += p.diag_add;
         }
         *reinterpret_cast<u32x2*>(region + (i * 32 + r_lane) * Epi::kPitch + (j * 32 + 8 * b + 4 * h) * 2) =
             u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
@@ -273,6 +302,153 @@ __device__ inline void store_whole_tile(const GemmParams& p, int64_t batch, int6
   FSH_STAMP(12);
   __syncthreads();
   store_staged_rows<Cfg::kWaveN, Cfg::kWaveM * 2, Epi::kPitchT>(region, Ct + wave_col * ldct + wave_row, ldct, lane);
+}
+
+// Orders the LDS traffic of one wave: lanes exchange data through the wave's
+// private staging region, which the hardware serves in program order; this
+// only keeps the compiler from moving a lane's reads above other lanes'
+// writes.  No counter is waited for and no workgroup barrier is taken.
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Epilogue of the large-tile kernel: the same steps as store_whole_tile, but
+// on the upper and then the lower 64 rows of the wave's 128x128 sub-tile, in a
+// staging region of 17 KB per wave that only the wave itself touches.  The
+// region then fits beside one k-loop stage, which leaves the other stage free
+// to receive the next tile's first operands while this runs, and no step
+// needs a workgroup barrier (whose memory fence would wait for those loads).
+template <typename Cfg>
+struct HalfTileEpilogue {
+  static constexpr int kRows = Cfg::kWaveM / 2;                 // 64
+  static constexpr int kPitch = Cfg::kWaveN * 2 + 8;            // [row][col] image
+  static constexpr int kPitchT = kRows * 2 + 8;                 // [col][row] image
+  static constexpr int kRegion =
+      (kRows * kPitch > Cfg::kWaveN * kPitchT) ? kRows * kPitch : Cfg::kWaveN * kPitchT;
+  static constexpr int kLdsBytes = Cfg::WM * Cfg::WN * kRegion;
+};
+
+template <typename Cfg>
+__device__ inline void store_tile_in_halves(const GemmParams& p, int64_t batch, int64_t m0, int64_t n0, int wm, int wn,
+                                            int lane, bool mirror, const f32x16 (&acc)[Cfg::TM][Cfg::TN],
+                                            uint8_t* staging) {
+  using Epi = HalfTileEpilogue<Cfg>;
+  using R = DRows<Cfg>;
+  constexpr int TM = Cfg::TM, TN = Cfg::TN, HM = TM / 2;
+  static_assert(TM % 2 == 0 && Epi::kRows == HM * 32, "two halves of whole 32-row blocks");
+  const bool has_d = p.D != nullptr;
+  uint16_t* C = p.C + batch * p.sC;
+  // A symmetric product mirrors its off-diagonal tiles into the lower triangle.
+  uint16_t* Ct = mirror ? C : (p.Ct ? p.Ct + batch * p.sCt : nullptr);
+  const int64_t ldct = mirror ? p.ldc : p.ldct;
+  const int64_t wave_row = m0 + wm * Cfg::kWaveM, wave_col = n0 + wn * Cfg::kWaveN;
+  uint8_t* region = staging + (wm * Cfg::WN + wn) * Epi::kRegion;
+  const int r_lane = lane & 31, h = lane >> 5;
+  const bool unit_alpha = p.alpha == 1.0f;
+  // Block tiles and wave sub-tiles are square, so C's diagonal runs through
+  // the (i, i) blocks of the diagonal sub-tiles of the diagonal tiles.
+  const bool on_diagonal = p.diag_add != 0.0f && m0 == n0 && wm == wn;
+
+  // The lower half of D is requested once the upper half has left its
+  // registers for LDS, and lands while the upper half is worked on.
+  DRows<Cfg> drows[2];
+  if (has_d) load_d_rows<Cfg>(p, batch, m0, n0, wm, wn, lane, 0, drows[0]);
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf) {
+    if (has_d) {
+      // stage_d_rows with the half's rows at the top of the region
+      const int r0 = lane / R::kLanesPerRow, chunk = lane % R::kLanesPerRow;
+#pragma unroll
+      for (int q = 0; q < R::kPasses; ++q) {
+        uint8_t* d = region + (r0 + q * R::kRowsPerPass) * Epi::kPitch + chunk * 16;
+        *reinterpret_cast<u32x2*>(d) = u32x2{drows[hf].t[q].x, drows[hf].t[q].y};
+        *reinterpret_cast<u32x2*>(d + 8) = u32x2{drows[hf].t[q].z, drows[hf].t[q].w};
+      }
+      if (hf == 0) load_d_rows<Cfg>(p, batch, m0, n0, wm, wn, lane, 1, drows[1]);
+      wave_lds_sync();
+    }
+#pragma unroll
+    for (int ih = 0; ih < HM; ++ih) {
+      u32x2 fin[TN][4];  // packed bf16 finals of this 32-row block, accumulator layout
+      const int i = hf * HM + ih;
+      u32x2 dv[TN][4];
+      if (has_d) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int b = 0; b < 4; ++b)
+            dv[j][b] = *reinterpret_cast<const u32x2*>(region + (ih * 32 + r_lane) * Epi::kPitch +
+                                                       (j * 32 + 8 * b + 4 * h) * 2);
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          float v[4];
+#pragma unroll
+          for (int t = 0; t < 4; ++t) v[t] = unit_alpha ? acc[i][j][4 * b + t] : p.alpha * acc[i][j][4 * b + t];
+          if (has_d) {
+            v[0] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].x << 16), v[0]);
+            v[1] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].x & 0xFFFF0000u), v[1]);
+            v[2] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].y << 16), v[2]);
+            v[3] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].y & 0xFFFF0000u), v[3]);
+          }
+          if (on_diagonal && i == j) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+              if (r_lane == 8 * b + 4 * h + t) v[t] += p.diag_add;
+          }
+          fin[j][b] = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+        }
+      // A lane's finals replace exactly the D values it read itself.
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          *reinterpret_cast<u32x2*>(region + (ih * 32 + r_lane) * Epi::kPitch + (j * 32 + 8 * b + 4 * h) * 2) =
+              fin[j][b];
+    }
+    if (hf == 1) FSH_STAMP(9);
+    wave_lds_sync();
+    store_staged_rows<Epi::kRows, Cfg::kWaveN * 2, Epi::kPitch>(
+        region, C + (wave_row + hf * Epi::kRows) * p.ldc + wave_col, p.ldc, lane);
+    if (hf == 1) FSH_STAMP(10);
+    if (Ct != nullptr) {  // uniform over the workgroup
+      // The finals come back in accumulator layout (every read before the
+      // first write: the transposed image reuses the region).
+      u32x2 fin[HM][TN][4];
+#pragma unroll
+      for (int ih = 0; ih < HM; ++ih)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int b = 0; b < 4; ++b)
+            fin[ih][j][b] = *reinterpret_cast<const u32x2*>(region + (ih * 32 + r_lane) * Epi::kPitch +
+                                                            (j * 32 + 8 * b + 4 * h) * 2);
+      wave_lds_sync();  // these reads and the row reads are done before the region is reused
+#pragma unroll
+      for (int ih = 0; ih < HM; ++ih)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int b = 0; b < 4; ++b)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+              const uint32_t pair = (t >> 1) ? fin[ih][j][b].y : fin[ih][j][b].x;
+              *reinterpret_cast<uint16_t*>(region + (j * 32 + 8 * b + 4 * h + t) * Epi::kPitchT +
+                                           (ih * 32 + r_lane) * 2) =
+                  static_cast<uint16_t>((t & 1) ? (pair >> 16) : pair);
+            }
+      if (hf == 1) FSH_STAMP(12);
+      wave_lds_sync();
+      store_staged_rows<Cfg::kWaveN, Epi::kRows * 2, Epi::kPitchT>(
+          region, Ct + wave_col * ldct + wave_row + hf * Epi::kRows, ldct, lane);
+    }
+    if (hf == 0) FSH_STAMP(8);
+    if (hf == 0) wave_lds_sync();  // before the lower half overwrites the region
+  }
 }
 
 // Scheduling-group masks of __builtin_amdgcn_sched_group_barrier.

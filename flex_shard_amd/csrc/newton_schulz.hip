@@ -187,6 +187,7 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_nt_kernel(const GemmParams
         for (int t = 0; t < 4; ++t) {
           float v = p.alpha * acc[i][j][4 * b + t];
           if (D != nullptr) v += p.beta * dv[t];
+          if (row == col + t) v += p.diag_add;
           packed[t] = f32_to_bf16_bits(v);
         }
         if (full && c_vec) {
@@ -373,13 +374,19 @@ struct DmaGemm {
   static constexpr int kLoadsPerOperand = BM / 8 / 4;        // wave-level 1 KB loads per wave: 8
 };
 
+// kPersistent: the grid is one workgroup per compute unit and workgroup g
+// takes the ids g, g + gridDim.x, ... of the launch (the same XCD every time,
+// and the 32 workgroups of an XCD stay on 32 neighbouring tiles).  While the
+// epilogue of a tile runs, the first operands of the next one are already on
+// their way into stage 0.  The schedule is static, so the host uses it only
+// when all tiles of the launch are equally long; otherwise each id is its own
+// workgroup and the hardware hands them out as compute units come free.
+template <bool kPersistent>
 __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const GemmLaunch launch) {
   using Cfg = DmaGemm;
-  int which = 0;
-#pragma unroll
-  for (int i = 1; i < kMaxGemmProblems; ++i) which += static_cast<int>(blockIdx.x) >= launch.first_workgroup[i] ? 1 : 0;
-  const GemmParams& p = launch.problem[which];
-  const int64_t local_id = static_cast<int64_t>(blockIdx.x) - launch.first_workgroup[which];
+#ifdef FSH_TRACE
+  const GemmParams& p = launch.problem[0];  // the profiling build stamps into the first problem's buffer
+#endif
   FSH_STAMP(0);
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds_bytes[];
   constexpr int TM = Cfg::TM, TN = Cfg::TN, KS = Cfg::KS;
@@ -388,30 +395,51 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
-  int64_t batch;
-  int tm, tn;
-  if (!tile_of_workgroup(p, local_id, &batch, &tm, &tn)) return;  // whole workgroup, before any barrier
-  const int64_t m0 = static_cast<int64_t>(tm) * Cfg::BM;
-  const int64_t n0 = static_cast<int64_t>(tn) * Cfg::BN;
-  const uint8_t* Ab = reinterpret_cast<const uint8_t*>(p.A + batch * p.sA + m0 * p.lda);
-  const uint8_t* Bb = reinterpret_cast<const uint8_t*>(p.B + batch * p.sB + n0 * p.ldb);
-  const int64_t ktiles = p.K / Cfg::BK;
+
+  // Tile of launch id `id`: problem index, batch, tile row and column (all
+  // uniform; moved to scalar registers explicitly).  False for padding ids.
+  auto locate = [&](int64_t id, int& which, int64_t& batch, int& tm, int& tn) -> bool {
+    int w = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxGemmProblems; ++i) w += id >= launch.first_workgroup[i] ? 1 : 0;
+    w = uniform_i32(w);
+    int64_t b;
+    int r, c;
+    if (!tile_of_workgroup(launch.problem[w], id - launch.first_workgroup[w], &b, &r, &c)) return false;
+    which = w;
+    batch = uniform_i64(b);
+    tm = uniform_i32(r);
+    tn = uniform_i32(c);
+    return true;
+  };
 
   // Load side.  Wave-level load q (0..7) of this wave fills tile rows
   // [32 q + 8 wave, +8); lane l fills slot l & 7 of row l >> 3 there.
   const int fill_row = lane >> 3;
   const int fill_chunk = (lane & 7) ^ fill_row;
-  uint32_t a_voff[Cfg::kLoadsPerOperand], b_voff[Cfg::kLoadsPerOperand];
-#pragma unroll
-  for (int q = 0; q < Cfg::kLoadsPerOperand; ++q) {
-    const int row = 32 * q + 8 * wave + fill_row;
-    a_voff[q] = static_cast<uint32_t>(row * p.lda * 2 + fill_chunk * 16);
-    b_voff[q] = static_cast<uint32_t>(row * p.ldb * 2 + fill_chunk * 16);
-  }
   // M0 takes the LDS byte address relative to the workgroup's allocation.
   typedef __attribute__((address_space(3))) uint8_t* lds_address;
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_address)lds_bytes));
   const uint32_t fill_lds = lds_base + static_cast<uint32_t>(wave * 1024);  // + q * 4096 (+ operand, + stage)
+  const uint32_t fill_row0 = static_cast<uint32_t>(8 * wave + fill_row);
+  // Operand tile bases of (problem, batch, tile row / column), k-tile 0.
+  auto a_base = [&](int which, int64_t batch, int tm) -> const uint8_t* {
+    const GemmParams& q = launch.problem[which];
+    return uniform_ptr(reinterpret_cast<const uint8_t*>(q.A + batch * q.sA + static_cast<int64_t>(tm) * Cfg::BM * q.lda));
+  };
+  auto b_base = [&](int which, int64_t batch, int tn) -> const uint8_t* {
+    const GemmParams& q = launch.problem[which];
+    return uniform_ptr(reinterpret_cast<const uint8_t*>(q.B + batch * q.sB + static_cast<int64_t>(tn) * Cfg::BN * q.ldb));
+  };
+  auto issue_tile_load = [&](const uint8_t* a_src, const uint8_t* b_src, uint32_t a_row_bytes, uint32_t b_row_bytes,
+                             int stage_off, int q_first, int q_last) {
+#pragma unroll
+    for (int q = q_first; q < q_last; ++q) {
+      dma_load_16((fill_row0 + 32 * q) * a_row_bytes + fill_chunk * 16, a_src, stage_off + fill_lds + q * 4096);
+      dma_load_16((fill_row0 + 32 * q) * b_row_bytes + fill_chunk * 16, b_src,
+                  stage_off + Cfg::kOperandBytes + fill_lds + q * 4096);
+    }
+  };
 
   // Fragment side.  Lane l reads row l & 31 of a 32-row block, k chunk
   // 2 ks + (l >> 5); its slot is that chunk XOR (row & 7), i.e. the ks = 0
@@ -426,13 +454,6 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   }
 
   f32x16 acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
   bf16x8 af[2][TM], bf[2][TN];
   auto read_a = [&](int set, int stage_off, int ks, int i) {
     af[set][i] = *reinterpret_cast<const bf16x8*>(lds_bytes + stage_off + a_frag[ks] + i * 32 * Cfg::kRowBytes);
@@ -449,34 +470,38 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   auto mfma = [&](int set, int i, int j) {
     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[set][j], af[set][i], acc[i][j], 0, 0, 0);
   };
-  auto issue_tile_load = [&](int64_t kt, int stage_off, int q_first, int q_last) {
-    const uint8_t* a_src = Ab + kt * Cfg::kRowBytes;
-    const uint8_t* b_src = Bb + kt * Cfg::kRowBytes;
-#pragma unroll
-    for (int q = q_first; q < q_last; ++q) {
-      dma_load_16(a_voff[q], a_src, stage_off + fill_lds + q * 4096);
-      dma_load_16(b_voff[q], b_src, stage_off + Cfg::kOperandBytes + fill_lds + q * 4096);
-    }
-  };
 
+  // Current tile: plain scalars, reassigned per tile.
+  int which = 0, tm = 0, tn = 0;
+  int64_t batch = 0;
+  int64_t id = blockIdx.x;
+  const int64_t stride = gridDim.x;
+  if (kPersistent) {
+    while (id < launch.total_workgroups && !locate(id, which, batch, tm, tn)) id = uniform_i64(id + stride);
+    if (id >= launch.total_workgroups) return;  // whole workgroup, before any barrier
+  } else if (!locate(id, which, batch, tm, tn)) {
+    return;  // whole workgroup, before any barrier
+  }
+  const uint8_t* Ab = a_base(which, batch, tm);
+  const uint8_t* Bb = b_base(which, batch, tn);
+  uint32_t a_row_bytes = static_cast<uint32_t>(launch.problem[which].lda * 2);
+  uint32_t b_row_bytes = static_cast<uint32_t>(launch.problem[which].ldb * 2);
   FSH_STAMP(1);
-  issue_tile_load(0, 0, 0, Cfg::kLoadsPerOperand);
-  wait_for_dma_loads();
-  __syncthreads();
-  read_frags(0, 0, 0);
-  FSH_STAMP(2);
+  issue_tile_load(Ab, Bb, a_row_bytes, b_row_bytes, 0, 0, Cfg::kLoadsPerOperand);
 
   auto k_tile = [&](int64_t kt, auto more_tag) {
     constexpr bool more = decltype(more_tag)::value;
     const int stage_off = static_cast<int>(kt & 1) * Cfg::kStageBytes;
     const int next_off = stage_off ^ Cfg::kStageBytes;
+    const uint8_t* a_next = Ab + (kt + 1) * Cfg::kRowBytes;
+    const uint8_t* b_next = Bb + (kt + 1) * Cfg::kRowBytes;
     // k step 0: one MFMA, one pair of loads of the next tile, one fragment
     // read of k step 1 at a time.  The other stage is free: every wave passed
     // the barrier that ended the previous tile after its last read of it.
 #pragma unroll
     for (int g = 0; g < TM * TN; ++g) {
       mfma(0, g / TN, g % TN);
-      if (more && g % 2 == 0) issue_tile_load(kt + 1, next_off, g / 2, g / 2 + 1);
+      if (more && g % 2 == 0) issue_tile_load(a_next, b_next, a_row_bytes, b_row_bytes, next_off, g / 2, g / 2 + 1);
       if (g < TM) read_a(1, stage_off, 1, g);
       else if (g < TM + TN) read_b(1, stage_off, 1, g - TM);
       __builtin_amdgcn_sched_barrier(0);
@@ -498,23 +523,57 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
     __syncthreads();
     if (more) read_frags(0, next_off, 0);
   };
-  for (int64_t kt = 0; kt + 1 < ktiles; ++kt) k_tile(kt, std::true_type{});
-  k_tile(ktiles - 1, std::false_type{});
-  FSH_STAMP(3);
 
-  store_whole_tile<Cfg>(p, batch, m0, n0, wm, wn, lane, p.symmetric && tm != tn, acc, lds_bytes);
-  FSH_STAMP(4);
+  while (true) {
+    const GemmParams& p = launch.problem[which];
+    const int64_t ktiles = p.K / Cfg::BK;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    FSH_STAMP(6);
+    wait_for_dma_loads();
+    FSH_STAMP(7);
+    __syncthreads();  // also: every wave has left the previous tile's epilogue
+    read_frags(0, 0, 0);
+    FSH_STAMP(2);
+
+    for (int64_t kt = 0; kt + 1 < ktiles; ++kt) k_tile(kt, std::true_type{});
+    k_tile(ktiles - 1, std::false_type{});
+    FSH_STAMP(3);
+
+    // Both stages are free now.  The next tile's first operands go to stage 0
+    // while the epilogue stages its output beside it, from stage 1 upward.
+    int next_which = 0, next_tm = 0, next_tn = 0;
+    int64_t next_batch = 0;
+    bool have_next = false;
+    if (kPersistent) {
+      id = uniform_i64(id + stride);
+      while (id < launch.total_workgroups && !(have_next = locate(id, next_which, next_batch, next_tm, next_tn)))
+        id = uniform_i64(id + stride);
+      if (have_next) {
+        Ab = a_base(next_which, next_batch, next_tm);
+        Bb = b_base(next_which, next_batch, next_tn);
+        a_row_bytes = static_cast<uint32_t>(launch.problem[next_which].lda * 2);
+        b_row_bytes = static_cast<uint32_t>(launch.problem[next_which].ldb * 2);
+        issue_tile_load(Ab, Bb, a_row_bytes, b_row_bytes, 0, 0, Cfg::kLoadsPerOperand);
+      }
+    }
+    store_tile_in_halves<Cfg>(p, batch, static_cast<int64_t>(tm) * Cfg::BM, static_cast<int64_t>(tn) * Cfg::BN, wm,
+                              wn, lane, p.symmetric && tm != tn, acc, lds_bytes + Cfg::kStageBytes);
+    FSH_STAMP(4);
 #ifdef FSH_TRACE
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  FSH_STAMP(5);
-  if (p.trace && threadIdx.x == 0) {
-    uint32_t hwid;
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-    uint32_t xcc;
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-    p.trace[blockIdx.x * 16 + 6] = (static_cast<uint64_t>(xcc) << 32) | hwid;
-  }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    FSH_STAMP(5);
 #endif
+    if (!have_next) break;
+    which = next_which;
+    batch = next_batch;
+    tm = next_tm;
+    tn = next_tn;
+  }
 }
 
 // A validated problem with its kernel chosen and its tile schedule filled in.
@@ -577,6 +636,7 @@ int plan_gemm(const fsh_gemm_desc& d, PlannedGemm* plan) {
   p.lda = d.lda; p.ldb = d.ldb; p.ldd = d.ldd; p.ldc = d.ldc; p.ldct = d.ldct;
   p.sA = d.stride_a; p.sB = d.stride_b; p.sD = d.stride_d; p.sC = d.stride_c; p.sCt = d.stride_ct;
   p.alpha = d.alpha; p.beta = d.beta;
+  p.diag_add = d.diag_add;
 #ifdef FSH_TRACE
   if (const char* e = getenv("FSH_GEMM_TRACE")) p.trace = reinterpret_cast<uint64_t*>(strtoull(e, nullptr, 0));
 #endif
@@ -585,6 +645,19 @@ int plan_gemm(const fsh_gemm_desc& d, PlannedGemm* plan) {
   const int64_t big_tiles = (d.symmetric ? big_n * (big_n + 1) / 2 : ceil_div(d.m, BigCfg::BM) * big_n) * d.batch;
   if (big_tiles >= 192) return plan_gemm_cfg<BigCfg>(plan, d.batch);
   return plan_gemm_cfg<SmallCfg>(plan, d.batch);
+}
+
+// Compute units of the current device (0 when the query fails).
+int64_t compute_units() {
+  static int cached[64] = {0};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 0;
+  if (cached[device] == 0) {
+    int count = 0;
+    if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return 0;
+    cached[device] = count;
+  }
+  return cached[device];
 }
 
 template <typename Kernel>
@@ -604,8 +677,9 @@ int launch_single(Kernel kernel, bool* reserved, int lds_bytes, int threads, con
 // round of another instead of each launch paying its own tail.  The problems
 // of one call must not depend on each other.
 int launch_planned(PlannedGemm* plans, int count, hipStream_t stream) {
-  static bool reserved_dma = false, reserved_small = false, reserved_edge_big = false, reserved_edge_small = false;
-  constexpr int kDmaLds = max_int(DmaGemm::kLoopLdsBytes, WholeTileEpilogue<DmaGemm>::kLdsBytes);
+  static bool reserved_dma = false, reserved_persistent = false, reserved_small = false, reserved_edge_big = false,
+              reserved_edge_small = false;
+  constexpr int kDmaLds = DmaGemm::kStageBytes + max_int(DmaGemm::kStageBytes, HalfTileEpilogue<DmaGemm>::kLdsBytes);
   int i = 0;
   while (i < count) {
     if (plans[i].kind != kKernelDma) {
@@ -648,12 +722,27 @@ int launch_planned(PlannedGemm* plans, int count, hipStream_t stream) {
         first += plans[order[k]].workgroups;
       }
     }
-    if (!reserved_dma) {
-      if (int rc = reserve_lds(&gemm_nt_dma_kernel, kDmaLds)) return rc;
-      reserved_dma = true;
+    launch.total_workgroups = static_cast<int32_t>(total);
+    // Equally long tiles and more of them than compute units: one resident
+    // workgroup per compute unit walks a static schedule.
+    bool equal_k = true;
+    for (int k = 1; k < n; ++k) equal_k = equal_k && plans[order[k]].p.K == plans[order[0]].p.K;
+    const int64_t units = compute_units();
+    if (equal_k && units >= kXcds && units % kXcds == 0 && total > units) {
+      if (!reserved_persistent) {
+        if (int rc = reserve_lds(&gemm_nt_dma_kernel<true>, kDmaLds)) return rc;
+        reserved_persistent = true;
+      }
+      hipLaunchKernelGGL(gemm_nt_dma_kernel<true>, dim3(static_cast<uint32_t>(units)), dim3(DmaGemm::kThreads),
+                         kDmaLds, stream, launch);
+    } else {
+      if (!reserved_dma) {
+        if (int rc = reserve_lds(&gemm_nt_dma_kernel<false>, kDmaLds)) return rc;
+        reserved_dma = true;
+      }
+      hipLaunchKernelGGL(gemm_nt_dma_kernel<false>, dim3(static_cast<uint32_t>(total)), dim3(DmaGemm::kThreads),
+                         kDmaLds, stream, launch);
     }
-    hipLaunchKernelGGL(gemm_nt_dma_kernel, dim3(static_cast<uint32_t>(total)), dim3(DmaGemm::kThreads), kDmaLds,
-                       stream, launch);
     if (int rc = check_launch("gemm_nt_dma_kernel")) return rc;
   }
   return FSH_OK;
@@ -868,9 +957,11 @@ int ns_begin(const fsh_ns_problem& q, int32_t steps, float eps, hipStream_t stre
   return check_launch("normalize_dual_kernel");
 }
 
-// The three products of one iteration; `which` = 0: G = X X^T, 1: P = b G +
-// c G G (symmetric because G is), 2: X' = a X + P X, also written transposed
-// into the other X^T buffer.
+// The three products of one iteration; `which` = 0: G = X X^T, 1: P = a I +
+// b G + c G G (symmetric because G is), 2: X' = P X = a X + (b G + c G G) X,
+// also written transposed into the other X^T buffer.  Carrying `a` on P's
+// diagonal (added in fp32 before P is rounded) spares the last product a
+// read of X from HBM per output tile.
 fsh_gemm_desc ns_product(const NsState& st, int which, float a, float b, float c) {
   const int64_t s = st.s, l = st.l, sl = s * l, ss = s * s;
   fsh_gemm_desc g;
@@ -887,12 +978,13 @@ fsh_gemm_desc ns_product(const NsState& st, int which, float a, float b, float c
     g.m = s; g.n = s; g.k = s; g.lda = s; g.ldb = s; g.ldd = s; g.ldc = s;
     g.stride_a = ss; g.stride_b = ss; g.stride_d = ss; g.stride_c = ss;
     g.alpha = c; g.beta = b;
+    g.diag_add = a;
     g.symmetric = 1;
   } else {
-    g.a_dev = st.P; g.b_dev = st.XT[st.cur]; g.d_dev = st.X; g.c_dev = st.X; g.ct_dev = st.XT[st.cur ^ 1];
-    g.m = s; g.n = l; g.k = s; g.lda = s; g.ldb = s; g.ldd = l; g.ldc = l; g.ldct = s;
-    g.stride_a = ss; g.stride_b = sl; g.stride_d = sl; g.stride_c = sl; g.stride_ct = sl;
-    g.alpha = 1.0f; g.beta = a;
+    g.a_dev = st.P; g.b_dev = st.XT[st.cur]; g.c_dev = st.X; g.ct_dev = st.XT[st.cur ^ 1];
+    g.m = s; g.n = l; g.k = s; g.lda = s; g.ldb = s; g.ldc = l; g.ldct = s;
+    g.stride_a = ss; g.stride_b = sl; g.stride_c = sl; g.stride_ct = sl;
+    g.alpha = 1.0f; g.beta = 0.0f;
   }
   return g;
 }

@@ -353,7 +353,7 @@ def newton_schulz_multi(
 
 def _gemm_desc(
     a: torch.Tensor, b: torch.Tensor, d: torch.Tensor | None, alpha: float, beta: float,
-    out: torch.Tensor | None, out_t: torch.Tensor | None, symmetric: bool,
+    out: torch.Tensor | None, out_t: torch.Tensor | None, symmetric: bool, diag_add: float = 0.0,
 ) -> tuple["_native.GemmDesc", torch.Tensor]:
     _require_gpu(a, b)
     if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16 or not a.is_contiguous() or not b.is_contiguous():
@@ -384,18 +384,20 @@ def _gemm_desc(
     desc.stride_d = desc.stride_c = desc.stride_ct = m * n
     desc.alpha, desc.beta = alpha, beta
     desc.symmetric = 1 if symmetric else 0
+    desc.diag_add = diag_add
     return desc, out
 
 
 def gemm_nt(
     a: torch.Tensor, b: torch.Tensor, *, d: torch.Tensor | None = None, alpha: float = 1.0, beta: float = 0.0,
     out: torch.Tensor | None = None, out_t: torch.Tensor | None = None, symmetric: bool = False,
+    diag_add: float = 0.0,
 ) -> torch.Tensor:
-    """``bf16(alpha * a @ b^T + beta * d)`` for contiguous bf16 [batch, m, k] /
-    [batch, n, k] (or 2-D) operands; optionally also the transpose.  With
-    ``symmetric`` the caller guarantees a symmetric result (m == n); only the
-    upper triangle of tiles is computed and mirrored."""
-    desc, out = _gemm_desc(a, b, d, alpha, beta, out, out_t, symmetric)
+    """``bf16(alpha * a @ b^T + beta * d + diag_add * I)`` for contiguous bf16
+    [batch, m, k] / [batch, n, k] (or 2-D) operands; optionally also the
+    transpose.  With ``symmetric`` the caller guarantees a symmetric result
+    (m == n); only the upper triangle of tiles is computed and mirrored."""
+    desc, out = _gemm_desc(a, b, d, alpha, beta, out, out_t, symmetric, diag_add)
     status = _native.lib().fsh_gemm_bf16_nt(ctypes.byref(desc), stream_ptr(a.device))
     _native.check(status, "fsh_gemm_bf16_nt")
     return out
@@ -411,7 +413,7 @@ def gemm_nt_group(problems: Sequence[dict]) -> list[torch.Tensor]:
     for i, q in enumerate(problems):
         desc, out = _gemm_desc(
             q["a"], q["b"], q.get("d"), q.get("alpha", 1.0), q.get("beta", 0.0), q.get("out"), q.get("out_t"),
-            q.get("symmetric", False),
+            q.get("symmetric", False), q.get("diag_add", 0.0),
         )
         descs[i] = desc
         outs.append(out)

@@ -203,7 +203,7 @@ int fsh_newton_schulz_multi(const fsh_ns_problem* problems, int32_t count, float
                             int32_t steps, float eps, void* stream);
 
 /* Batched bf16 "NT" GEMM, the building block of (6), exported for tests:
- *   C[b] = bf16(alpha * A[b] . B[b]^T + beta * D[b])      fp32 accumulation
+ *   C[b] = bf16(alpha * A[b] . B[b]^T + beta * D[b] + diag_add * I)   fp32 accumulation
  * A is [m, k] with row stride lda, B is [n, k] with row stride ldb (both
  * k-contiguous), D and C are [m, n] with row strides ldd / ldc.  D may be NULL
  * (beta ignored) or alias C.  ct_dev, when not NULL, also receives C[b]^T as
@@ -224,7 +224,7 @@ typedef struct fsh_gemm_desc {
   int32_t symmetric; /* nonzero: the caller guarantees a symmetric result (m == n, e.g. b == a
                         and d symmetric); only the tiles on or above the diagonal are
                         computed and the rest is mirrored.  ct_dev must be null. */
-  int32_t reserved;  /* 0 */
+  float diag_add;    /* added to C[b][i][i] in fp32 before the rounding to bf16 (0: plain product) */
 } fsh_gemm_desc;
 int fsh_gemm_bf16_nt(const fsh_gemm_desc* desc, void* stream);
 /* `count` independent products; those that qualify for the large-tile kernel

@@ -411,6 +411,32 @@ def test_gemm_symmetric_mode_mirrors_the_upper_triangle(device, batch, n, k):
         hip_ops.gemm_nt(a, a[:, : n - 8].contiguous(), symmetric=True)
 
 
+@pytest.mark.parametrize(
+    "batch,n,k,symmetric",
+    [(10, 1536, 128, True), (7, 1536, 192, False), (1, 512, 96, True), (3, 264, 72, False)],
+)
+def test_gemm_diagonal_addend(device, batch, n, k, symmetric):
+    """C = alpha A B^T + beta D + diag_add I on every kernel: the addend enters
+    in fp32 before the one rounding, on the diagonal only (this is how the
+    iteration carries `a X` inside `P X`)."""
+    gen = torch.Generator().manual_seed(n + k)
+    a = torch.randn(batch, n, k, generator=gen).bfloat16().to(device)
+    b = a if symmetric else torch.randn(batch, n, k, generator=gen).bfloat16().to(device)
+    d = torch.randn(batch, n, n, generator=gen).bfloat16().to(device)
+    if symmetric:
+        d = torch.triu(d) + torch.triu(d, 1).transpose(1, 2)
+    plain = hip_ops.gemm_nt(a, b, d=d, alpha=0.25, beta=-0.5, symmetric=symmetric)
+    shifted = hip_ops.gemm_nt(a, b, d=d, alpha=0.25, beta=-0.5, symmetric=symmetric, diag_add=3.4445)
+    eye = torch.eye(n, dtype=torch.bool, device=device).expand(batch, n, n)
+    assert torch.equal(shifted[~eye], plain[~eye])
+    ref = _gemm_reference(a, b, d, 0.25, -0.5) + 3.4445 * torch.eye(n, dtype=torch.float64)
+    assert torch.allclose(shifted.cpu().double(), ref, rtol=2.0**-8, atol=2e-2)
+    # one rounding: the diagonal is within about half a bf16 ulp of the exact value
+    want = ref[eye.cpu()]
+    ulp = torch.exp2(torch.floor(torch.log2(want.abs())) - 7)
+    assert ((shifted[eye].cpu().double() - want).abs() <= 0.51 * ulp + 1e-3).all()
+
+
 def test_gemm_group_equals_separate_calls(device):
     """Problems of different shapes and kernels in one call: the ones on the
     large-tile kernel share a launch (longest k first), every result is bit
@@ -454,6 +480,39 @@ def test_gemm_group_equals_separate_calls(device):
     for buf in buffers:
         assert (buf[:pad] == 7).all() and (buf[-pad:] == 7).all()
     assert hip_ops.gemm_nt_group([]) == []
+
+
+def test_gemm_static_schedule_when_tiles_are_equally_long(device):
+    """More large tiles than compute units, all with the same k: one resident
+    workgroup per compute unit walks the tiles of both problems (next tile's
+    operands requested during the epilogue).  Against fp64 and against the
+    symmetric / transposed identities, with guard bands."""
+    gen = torch.Generator().manual_seed(33)
+    batch, m, n, k = 11, 1536, 1792, 192  # 6 x 7 x 11 = 462 tiles
+    a = torch.randn(batch, m, k, generator=gen).bfloat16().to(device)
+    b = torch.randn(batch, n, k, generator=gen).bfloat16().to(device)
+    d = torch.randn(batch, m, n, generator=gen).bfloat16().to(device)
+    s = torch.randn(9, 1280, k, generator=gen).bfloat16().to(device)  # 15 x 9 = 135 symmetric tiles
+    pad = 4096
+    c_buf = torch.full((batch * m * n + 2 * pad,), 7.0, dtype=torch.bfloat16, device=device)
+    t_buf = torch.full((batch * m * n + 2 * pad,), 7.0, dtype=torch.bfloat16, device=device)
+    s_buf = torch.full((9 * 1280 * 1280 + 2 * pad,), 7.0, dtype=torch.bfloat16, device=device)
+    c, ct, sc = c_buf[pad:-pad].view(batch, m, n), t_buf[pad:-pad].view(batch, n, m), s_buf[pad:-pad].view(9, 1280, 1280)
+    hip_ops.gemm_nt_group([
+        dict(a=a, b=b, d=d, alpha=0.5, beta=2.0, out=c, out_t=ct),
+        dict(a=s, b=s, alpha=1.0, symmetric=True, out=sc),
+    ])
+    ref = _gemm_reference(a, b, d, 0.5, 2.0)
+    assert torch.allclose(c.cpu().double(), ref, rtol=2.0**-8, atol=2e-2)
+    assert torch.equal(ct, c.transpose(1, 2).contiguous())
+    assert torch.equal(sc, sc.transpose(1, 2))
+    assert torch.allclose(sc.cpu().double(), _gemm_reference(s, s), rtol=2.0**-8, atol=2e-2)
+    for buf in (c_buf, t_buf, s_buf):
+        assert (buf[:pad] == 7).all() and (buf[-pad:] == 7).all()
+    # in place, as the iteration uses it: X' = a X + P X with C = D
+    x = d.clone()
+    hip_ops.gemm_nt(a, b, d=x, alpha=0.5, beta=2.0, out=x)
+    assert torch.equal(x, c)
 
 
 def test_newton_schulz_multi_equals_one_call_per_shape(device):
