@@ -372,7 +372,14 @@ struct DmaGemm {
   static constexpr int kStageBytes = 2 * kOperandBytes;      // 64 KB
   static constexpr int kLoopLdsBytes = 2 * kStageBytes;
   static constexpr int kLoadsPerOperand = BM / 8 / 4;        // wave-level 1 KB loads per wave: 8
+  static constexpr int kTouchAhead = 3;                      // k-tiles between an L2 touch and its use
+  static constexpr int kScrapBytes = 1024;                   // landing area of the touches, 256 B per wave
 };
+
+// LDS of the kernel: two operand stages, the epilogue's staging region from
+// stage 1 upward, and the touches' scrap area at the very end.
+constexpr int kDmaGemmLdsBytes =
+    DmaGemm::kStageBytes + max_int(DmaGemm::kStageBytes, HalfTileEpilogue<DmaGemm>::kLdsBytes) + DmaGemm::kScrapBytes;
 
 // kPersistent: the grid is one workgroup per compute unit and workgroup g
 // takes the ids g, g + gridDim.x, ... of the launch (the same XCD every time,
@@ -452,6 +459,7 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
     a_frag[ks] = (frag_base ^ (ks * 32)) + wm * Cfg::kWaveM * Cfg::kRowBytes;
     b_frag[ks] = (frag_base ^ (ks * 32)) + Cfg::kOperandBytes + wn * Cfg::kWaveN * Cfg::kRowBytes;
   }
+  constexpr int scrap_offset = kDmaGemmLdsBytes - Cfg::kScrapBytes;
 
   f32x16 acc[TM][TN];
   bf16x8 af[2][TM], bf[2][TN];
@@ -489,12 +497,22 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   FSH_STAMP(1);
   issue_tile_load(Ab, Bb, a_row_bytes, b_row_bytes, 0, 0, Cfg::kLoadsPerOperand);
 
-  auto k_tile = [&](int64_t kt, auto more_tag) {
+  // L2 touches.  A k-tile's operands are requested one k-tile (about 2 us)
+  // before they are needed, which a miss to HBM does not always make; so three
+  // k-tiles ahead each lane asks for 4 bytes of one operand row (one 128-byte
+  // line each: 256 rows of A and of B = two requests per wave), which brings
+  // the lines into L2 and makes the real request a hit.  The touches are
+  // issued after the k-tile's real requests and may still be in flight when
+  // those are waited for (requests complete in order).
+  const uint32_t touch_row = static_cast<uint32_t>(64 * wave + lane);
+  const uint32_t scrap_lds = lds_base + static_cast<uint32_t>(scrap_offset + wave * 256);
+  auto k_tile = [&](int64_t kt, int64_t ktiles, auto more_tag) {
     constexpr bool more = decltype(more_tag)::value;
     const int stage_off = static_cast<int>(kt & 1) * Cfg::kStageBytes;
     const int next_off = stage_off ^ Cfg::kStageBytes;
     const uint8_t* a_next = Ab + (kt + 1) * Cfg::kRowBytes;
     const uint8_t* b_next = Bb + (kt + 1) * Cfg::kRowBytes;
+    const bool touch = more && kt + Cfg::kTouchAhead < ktiles;
     // k step 0: one MFMA, one pair of loads of the next tile, one fragment
     // read of k step 1 at a time.  The other stage is free: every wave passed
     // the barrier that ended the previous tile after its last read of it.
@@ -505,6 +523,10 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
       if (g < TM) read_a(1, stage_off, 1, g);
       else if (g < TM + TN) read_b(1, stage_off, 1, g - TM);
       __builtin_amdgcn_sched_barrier(0);
+    }
+    if (touch) {
+      dma_touch_4(touch_row * a_row_bytes, Ab + (kt + Cfg::kTouchAhead) * Cfg::kRowBytes, scrap_lds);
+      dma_touch_4(touch_row * b_row_bytes, Bb + (kt + Cfg::kTouchAhead) * Cfg::kRowBytes, scrap_lds);
     }
 #pragma unroll
     for (int ks = 1; ks < KS; ++ks) {
@@ -519,7 +541,10 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
         }
       }
     }
-    if (more) wait_for_dma_loads();  // this wave's part of the next tile has landed
+    if (more) {  // this wave's part of the next tile has landed
+      if (touch) wait_for_dma_loads_except<2>();
+      else wait_for_dma_loads();
+    }
     __syncthreads();
     if (more) read_frags(0, next_off, 0);
   };
@@ -540,8 +565,8 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
     read_frags(0, 0, 0);
     FSH_STAMP(2);
 
-    for (int64_t kt = 0; kt + 1 < ktiles; ++kt) k_tile(kt, std::true_type{});
-    k_tile(ktiles - 1, std::false_type{});
+    for (int64_t kt = 0; kt + 1 < ktiles; ++kt) k_tile(kt, ktiles, std::true_type{});
+    k_tile(ktiles - 1, ktiles, std::false_type{});
     FSH_STAMP(3);
 
     // Both stages are free now.  The next tile's first operands go to stage 0
@@ -679,7 +704,7 @@ int launch_single(Kernel kernel, bool* reserved, int lds_bytes, int threads, con
 int launch_planned(PlannedGemm* plans, int count, hipStream_t stream) {
   static bool reserved_dma = false, reserved_persistent = false, reserved_small = false, reserved_edge_big = false,
               reserved_edge_small = false;
-  constexpr int kDmaLds = DmaGemm::kStageBytes + max_int(DmaGemm::kStageBytes, HalfTileEpilogue<DmaGemm>::kLdsBytes);
+  constexpr int kDmaLds = kDmaGemmLdsBytes;
   int i = 0;
   while (i < count) {
     if (plans[i].kind != kKernelDma) {
