@@ -131,6 +131,12 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     ),
     "fsh_gemm_bf16_nt": (c_int, [POINTER(GemmDesc), c_void_p]),
     "fsh_gemm_bf16_nt_group": (c_int, [POINTER(GemmDesc), c_int32, c_void_p]),
+    "fsh_act_quant_1x128": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int32, c_void_p]),
+    "fsh_fp8_gemm_1x128_128x128": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+         c_void_p],
+    ),
     "fsh_muon_prepare": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_float, c_float, c_int32, c_void_p]),
     "fsh_muon_apply": (c_int, [c_void_p, c_void_p, c_int64, c_float, c_float, c_float, c_void_p]),
 }

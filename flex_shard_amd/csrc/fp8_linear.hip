@@ -1,0 +1,388 @@
+// Forward GEMM of a linear layer whose weight arrives already quantized
+// (128x128 tiles, FP8 E4M3FN) from the bucket unpack: 1x128 quantization of
+// the activation and the FP8 product with both sets of scales.
+//
+//   xq, xs = quantize each run of 128 consecutive elements of a row of x
+//            (amax floored at 1e-12, scale = fp32(448 / fp64(amax)),
+//            q = e4m3fn(fp32(x) * scale), stored scale = 1.0f / scale)
+//   out[m][n] = bf16( sum over k-blocks kb of
+//                     dot(xq[m][kb], wq[n][kb]) * (xs[kb][m] * ws[n / 128][kb]) )
+//
+// Matrix cores: v_mfma_f32_32x32x64_f8f6f4 (64 FP8 products per lane pair and
+// instruction, twice the rate of the 32x32x16 FP8 form on gfx950).  A k-tile
+// is one scale block (128 bytes of each row), so its partial products are
+// accumulated from zero in a scratch accumulator and folded into the result
+// with one fused multiply-add per element; the folds of one 32x32 block run
+// on the vector ALU while the matrix core works on the next.
+#include "mfma_tiles.hpp"
+
+namespace fsh {
+namespace {
+
+// ------------------------------------------------------------ 1x128 quantize
+// A workgroup owns 64 rows x 512 columns (4 scale blocks per row).  Sixteen
+// lanes own one run of 128 elements (16 bytes each); a wavefront load covers
+// four runs = 1 KB of one row.  All sixteen loads of a thread are issued
+// before the first is used.  The maximum of a run stays inside its row of 16
+// lanes (four DPP steps, no LDS, no barrier).  Scales go through LDS so that
+// they leave as 256-byte runs of the [k-block][row] table.
+constexpr int kActThreads = 256;
+constexpr int kActRows = 64;
+constexpr int kActBlocks = 4;  // 128-element runs per row and workgroup
+constexpr int kActPasses = kActRows * kActBlocks * 16 / kActThreads;
+
+struct ActQuantParams {
+  const uint8_t* x;
+  uint8_t* q;
+  float* scales;
+  int64_t rows, cols, ldx, ldq;  // elements; ldq = cols rounded up to 128
+  int32_t col_groups;            // ceil(ceil(cols / 128) / 4)
+  float eps;
+};
+
+__device__ __forceinline__ uint32_t row16_max_u32(uint32_t v) {
+  v = dpp_max_u32<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
+  v = dpp_max_u32<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
+  v = dpp_max_u32<0x141, 0xF>(v);  // row_half_mirror
+  v = dpp_max_u32<0x140, 0xF>(v);  // row_mirror
+  return v;
+}
+
+__global__ __launch_bounds__(kActThreads) void act_quant_1x128_kernel(const ActQuantParams p) {
+  __shared__ float lds_scales[kActBlocks * kActRows];
+  const int tid = threadIdx.x;
+  const int sub = tid & 15, run_lane = tid >> 4;
+  const int64_t tile_r = blockIdx.x / p.col_groups, tile_c = blockIdx.x % p.col_groups;
+  const int64_t row0 = tile_r * kActRows, kb0 = tile_c * kActBlocks;
+
+  u32x4 v[kActPasses];
+#pragma unroll
+  for (int pass = 0; pass < kActPasses; ++pass) {
+    const int run = pass * 16 + run_lane;  // 0..255 within the tile
+    const int64_t row = row0 + run / kActBlocks;
+    const int64_t col = (kb0 + run % kActBlocks) * 128 + sub * 8;
+    v[pass] = u32x4{0, 0, 0, 0};
+    if (row < p.rows && col < p.cols) v[pass] = load_stream_u32x4(p.x + (row * p.ldx + col) * 2);
+  }
+#pragma unroll
+  for (int pass = 0; pass < kActPasses; ++pass) {
+    const int run = pass * 16 + run_lane;
+    const int64_t row = row0 + run / kActBlocks;
+    const int64_t col = (kb0 + run % kActBlocks) * 128 + sub * 8;
+    uint32_t m = pk_max_u16(v[pass].x & 0x7FFF7FFFu, v[pass].y & 0x7FFF7FFFu);
+    m = pk_max_u16(m, v[pass].z & 0x7FFF7FFFu);
+    m = pk_max_u16(m, v[pass].w & 0x7FFF7FFFu);
+    const uint32_t lo = m & 0xFFFFu, hi = m >> 16;
+    m = row16_max_u32(lo > hi ? lo : hi);
+    float scale, recip;
+    tile_scale(bf16_bits_to_f32(m), p.eps, scale, recip);
+    if (sub == 0) lds_scales[(run % kActBlocks) * kActRows + run / kActBlocks] = recip;
+    if (row < p.rows && col < p.ldq) {
+      const uint32_t d[4] = {v[pass].x, v[pass].y, v[pass].z, v[pass].w};
+      uint32_t w[2] = {0, 0};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float e0 = u32_as_f32(d[j] << 16) * scale;
+        const float e1 = u32_as_f32(d[j] & 0xFFFF0000u) * scale;
+        w[j >> 1] = cvt2_fp8(e0, e1, w[j >> 1], (j & 1) != 0);
+      }
+      store_stream_u32x2(p.q + row * p.ldq + col, w[0], w[1]);
+    }
+  }
+  __syncthreads();
+  {
+    const int kbl = tid / kActRows, r = tid % kActRows;
+    const int64_t kb = kb0 + kbl, row = row0 + r;
+    if (row < p.rows && kb * 128 < p.ldq) p.scales[kb * p.rows + row] = lds_scales[tid];
+  }
+}
+
+// ----------------------------------------------------------------- FP8 GEMM
+// 128 x 256 output tile per workgroup, four waves of 64 x 128 (two by four
+// 32x32 blocks).  Operand tiles are 128 bytes per row and k-tile and travel
+// global -> LDS directly, 16-byte chunk c of row r in slot c ^ (r & 7), two
+// stages.  A lane feeds the matrix core bytes [32 h, 32 h + 32) of each half
+// of its row (h = lane / 32), i.e. chunks 2h and 2h+1 of a 64-byte half.
+struct Fp8Gemm {
+  static constexpr int BM = 128, BN = 256, BK = 128, WM = 2, WN = 2, TM = 2, TN = 4;
+  static constexpr int kThreads = 256, kWaveM = 64, kWaveN = 128;
+  static constexpr int kRowBytes = 128;
+  static constexpr int kABytes = BM * kRowBytes;               // 16 KB
+  static constexpr int kStageBytes = (BM + BN) * kRowBytes;    // 48 KB
+  static constexpr int kLoadsA = BM / 8 / 4, kLoadsB = BN / 8 / 4;  // per wave: 4 and 8
+  static constexpr int kPitch = kWaveN * 2 + 8;                // epilogue staging, bytes
+  static constexpr int kRegion = kWaveM * kPitch;              // per wave
+  static constexpr int kLdsBytes = max_int(2 * kStageBytes, 4 * kRegion);
+};
+
+struct Fp8GemmParams {
+  const uint8_t* xq;
+  const float* xs;   // [k / 128][m]
+  const uint8_t* wq;
+  const float* ws;   // [ceil(n / 128)][ws_cols]
+  uint16_t* out;
+  int64_t m, n, k;
+  int64_t ldxq, ldwq, ldo, ws_cols;
+  GemmParams schedule;  // tile order only
+};
+
+typedef int v8i32 __attribute__((ext_vector_type(8)));
+
+__global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(const Fp8GemmParams p) {
+  using Cfg = Fp8Gemm;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds_bytes[];
+  constexpr int TM = Cfg::TM, TN = Cfg::TN;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+  int64_t unused_batch;
+  int tm, tn;
+  if (!tile_of_workgroup(p.schedule, blockIdx.x, &unused_batch, &tm, &tn)) return;  // whole workgroup
+  tm = uniform_i32(tm);
+  tn = uniform_i32(tn);
+  const int64_t m0 = static_cast<int64_t>(tm) * Cfg::BM, n0 = static_cast<int64_t>(tn) * Cfg::BN;
+  const int64_t ktiles = p.k / Cfg::BK;
+
+  // Load side: wave-level load q of a wave fills tile rows [32 q + 8 wave, +8);
+  // lane l fills slot l & 7 of row l >> 3 there.  Rows past the matrix are
+  // read from its last row (their products are never stored).
+  const int fill_row = lane >> 3;
+  const int fill_chunk = (lane & 7) ^ fill_row;
+  uint32_t a_voff[Cfg::kLoadsA], b_voff[Cfg::kLoadsB];
+#pragma unroll
+  for (int q = 0; q < Cfg::kLoadsA; ++q) {
+    int64_t row = m0 + 32 * q + 8 * wave + fill_row;
+    row = row < p.m ? row : p.m - 1;
+    a_voff[q] = static_cast<uint32_t>((row - m0) * p.ldxq + fill_chunk * 16);
+  }
+#pragma unroll
+  for (int q = 0; q < Cfg::kLoadsB; ++q) {
+    int64_t row = n0 + 32 * q + 8 * wave + fill_row;
+    row = row < p.n ? row : p.n - 1;
+    b_voff[q] = static_cast<uint32_t>((row - n0) * p.ldwq + fill_chunk * 16);
+  }
+  const uint8_t* Ab = uniform_ptr(p.xq + m0 * p.ldxq);
+  const uint8_t* Bb = uniform_ptr(p.wq + n0 * p.ldwq);
+  typedef __attribute__((address_space(3))) uint8_t* lds_address;
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_address)lds_bytes));
+  const uint32_t fill_lds = lds_base + static_cast<uint32_t>(wave * 1024);
+  auto issue_tile_load = [&](int64_t kt, int stage_off) {
+    const uint8_t* a_src = Ab + kt * Cfg::kRowBytes;
+    const uint8_t* b_src = Bb + kt * Cfg::kRowBytes;
+#pragma unroll
+    for (int q = 0; q < Cfg::kLoadsA; ++q) dma_load_16(a_voff[q], a_src, stage_off + fill_lds + q * 4096);
+#pragma unroll
+    for (int q = 0; q < Cfg::kLoadsB; ++q)
+      dma_load_16(b_voff[q], b_src, stage_off + Cfg::kABytes + fill_lds + q * 4096);
+  };
+
+  // Fragment side: row = lane & 31 of a 32-row block; chunks 4 kh + 2 h and
+  // 4 kh + 2 h + 1 of the row (kh = 64-byte half), each in slot chunk ^ (row & 7).
+  const int frag_row = lane & 31, h = lane >> 5;
+  uint32_t frag_off[2][2];
+#pragma unroll
+  for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+      frag_off[kh][c] = static_cast<uint32_t>(frag_row * Cfg::kRowBytes + (((4 * kh + 2 * h + c) ^ (frag_row & 7)) * 16));
+  auto read_frag = [&](int stage_off, int operand_off, int block, int kh) -> v8i32 {
+    const uint8_t* base = lds_bytes + stage_off + operand_off + block * 32 * Cfg::kRowBytes;
+    const u32x4 lo = *reinterpret_cast<const u32x4*>(base + frag_off[kh][0]);
+    const u32x4 hi = *reinterpret_cast<const u32x4*>(base + frag_off[kh][1]);
+    return v8i32{static_cast<int>(lo.x), static_cast<int>(lo.y), static_cast<int>(lo.z), static_cast<int>(lo.w),
+                 static_cast<int>(hi.x), static_cast<int>(hi.y), static_cast<int>(hi.z), static_cast<int>(hi.w)};
+  };
+
+  // Scales: a lane owns output row lane & 31 of each of its two 32-row blocks,
+  // so it needs xs[kb][row] for two rows and the one weight scale of the
+  // wave's 128 columns.
+  int64_t srow[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int64_t row = m0 + wm * Cfg::kWaveM + i * 32 + frag_row;
+    srow[i] = row < p.m ? row : p.m - 1;
+  }
+  const int64_t wcol = n0 + wn * Cfg::kWaveN;
+  const int64_t wblock = (wcol < p.n ? wcol : p.n - 1) / 128;
+  const float* ws_row = p.ws + wblock * p.ws_cols;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  issue_tile_load(0, 0);
+  float xs_next[TM], ws_next;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) xs_next[i] = p.xs[srow[i]];
+  ws_next = ws_row[0];
+  wait_for_dma_loads();
+  __syncthreads();
+
+  for (int64_t kt = 0; kt < ktiles; ++kt) {
+    const int stage_off = static_cast<int>(kt & 1) * Cfg::kStageBytes;
+    const bool more = kt + 1 < ktiles;
+    if (more) issue_tile_load(kt + 1, stage_off ^ Cfg::kStageBytes);
+    float s[TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) s[i] = xs_next[i] * ws_next;
+    if (more) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) xs_next[i] = p.xs[(kt + 1) * p.m + srow[i]];
+      ws_next = ws_row[kt + 1];
+    }
+    v8i32 bfrag[TN][2];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int kh = 0; kh < 2; ++kh) bfrag[j][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32) + j, kh);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      v8i32 afrag[2];
+#pragma unroll
+      for (int kh = 0; kh < 2; ++kh) afrag[kh] = read_frag(stage_off, 0, wm * (Cfg::kWaveM / 32) + i, kh);
+      f32x16 part[TN];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        part[j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j][0], afrag[0], zero, 0, 0, 0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        part[j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j][1], afrag[1], part[j], 0, 0, 0, 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = __builtin_fmaf(part[j][r], s[i], acc[i][j][r]);
+    }
+    if (more) wait_for_dma_loads();
+    __syncthreads();
+  }
+
+  // Epilogue: bf16 finals to the wave's staging region as [row][col], then
+  // 16-byte row stores, rows and 8-column groups past the matrix skipped.
+  uint8_t* region = lds_bytes + wave * Cfg::kRegion;
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+        *reinterpret_cast<u32x2*>(region + (i * 32 + frag_row) * Cfg::kPitch + (j * 32 + 8 * b + 4 * h) * 2) =
+            u32x2{pack_bf16x2(acc[i][j][4 * b], acc[i][j][4 * b + 1]),
+                  pack_bf16x2(acc[i][j][4 * b + 2], acc[i][j][4 * b + 3])};
+  wave_lds_sync();
+  {
+    constexpr int kLanesPerRow = Cfg::kWaveN * 2 / 16, kRowsPerPass = 64 / kLanesPerRow;
+    const int r0 = lane / kLanesPerRow, chunk = lane % kLanesPerRow;
+    const int64_t wave_row = m0 + wm * Cfg::kWaveM, col = n0 + wn * Cfg::kWaveN + chunk * 8;
+    const bool vec_ok = (p.ldo % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+#pragma unroll
+    for (int pass = 0; pass < Cfg::kWaveM / kRowsPerPass; ++pass) {
+      const int r = pass * kRowsPerPass + r0;
+      const int64_t row = wave_row + r;
+      if (row >= p.m || col >= p.n) continue;
+      const uint8_t* src = region + r * Cfg::kPitch + chunk * 16;
+      const u32x2 lo = *reinterpret_cast<const u32x2*>(src);
+      const u32x2 hi = *reinterpret_cast<const u32x2*>(src + 8);
+      uint16_t* dst = p.out + row * p.ldo + col;
+      if (vec_ok && col + 8 <= p.n) {
+        *reinterpret_cast<u32x4*>(dst) = u32x4{lo.x, lo.y, hi.x, hi.y};
+      } else {
+        const uint32_t w[4] = {lo.x, lo.y, hi.x, hi.y};
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (col + e < p.n) dst[e] = static_cast<uint16_t>(w[e >> 1] >> (16 * (e & 1)));
+      }
+    }
+  }
+}
+
+}  // namespace
+}  // namespace fsh
+
+FSH_API int fsh_act_quant_1x128(const void* x_dev, int64_t rows, int64_t cols, int64_t ldx, void* q_dev,
+                                int64_t ldq, float* scales_dev, int32_t eps_mode, void* stream) {
+  using namespace fsh;
+  if (rows < 0 || cols < 0) return fail(FSH_EINVAL, "fsh_act_quant_1x128: negative shape");
+  if (rows == 0 || cols == 0) return FSH_OK;
+  if (!x_dev || !q_dev || !scales_dev) return fail(FSH_EINVAL, "fsh_act_quant_1x128: null pointer");
+  if (eps_mode != FSH_EPS_INPUT_DTYPE && eps_mode != FSH_EPS_FP32)
+    return fail(FSH_EINVAL, "fsh_act_quant_1x128: unknown eps_mode %d", eps_mode);
+  const int64_t padded = ceil_div(cols, (int64_t)128) * 128;
+  if (ldx < cols || ldq != padded)
+    return fail(FSH_EINVAL, "fsh_act_quant_1x128: ldx %lld < cols %lld, or ldq %lld is not cols rounded up to 128 (%lld)",
+                (long long)ldx, (long long)cols, (long long)ldq, (long long)padded);
+  if (cols % 8 || ldx % 8 || !aligned(x_dev, 16) || !aligned(q_dev, 8) || !aligned(scales_dev, 4))
+    return fail(FSH_ENOTSUP, "fsh_act_quant_1x128: cols and ldx must be multiples of 8, x 16-byte and q 8-byte aligned");
+  ActQuantParams p;
+  p.x = static_cast<const uint8_t*>(x_dev);
+  p.q = static_cast<uint8_t*>(q_dev);
+  p.scales = scales_dev;
+  p.rows = rows;
+  p.cols = cols;
+  p.ldx = ldx;
+  p.ldq = ldq;
+  const int64_t col_groups = ceil_div(padded / 128, (int64_t)kActBlocks);
+  p.col_groups = static_cast<int32_t>(col_groups);
+  const float eps32 = 1e-12f;
+  uint32_t bits;
+  memcpy(&bits, &eps32, 4);
+  bits = (bits + 0x7FFFu + ((bits >> 16) & 1u)) & 0xFFFF0000u;
+  float eps_bf16;
+  memcpy(&eps_bf16, &bits, 4);
+  p.eps = eps_mode == FSH_EPS_FP32 ? eps32 : eps_bf16;
+  const int64_t grid = ceil_div(rows, (int64_t)kActRows) * col_groups;
+  if (grid > 0x7FFFFFFFLL || col_groups > 0x7FFFFFFFLL) return fail(FSH_ENOTSUP, "fsh_act_quant_1x128: too many tiles");
+  hipLaunchKernelGGL(act_quant_1x128_kernel, dim3(static_cast<uint32_t>(grid)), dim3(kActThreads), 0,
+                     static_cast<hipStream_t>(stream), p);
+  return check_launch("act_quant_1x128_kernel");
+}
+
+FSH_API int fsh_fp8_gemm_1x128_128x128(const void* xq_dev, const float* xs_dev, const void* wq_dev,
+                                       const float* ws_dev, void* out_dev, int64_t m, int64_t n, int64_t k,
+                                       int64_t ldxq, int64_t ldwq, int64_t ldo, int64_t ws_cols, void* stream) {
+  using namespace fsh;
+  if (m < 0 || n < 0 || k < 0) return fail(FSH_EINVAL, "fsh_fp8_gemm_1x128_128x128: negative size");
+  if (m == 0 || n == 0) return FSH_OK;
+  if (!xq_dev || !xs_dev || !wq_dev || !ws_dev || !out_dev)
+    return fail(FSH_EINVAL, "fsh_fp8_gemm_1x128_128x128: null pointer");
+  if (k == 0 || k % 128)
+    return fail(FSH_ENOTSUP, "fsh_fp8_gemm_1x128_128x128: k must be a positive multiple of 128, got %lld (pad the operands)",
+                (long long)k);
+  if (ldxq < k || ldwq < k || ldo < n || ws_cols < k / 128)
+    return fail(FSH_EINVAL, "fsh_fp8_gemm_1x128_128x128: a leading dimension is smaller than its row");
+  if (ldxq % 16 || ldwq % 16 || !aligned(xq_dev, 16) || !aligned(wq_dev, 16) || !aligned(out_dev, 2))
+    return fail(FSH_ENOTSUP, "fsh_fp8_gemm_1x128_128x128: operand rows must be 16-byte aligned");
+  if (static_cast<int64_t>(Fp8Gemm::BN) * ldwq >= (1LL << 31) || static_cast<int64_t>(Fp8Gemm::BM) * ldxq >= (1LL << 31))
+    return fail(FSH_ENOTSUP, "fsh_fp8_gemm_1x128_128x128: a tile spans more than 2 GiB");
+  Fp8GemmParams p;
+  memset(&p, 0, sizeof(p));
+  p.xq = static_cast<const uint8_t*>(xq_dev);
+  p.xs = xs_dev;
+  p.wq = static_cast<const uint8_t*>(wq_dev);
+  p.ws = ws_dev;
+  p.out = static_cast<uint16_t*>(out_dev);
+  p.m = m; p.n = n; p.k = k;
+  p.ldxq = ldxq; p.ldwq = ldwq; p.ldo = ldo; p.ws_cols = ws_cols;
+  GemmParams& s = p.schedule;
+  s.tiles_m = static_cast<int32_t>(ceil_div(m, (int64_t)Fp8Gemm::BM));
+  s.tiles_n = static_cast<int32_t>(ceil_div(n, (int64_t)Fp8Gemm::BN));
+  const int64_t tiles = static_cast<int64_t>(s.tiles_m) * s.tiles_n;
+  if (tiles > 0x3FFFFFFFLL) return fail(FSH_ENOTSUP, "fsh_fp8_gemm_1x128_128x128: too many tiles");
+  s.tiles_per_matrix = static_cast<int32_t>(tiles);
+  s.work_items = tiles;
+  s.items_per_xcd = ceil_div(tiles, static_cast<int64_t>(kXcds));
+  static bool reserved = false;
+  if (!reserved) {
+    if (int rc = reserve_lds(&fp8_gemm_blockwise_kernel, Fp8Gemm::kLdsBytes)) return rc;
+    reserved = true;
+  }
+  hipLaunchKernelGGL(fp8_gemm_blockwise_kernel, dim3(static_cast<uint32_t>(s.items_per_xcd * kXcds)),
+                     dim3(Fp8Gemm::kThreads), Fp8Gemm::kLdsBytes, static_cast<hipStream_t>(stream), p);
+  return check_launch("fp8_gemm_blockwise_kernel");
+}

@@ -424,6 +424,62 @@ def gemm_nt_group(problems: Sequence[dict]) -> list[torch.Tensor]:
     return outs
 
 
+def act_quant_1x128(x: torch.Tensor, *, eps_fp32: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
+    """Quantize every run of 128 consecutive elements of each row of the bf16
+    matrix ``x`` to float8_e4m3fn.  Returns the bytes as ``[rows, cols rounded
+    up to 128]`` (pad columns zero) and the reciprocal scales as a
+    ``[cols / 128, rows]`` fp32 table.  ``eps_fp32`` floors an all-zero run's
+    amax at fp32 1e-12 (the activation quantizer's rule); ``False`` rounds the
+    floor to bf16 like the weight quantizer."""
+    _require_gpu(x)
+    if x.dtype != torch.bfloat16 or x.ndim != 2 or x.stride(1) != 1:
+        raise ValueError("x must be a bf16 matrix with contiguous rows")
+    rows, cols = x.shape
+    padded = -(-cols // 128) * 128
+    q = torch.empty((rows, padded), dtype=torch.float8_e4m3fn, device=x.device)
+    scales = torch.empty((padded // 128, rows), dtype=torch.float32, device=x.device)
+    if rows == 0 or cols == 0:
+        return q, scales
+    status = _native.lib().fsh_act_quant_1x128(
+        x.data_ptr(), rows, cols, x.stride(0), q.data_ptr(), padded, scales.data_ptr(),
+        EPS_FP32 if eps_fp32 else EPS_INPUT_DTYPE, stream_ptr(x.device),
+    )
+    _native.check(status, "fsh_act_quant_1x128")
+    return q, scales
+
+
+def fp8_gemm_1x128_128x128(
+    xq: torch.Tensor, xs: torch.Tensor, wq: torch.Tensor, ws: torch.Tensor, out: torch.Tensor | None = None
+) -> torch.Tensor:
+    """``out[i, j] = bf16(sum_kb dot(xq[i, kb], wq[j, kb]) * xs[kb, i] * ws[j // 128, kb])``
+    for float8_e4m3fn ``xq`` [m, k], ``wq`` [n, k] (rows contiguous, k a
+    multiple of 128), ``xs`` [k / 128, m] and ``ws`` [ceil(n / 128), >= k / 128]."""
+    _require_gpu(xq, xs, wq, ws)
+    for name, t in (("xq", xq), ("wq", wq)):
+        if t.dtype not in (torch.float8_e4m3fn, torch.uint8) or t.ndim != 2 or t.stride(1) != 1:
+            raise ValueError(f"{name} must be a float8_e4m3fn matrix with contiguous rows")
+    m, k = xq.shape
+    n = wq.shape[0]
+    if wq.shape[1] != k:
+        raise ValueError(f"inner dimensions differ: xq {tuple(xq.shape)} vs wq {tuple(wq.shape)}")
+    blocks = k // 128
+    if xs.dtype != torch.float32 or not xs.is_contiguous() or tuple(xs.shape) != (blocks, m):
+        raise ValueError(f"xs must be contiguous fp32 of shape {(blocks, m)}, got {tuple(xs.shape)}")
+    if ws.dtype != torch.float32 or ws.ndim != 2 or ws.stride(1) != 1 or ws.shape[0] != -(-n // 128) or ws.shape[1] < blocks:
+        raise ValueError(f"ws must be fp32 [{-(-n // 128)}, >= {blocks}] with contiguous rows, got {tuple(ws.shape)}")
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=xq.device)
+    _require_gpu(xq, out)
+    if out.dtype != torch.bfloat16 or tuple(out.shape) != (m, n) or out.stride(1) != 1:
+        raise ValueError(f"out must be bf16 [{m}, {n}] with contiguous rows")
+    status = _native.lib().fsh_fp8_gemm_1x128_128x128(
+        xq.data_ptr(), xs.data_ptr(), wq.data_ptr(), ws.data_ptr(), out.data_ptr(), m, n, k, xq.stride(0),
+        wq.stride(0), out.stride(0), ws.stride(0), stream_ptr(xq.device),
+    )
+    _native.check(status, "fsh_fp8_gemm_1x128_128x128")
+    return out
+
+
 def muon_prepare(
     momentum_buffer: torch.Tensor, grad: torch.Tensor, out: torch.Tensor, *, momentum: float, nesterov: bool
 ) -> None:

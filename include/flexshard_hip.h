@@ -243,6 +243,34 @@ int fsh_muon_prepare(void* momentum_dev, const void* grad_dev, void* out_dev, in
 int fsh_muon_apply(void* param_dev, const void* direction_dev, int64_t numel, float decay_factor,
                    float neg_adjusted_lr, float direction_scale, void* stream);
 
+/* ------------------------------------------------------------------------
+ * 8. Forward product of a linear layer with a prequantized weight.
+ * Replaces the device work of blockwise_fp8/fp8_blockwise_linear.py:50-91
+ * (Fp8BlockwiseGemms.forward): the activation quantizer and the scaled FP8
+ * GEMM it takes from torchao (triton_fp8_blockwise_act_quant_lhs and
+ * triton_fp8_gemm_1x128_128x128 of torchao.prototype.blockwise_fp8_training,
+ * torchao >= 0.18, not vendored by the reference).
+ *
+ * fsh_act_quant_1x128: x is [rows, cols] bf16 with row stride ldx.  Every
+ * run of 128 consecutive elements of a row (the last one zero-padded) is
+ * quantized like a weight tile: amax floored at 1e-12, scale = fp32(448 /
+ * fp64(amax)), q = e4m3fn(fp32(x) * scale).  q_dev is [rows, ldq] bytes with
+ * ldq = cols rounded up to 128 (pad bytes are written as zero), scales_dev is
+ * the [ldq / 128, rows] table of 1.0f / scale (row index contiguous).
+ *
+ * fsh_fp8_gemm_1x128_128x128:
+ *   out[i][j] = bf16( sum over kb of dot(xq[i][kb], wq[j][kb])
+ *                                  * (xs[kb][i] * ws[j / 128][kb]) ),  fp32 sums,
+ * xq [m, k] and wq [n, k] E4M3FN bytes with row strides ldxq / ldwq, xs the
+ * [k / 128, m] table above, ws the weight's [ceil(n / 128), ws_cols] scales,
+ * out [m, n] bf16 with row stride ldo.  k must be a multiple of 128.
+ * ---------------------------------------------------------------------- */
+int fsh_act_quant_1x128(const void* x_dev, int64_t rows, int64_t cols, int64_t ldx, void* q_dev,
+                        int64_t ldq, float* scales_dev, int32_t eps_mode, void* stream);
+int fsh_fp8_gemm_1x128_128x128(const void* xq_dev, const float* xs_dev, const void* wq_dev,
+                               const float* ws_dev, void* out_dev, int64_t m, int64_t n, int64_t k,
+                               int64_t ldxq, int64_t ldwq, int64_t ldo, int64_t ws_cols, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -58,6 +58,55 @@ def dequant_blockwise(
     return deq.reshape(tiles_r * block, tiles_c * block)[:rows, :cols].to(out_dtype)
 
 
+def act_quant_1x128(
+    x: torch.Tensor, block: int = 128, fp8_dtype: torch.dtype = torch.float8_e4m3fn
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """Activation quantizer of blockwise_fp8/fp8_blockwise_linear.py:66-71.  The
+    kernel is torchao's ``triton_fp8_blockwise_act_quant_lhs``
+    (torchao.prototype.blockwise_fp8_training.kernels, torchao >= 0.18, absent
+    from the reference checkout and from this image); its published algorithm
+    per 1 x block run of a row: amax floored at 1e-12 (fp32), float64 division
+    448 / amax, float32 scale, ``x * scale`` clamped and cast, reciprocal scale
+    stored.  PARITY UNPINNED against torchao itself; pinned here through the
+    tile quantizer (a run is a 1-row tile) and closed forms.  Returns the FP8
+    matrix padded with zero columns to whole runs and the reciprocal scales as
+    ``[runs per row, rows]`` (torchao's column-major ``[rows, runs]``)."""
+    if x.ndim != 2:
+        raise ValueError(f"expects a 2D matrix, got {tuple(x.shape)}")
+    rows, cols = x.shape
+    runs = -(-cols // block)
+    padded = x.new_zeros((rows, runs * block))
+    padded[:, :cols] = x
+    groups = padded.view(rows, runs, block)
+    fp8_max = torch.finfo(fp8_dtype).max
+    amax = groups.to(torch.float32).abs().amax(dim=2, keepdim=True).clamp(min=EPS).to(torch.float64)
+    scale = (fp8_max / amax).to(torch.float32)
+    quant = (groups.to(torch.float32) * scale).clamp(-fp8_max, fp8_max).to(fp8_dtype)
+    recip = (1.0 / scale).reshape(rows, runs).to(torch.float32)
+    return quant.reshape(rows, runs * block).contiguous(), recip.t().contiguous()
+
+
+def fp8_gemm_1x128_128x128(
+    xq: torch.Tensor, xs: torch.Tensor, wq: torch.Tensor, ws: torch.Tensor, block: int = 128,
+    out_dtype: torch.dtype = torch.bfloat16,
+) -> torch.Tensor:
+    """Scaled product of blockwise_fp8/fp8_blockwise_linear.py:74-90 (torchao's
+    ``triton_fp8_gemm_1x128_128x128``, same provenance and PARITY UNPINNED note
+    as above): for every k-block the fp32 dot products of the FP8 operands are
+    multiplied by the activation run's and the weight tile's reciprocal scales
+    and added to an fp32 accumulator in k order; one cast at the end.
+    ``xq`` [m, k], ``xs`` [k / block, m], ``wq`` [n, k], ``ws`` [ceil(n / block), k / block]."""
+    m, k = xq.shape
+    n = wq.shape[0]
+    acc = torch.zeros((m, n), dtype=torch.float32)
+    col_block = torch.arange(n) // block
+    for kb in range(k // block):
+        a = xq[:, kb * block : (kb + 1) * block].to(torch.float32)
+        b = wq[:, kb * block : (kb + 1) * block].to(torch.float32)
+        acc += (a @ b.t()) * xs[kb].to(torch.float32)[:, None] * ws[:, kb].to(torch.float32)[col_block][None, :]
+    return acc.to(out_dtype)
+
+
 def accumulate_microbatches(grads: list[torch.Tensor]) -> torch.Tensor:
     """flex_shard/bucket_runtime.py:931-933 -- each microbatch's bf16 grad is
     cast to the fp32 accumulation dtype and added in arrival order."""
