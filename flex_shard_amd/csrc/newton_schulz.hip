@@ -372,7 +372,7 @@ struct DmaGemm {
   static constexpr int kStageBytes = 2 * kOperandBytes;      // 64 KB
   static constexpr int kLoopLdsBytes = 2 * kStageBytes;
   static constexpr int kLoadsPerOperand = BM / 8 / 4;        // wave-level 1 KB loads per wave: 8
-  static constexpr int kTouchAhead = 3;                      // k-tiles between an L2 touch and its use
+  static constexpr int kTouchAhead = 3;                      // k-tiles between an L2 touch and the MFMAs on its data
   static constexpr int kScrapBytes = 1024;                   // landing area of the touches, 256 B per wave
 };
 
@@ -497,56 +497,63 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   FSH_STAMP(1);
   issue_tile_load(Ab, Bb, a_row_bytes, b_row_bytes, 0, 0, Cfg::kLoadsPerOperand);
 
-  // L2 touches.  A k-tile's operands are requested one k-tile (about 2 us)
-  // before they are needed, which a miss to HBM does not always make; so three
-  // k-tiles ahead each lane asks for 4 bytes of one operand row (one 128-byte
-  // line each: 256 rows of A and of B = two requests per wave), which brings
-  // the lines into L2 and makes the real request a hit.  The touches are
-  // issued after the k-tile's real requests and may still be in flight when
-  // those are waited for (requests complete in order).
+  // One k-tile, rotated by a quarter: the barrier that hands over the next
+  // tile's operands sits before the last k step, so that step's MFMAs cover
+  // the first fragment reads of the next tile (otherwise exposed after every
+  // barrier) and the requests for the tile after it (the stage they fill was
+  // released by the same barrier: every wave holds its last fragments of it
+  // in registers).
+  //   entering:  set 0 holds the fragments of (kt, k step 0); the operands of
+  //              kt + 1 are on their way
+  //   k steps 0 .. KS-2: MFMAs while the next step's fragments are read
+  //   wait for kt + 1, barrier
+  //   k step KS-1: one MFMA, one fragment read of (kt + 1, 0), one pair of
+  //              requests for kt + 2 at a time, then the L2 touches
+  // L2 touches: two k-tiles ahead of the requested one, each lane asks for
+  // 4 bytes of one operand row (one 128-byte line each: 256 rows of A and of
+  // B = two requests per wave) into a scrap area, which brings the lines into
+  // L2 early.  They are issued after the real requests and may still be in
+  // flight when those are waited for (requests complete in order).
   const uint32_t touch_row = static_cast<uint32_t>(64 * wave + lane);
   const uint32_t scrap_lds = lds_base + static_cast<uint32_t>(scrap_offset + wave * 256);
   auto k_tile = [&](int64_t kt, int64_t ktiles, auto more_tag) {
     constexpr bool more = decltype(more_tag)::value;
     const int stage_off = static_cast<int>(kt & 1) * Cfg::kStageBytes;
     const int next_off = stage_off ^ Cfg::kStageBytes;
-    const uint8_t* a_next = Ab + (kt + 1) * Cfg::kRowBytes;
-    const uint8_t* b_next = Bb + (kt + 1) * Cfg::kRowBytes;
-    const bool touch = more && kt + Cfg::kTouchAhead < ktiles;
-    // k step 0: one MFMA, one pair of loads of the next tile, one fragment
-    // read of k step 1 at a time.  The other stage is free: every wave passed
-    // the barrier that ended the previous tile after its last read of it.
 #pragma unroll
-    for (int g = 0; g < TM * TN; ++g) {
-      mfma(0, g / TN, g % TN);
-      if (more && g % 2 == 0) issue_tile_load(a_next, b_next, a_row_bytes, b_row_bytes, next_off, g / 2, g / 2 + 1);
-      if (g < TM) read_a(1, stage_off, 1, g);
-      else if (g < TM + TN) read_b(1, stage_off, 1, g - TM);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    if (touch) {
-      dma_touch_4(touch_row * a_row_bytes, Ab + (kt + Cfg::kTouchAhead) * Cfg::kRowBytes, scrap_lds);
-      dma_touch_4(touch_row * b_row_bytes, Bb + (kt + Cfg::kTouchAhead) * Cfg::kRowBytes, scrap_lds);
-    }
-#pragma unroll
-    for (int ks = 1; ks < KS; ++ks) {
-      if (ks + 1 < KS) read_frags((ks + 1) & 1, stage_off, ks + 1);
+    for (int ks = 0; ks + 1 < KS; ++ks) {
+      read_frags((ks + 1) & 1, stage_off, ks + 1);
 #pragma unroll
       for (int g = 0; g < TM * TN; ++g) mfma(ks & 1, g / TN, g % TN);
-      if (ks + 1 < KS) {
 #pragma unroll
-        for (int g = 0; g < TM + TN; ++g) {
-          __builtin_amdgcn_sched_group_barrier(kSchedDsRead, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(kSchedMfma, TM * TN / (TM + TN), 0);
-        }
+      for (int g = 0; g < TM + TN; ++g) {
+        __builtin_amdgcn_sched_group_barrier(kSchedDsRead, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(kSchedMfma, TM * TN / (TM + TN), 0);
       }
     }
     if (more) {  // this wave's part of the next tile has landed
-      if (touch) wait_for_dma_loads_except<2>();
+      // touches followed its requests iff the k-tile before this one issued them
+      if (kt >= 1 && kt + Cfg::kTouchAhead < ktiles) wait_for_dma_loads_except<2>();
       else wait_for_dma_loads();
     }
     __syncthreads();
-    if (more) read_frags(0, next_off, 0);
+    const bool more2 = more && kt + 2 < ktiles;
+    const uint8_t* a_next = Ab + (kt + 2) * Cfg::kRowBytes;
+    const uint8_t* b_next = Bb + (kt + 2) * Cfg::kRowBytes;
+#pragma unroll
+    for (int g = 0; g < TM * TN; ++g) {
+      mfma((KS - 1) & 1, g / TN, g % TN);
+      if (more) {
+        if (g < TM) read_a(0, next_off, 0, g);
+        else if (g < TM + TN) read_b(0, next_off, 0, g - TM);
+      }
+      if (more2 && g % 2 == 0) issue_tile_load(a_next, b_next, a_row_bytes, b_row_bytes, stage_off, g / 2, g / 2 + 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (more2 && kt + 1 + Cfg::kTouchAhead < ktiles) {
+      dma_touch_4(touch_row * a_row_bytes, Ab + (kt + 1 + Cfg::kTouchAhead) * Cfg::kRowBytes, scrap_lds);
+      dma_touch_4(touch_row * b_row_bytes, Bb + (kt + 1 + Cfg::kTouchAhead) * Cfg::kRowBytes, scrap_lds);
+    }
   };
 
   while (true) {
@@ -563,6 +570,9 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
     FSH_STAMP(7);
     __syncthreads();  // also: every wave has left the previous tile's epilogue
     read_frags(0, 0, 0);
+    if (ktiles > 1)
+      issue_tile_load(Ab + Cfg::kRowBytes, Bb + Cfg::kRowBytes, a_row_bytes, b_row_bytes, Cfg::kStageBytes, 0,
+                      Cfg::kLoadsPerOperand);
     FSH_STAMP(2);
 
     for (int64_t kt = 0; kt + 1 < ktiles; ++kt) k_tile(kt, ktiles, std::true_type{});
