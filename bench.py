@@ -15,7 +15,9 @@ One JSON line is printed.  Besides the contract fields it carries
   cpu_baseline  the oracle's eager-torch restatement of the reference path on
                 the host cores, on the same rank-0 share
   secondary     unpack+dequant of the 8-rank gathered layout, the fp32
-                gradient path, and the 48-matrix Muon / Newton-Schulz step
+                gradient path, the 48-matrix Muon / Newton-Schulz step, and the
+                forward product of the prequantized-weight linear (1x128
+                activation quantizer + scaled FP8 GEMM) on Llama-3-8B shapes
 """
 
 from __future__ import annotations
@@ -33,7 +35,8 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor figure
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
-# HBM bytes per launch of quantize_pack_kernel on the default workload, from
+FP8_MFMA_PEAK_TFLOPS = 5000.0  # MI355X dense fp8, vendor figure
+# HBM bytes per launch of quantize_pack_bf16_kernel on the default workload, from
 # two counter runs (FETCH_SIZE, then WRITE_SIZE) of this script, each scaled by
 # the same counter's reading for the 256 MiB --calibrate-copy kernel:
 # 26 669.0 KiB x 1.9937 read + 26 932.2 KiB x 1.0 written.  Counters cannot be
@@ -265,6 +268,37 @@ def bench_muon(device, reps=3):
             "frac_of_bf16_mfma_peak": flops / per / 1e9 / BF16_MFMA_PEAK_TFLOPS}
 
 
+def bench_fp8_linear(device, tokens: int = 8192, reps: int = 10):
+    """Forward of the blockwise FP8 linear on the layer's projections: 8192
+    tokens against q/o [4096, 4096], gate/up [14336, 4096] and down
+    [4096, 14336], weights quantized by the tile quantizer."""
+    from flex_shard_amd import hip_ops
+    from flex_shard_amd.testing import seeded_normal
+
+    out = {}
+    for name, (n, k) in (("q_o_4096x4096", (4096, 4096)), ("gate_up_14336x4096", (14336, 4096)),
+                         ("down_4096x14336", (4096, 14336))):
+        x = seeded_normal((tokens, k), 1.0, 4000 + n, device)
+        w = seeded_normal((n, k), 0.02, 4100 + k, device)
+        wq, ws = hip_ops.act_quant_1x128(w)  # any valid FP8 operand: bytes and fp32 scales of the right shapes
+        ws = ws.t().contiguous()[: n // 128].contiguous()  # [n / 128, k / 128] table for the timing
+        _, q_ms = _event_ms(lambda i: hip_ops.act_quant_1x128(x), reps, 2)
+        xq, xs = hip_ops.act_quant_1x128(x)
+        y = torch.empty((tokens, n), dtype=torch.bfloat16, device=device)
+        _, g_ms = _event_ms(lambda i: hip_ops.fp8_gemm_1x128_128x128(xq, xs, wq, ws, out=y), reps, 2)
+        q_us, g_us = q_ms / reps * 1e3, g_ms / reps * 1e3
+        flop = 2 * tokens * n * k
+        out[name] = {
+            "act_quant_us": q_us,
+            "act_quant_GBps": tokens * k * (3 + 4 / 128) / q_us / 1e3,  # 2 B read + 1 B + 4/128 B written per element
+            "gemm_us": g_us,
+            "gemm_TFLOPs": flop / g_us / 1e6,
+            "frac_of_fp8_mfma_peak": flop / g_us / 1e6 / FP8_MFMA_PEAK_TFLOPS,
+        }
+        del x, w, wq, ws, xq, xs, y
+    return out
+
+
 def calibrate_copy(device, nbytes: int = 256 << 20, reps: int = 4) -> None:
     """A plain copy of known size through copy_segments_kernel: reads `nbytes`
     and writes `nbytes` per launch."""
@@ -337,7 +371,7 @@ def main() -> None:
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "quantize_pack_kernel",
+            "kernel": "quantize_pack_bf16_kernel",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
@@ -374,6 +408,10 @@ def main() -> None:
         torch.cuda.empty_cache()
         muon = bench_muon(device)
         secondary["muon_newton_schulz"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in muon.items()}
+        torch.cuda.empty_cache()
+        secondary["fp8_linear_forward_8192_tokens"] = {
+            name: {k: round(v, 4) for k, v in d.items()} for name, d in bench_fp8_linear(device).items()
+        }
         result["secondary"] = secondary
     print(json.dumps(result))
 
