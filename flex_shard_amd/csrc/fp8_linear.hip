@@ -100,8 +100,8 @@ __global__ __launch_bounds__(kActThreads) void act_quant_1x128_kernel(const ActQ
 // ----------------------------------------------------------------- FP8 GEMM
 // 128 x 256 output tile per workgroup, four waves of 64 x 128 (two by four
 // 32x32 blocks).  Operand tiles are 128 bytes per row and k-tile and travel
-// global -> LDS directly, 16-byte chunk c of row r in slot c ^ (r & 7), two
-// stages.  A lane feeds the matrix core bytes [32 h, 32 h + 32) of each half
+// global -> LDS directly, 16-byte chunk c of row r in slot c ^ (r & 7), into
+// one of three stages.  A lane feeds the matrix core bytes [32 h, 32 h + 32) of each half
 // of its row (h = lane / 32), i.e. chunks 2h and 2h+1 of a 64-byte half.
 struct Fp8Gemm {
   static constexpr int BM = 128, BN = 256, BK = 128, WM = 2, WN = 2, TM = 2, TN = 4;
@@ -112,7 +112,11 @@ struct Fp8Gemm {
   static constexpr int kLoadsA = BM / 8 / 4, kLoadsB = BN / 8 / 4;  // per wave: 4 and 8
   static constexpr int kPitch = kWaveN * 2 + 8;                // epilogue staging, bytes
   static constexpr int kRegion = kWaveM * kPitch;              // per wave
-  static constexpr int kLdsBytes = max_int(2 * kStageBytes, 4 * kRegion);
+  static constexpr int kStages = 3;
+  static constexpr int kScaleOffset = kStages * kStageBytes;   // [stage][wave][64] activation scales
+  static constexpr int kWeightScaleOffset = kScaleOffset + kStages * 1024;  // [wave][256] weight scales
+  static constexpr int kMaxKTilesInLds = 256;
+  static constexpr int kLdsBytes = max_int(kWeightScaleOffset + 4 * kMaxKTilesInLds * 4, 4 * kRegion);
 };
 
 struct Fp8GemmParams {
@@ -197,15 +201,9 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
   // Scales: a lane owns output row lane & 31 of each of its two 32-row blocks,
   // so it needs xs[kb][row] for two rows and the one weight scale of the
   // wave's 128 columns.
-  int64_t srow[TM];
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int64_t row = m0 + wm * Cfg::kWaveM + i * 32 + frag_row;
-    srow[i] = row < p.m ? row : p.m - 1;
-  }
   const int64_t wcol = n0 + wn * Cfg::kWaveN;
   const int64_t wblock = (wcol < p.n ? wcol : p.n - 1) / 128;
-  const float* ws_row = p.ws + wblock * p.ws_cols;
+  const float* ws_row = uniform_ptr(p.ws + wblock * p.ws_cols);  // scalar loads: no vector-memory wait
 
   f32x16 acc[TM][TN];
 #pragma unroll
@@ -215,52 +213,84 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  issue_tile_load(0, 0);
-  float xs_next[TM], ws_next;
-#pragma unroll
-  for (int i = 0; i < TM; ++i) xs_next[i] = p.xs[srow[i]];
-  ws_next = ws_row[0];
-  wait_for_dma_loads();
+  // Three stages: the operands of k-tiles kt + 1 and kt + 2 are in flight
+  // while kt is multiplied (a k-tile is under a microsecond of MFMA work, a
+  // miss to HBM takes two).  The activation scales ride the same global->LDS
+  // path (one 4-byte-per-lane request per wave and k-tile for the wave's 64
+  // rows): a compiler-visible load here would make the compiler wait for
+  // everything in flight, the prefetched tiles included.  Requests complete
+  // in order, so "at most 13 outstanding" means all but the youngest tile's.
+  const uint32_t scale_lds0 = lds_base + static_cast<uint32_t>(Cfg::kScaleOffset + wave * 256);
+  const int64_t scale_row0 = m0 + wm * Cfg::kWaveM + lane;
+  const uint32_t scale_voff = static_cast<uint32_t>((scale_row0 < p.m ? scale_row0 : p.m - 1) * 4);
+  auto issue_k_tile = [&](int64_t kt, int stage) {
+    issue_tile_load(kt, stage * Cfg::kStageBytes);
+    dma_touch_4(scale_voff, reinterpret_cast<const uint8_t*>(p.xs + kt * p.m), scale_lds0 + stage * 1024);
+  };
+  // The weight scales of the wave's 128 columns, one per k-tile, are copied
+  // to LDS once (a load from global memory inside the loop would again wait
+  // for the prefetched tiles).
+  float* ws_lds = reinterpret_cast<float*>(lds_bytes + Cfg::kWeightScaleOffset + wave * Cfg::kMaxKTilesInLds * 4);
+  for (int64_t i = lane; i < ktiles; i += 64) ws_lds[i] = ws_row[i];  // ktiles <= kMaxKTilesInLds (host check)
+  issue_k_tile(0, 0);
+  if (ktiles > 1) {
+    issue_k_tile(1, 1);
+    wait_for_dma_loads_except<Cfg::kLoadsA + Cfg::kLoadsB + 1>();
+  } else {
+    wait_for_dma_loads();
+  }
   __syncthreads();
 
+  int stage = 0;
   for (int64_t kt = 0; kt < ktiles; ++kt) {
-    const int stage_off = static_cast<int>(kt & 1) * Cfg::kStageBytes;
-    const bool more = kt + 1 < ktiles;
-    if (more) issue_tile_load(kt + 1, stage_off ^ Cfg::kStageBytes);
+    const int stage_off = stage * Cfg::kStageBytes;
+    const int stage2 = stage >= 1 ? stage - 1 : Cfg::kStages - 1;  // (stage + 2) % 3
+    if (kt + 2 < ktiles) issue_k_tile(kt + 2, stage2);  // its stage was released by the barrier that ended kt - 1
+    const float ws_now = ws_lds[kt];
     float s[TM];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) s[i] = xs_next[i] * ws_next;
-    if (more) {
-#pragma unroll
-      for (int i = 0; i < TM; ++i) xs_next[i] = p.xs[(kt + 1) * p.m + srow[i]];
-      ws_next = ws_row[kt + 1];
-    }
-    v8i32 bfrag[TN][2];
+    for (int i = 0; i < TM; ++i)
+      s[i] = *reinterpret_cast<const float*>(lds_bytes + Cfg::kScaleOffset + stage * 1024 + wave * 256 +
+                                             (i * 32 + frag_row) * 4) * ws_now;
+    v8i32 bfrag[TN][2], afrag[TM][2];
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int kh = 0; kh < 2; ++kh) bfrag[j][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32) + j, kh);
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      v8i32 afrag[2];
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int kh = 0; kh < 2; ++kh) afrag[kh] = read_frag(stage_off, 0, wm * (Cfg::kWaveM / 32) + i, kh);
-      f32x16 part[TN];
+      for (int kh = 0; kh < 2; ++kh) afrag[i][kh] = read_frag(stage_off, 0, wm * (Cfg::kWaveM / 32) + i, kh);
+    // The eight 32x32 blocks in turn: two MFMAs give a block's partial product
+    // for this scale block; it is folded into the result (16 fused multiply-
+    // adds) while the next block's MFMAs run.
+    f32x16 part_prev;
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        part[j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j][0], afrag[0], zero, 0, 0, 0, 0, 0, 0);
+    for (int blk = 0; blk < TM * TN; ++blk) {
+      const int i = blk / TN, j = blk % TN;
+      const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      f32x16 part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j][0], afrag[i][0], zero, 0, 0, 0, 0, 0, 0);
+      part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j][1], afrag[i][1], part, 0, 0, 0, 0, 0, 0);
+      if (blk > 0) {
+        const int pi = (blk - 1) / TN, pj = (blk - 1) % TN;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[pi][pj][r] = __builtin_fmaf(part_prev[r], s[pi], acc[pi][pj][r]);
+        // An empty statement that "uses" the folded block keeps the folds on
+        // this side of the scheduling barrier (plain arithmetic may otherwise
+        // be moved past it and end up after the last MFMA).
+        asm volatile("" : "+v"(acc[pi][pj]));
       }
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        part[j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j][1], afrag[1], part[j], 0, 0, 0, 0, 0, 0);
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = __builtin_fmaf(part[j][r], s[i], acc[i][j][r]);
+      part_prev = part;
+      __builtin_amdgcn_sched_barrier(0);  // MFMA pair, then the previous block's folds, in that order
     }
-    if (more) wait_for_dma_loads();
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[TM - 1][TN - 1][r] = __builtin_fmaf(part_prev[r], s[TM - 1], acc[TM - 1][TN - 1][r]);
+    if (kt + 1 < ktiles) {  // k-tile kt + 1 has landed; kt + 2 may still be on its way
+      if (kt + 2 < ktiles) wait_for_dma_loads_except<Cfg::kLoadsA + Cfg::kLoadsB + 1>();
+      else wait_for_dma_loads();
+    }
     __syncthreads();
+    stage = stage + 1 == Cfg::kStages ? 0 : stage + 1;
   }
 
   // Epilogue: bf16 finals to the wave's staging region as [row][col], then
@@ -351,14 +381,16 @@ FSH_API int fsh_fp8_gemm_1x128_128x128(const void* xq_dev, const float* xs_dev, 
   if (m == 0 || n == 0) return FSH_OK;
   if (!xq_dev || !xs_dev || !wq_dev || !ws_dev || !out_dev)
     return fail(FSH_EINVAL, "fsh_fp8_gemm_1x128_128x128: null pointer");
-  if (k == 0 || k % 128)
-    return fail(FSH_ENOTSUP, "fsh_fp8_gemm_1x128_128x128: k must be a positive multiple of 128, got %lld (pad the operands)",
-                (long long)k);
+  if (k == 0 || k % 128 || k / 128 > Fp8Gemm::kMaxKTilesInLds)
+    return fail(FSH_ENOTSUP,
+                "fsh_fp8_gemm_1x128_128x128: k must be a positive multiple of 128 (pad the operands) and at most %d, got %lld",
+                128 * Fp8Gemm::kMaxKTilesInLds, (long long)k);
   if (ldxq < k || ldwq < k || ldo < n || ws_cols < k / 128)
     return fail(FSH_EINVAL, "fsh_fp8_gemm_1x128_128x128: a leading dimension is smaller than its row");
   if (ldxq % 16 || ldwq % 16 || !aligned(xq_dev, 16) || !aligned(wq_dev, 16) || !aligned(out_dev, 2))
     return fail(FSH_ENOTSUP, "fsh_fp8_gemm_1x128_128x128: operand rows must be 16-byte aligned");
-  if (static_cast<int64_t>(Fp8Gemm::BN) * ldwq >= (1LL << 31) || static_cast<int64_t>(Fp8Gemm::BM) * ldxq >= (1LL << 31))
+  if (static_cast<int64_t>(Fp8Gemm::BN) * ldwq >= (1LL << 31) || static_cast<int64_t>(Fp8Gemm::BM) * ldxq >= (1LL << 31) ||
+      m >= (1LL << 30))
     return fail(FSH_ENOTSUP, "fsh_fp8_gemm_1x128_128x128: a tile spans more than 2 GiB");
   Fp8GemmParams p;
   memset(&p, 0, sizeof(p));

@@ -452,7 +452,7 @@ __device__ inline void store_tile_in_halves(const GemmParams& p, int64_t batch, 
 }
 
 // Scheduling-group masks of __builtin_amdgcn_sched_group_barrier.
-constexpr int kSchedMfma = 0x008, kSchedVmemRead = 0x020, kSchedDsRead = 0x100, kSchedDsWrite = 0x200;
+constexpr int kSchedValu = 0x002, kSchedMfma = 0x008, kSchedVmemRead = 0x020, kSchedDsRead = 0x100, kSchedDsWrite = 0x200;
 
 // gfx950 loads 16 bytes per lane from global memory straight into LDS: lane l
 // of a wave writes LDS bytes [M0 + 16 l, M0 + 16 l + 16).  The address is a
@@ -471,8 +471,9 @@ __device__ inline void dma_touch_4(uint32_t voffset, const uint8_t* base, uint32
 // of interest, those are complete once at most `younger` are outstanding.
 template <int younger>
 __device__ inline void wait_for_dma_loads_except() {
-  static_assert(younger == 2, "one immediate per use");
-  asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+  static_assert(younger == 2 || younger == 13, "one immediate per use");
+  if (younger == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(13)" ::: "memory");
 }
 
 constexpr int max_int(int a, int b) { return a > b ? a : b; }
