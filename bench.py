@@ -16,8 +16,9 @@ One JSON line is printed.  Besides the contract fields it carries
                 the host cores, on the same rank-0 share
   secondary     unpack+dequant of the 8-rank gathered layout, the fp32
                 gradient path, the 48-matrix Muon / Newton-Schulz step, and the
-                forward product of the prequantized-weight linear (1x128
-                activation quantizer + scaled FP8 GEMM) on Llama-3-8B shapes
+                forward and backward products of the prequantized-weight
+                linear (activation quantizers + scaled FP8 GEMMs) on
+                Llama-3-8B shapes
 """
 
 from __future__ import annotations
@@ -299,6 +300,56 @@ def bench_fp8_linear(device, tokens: int = 8192, reps: int = 10):
     return out
 
 
+def bench_fp8_linear_backward(device, tokens: int = 8192, reps: int = 10):
+    """Backward of the same linear, per kernel: the input gradient
+    (1x128 quantizer on grad_out, byte transpose of the weight, GEMM) and the
+    weight gradient (token-run quantizer on grad_out and on x, GEMM)."""
+    from flex_shard_amd import hip_ops
+    from flex_shard_amd.testing import seeded_normal
+
+    out = {}
+    for name, (n, k) in (("q_o_4096x4096", (4096, 4096)), ("gate_up_14336x4096", (14336, 4096)),
+                         ("down_4096x14336", (4096, 14336))):
+        x = seeded_normal((tokens, k), 1.0, 4200 + n, device)
+        g = seeded_normal((tokens, n), 0.01, 4300 + k, device)
+        w = seeded_normal((n, k), 0.02, 4400 + k, device)
+        wq, ws = hip_ops.act_quant_1x128(w)  # any valid FP8 operand of the right shape
+        ws = ws.t().contiguous()[: n // 128].contiguous()
+        del w
+        us = {}
+        _, ms = _event_ms(lambda i: hip_ops.fp8_transpose(wq), reps, 2)
+        us["transpose"] = ms / reps * 1e3
+        _, ms = _event_ms(lambda i: hip_ops.act_quant_128x1_transposed(g), reps, 2)
+        us["quant_grad_t"] = ms / reps * 1e3
+        _, ms = _event_ms(lambda i: hip_ops.act_quant_128x1_transposed(x), reps, 2)
+        us["quant_x_t"] = ms / reps * 1e3
+        wt = hip_ops.fp8_transpose(wq)
+        gq, gs = hip_ops.act_quant_1x128(g)
+        _, ms = _event_ms(lambda i: hip_ops.fp8_gemm_1x128_128x128_dgrad(gq, gs, wt, ws), reps, 2)
+        us["dgrad_gemm"] = ms / reps * 1e3
+        del wt, gq, gs
+        gtq, gts = hip_ops.act_quant_128x1_transposed(g)
+        xtq, xts = hip_ops.act_quant_128x1_transposed(x)
+        _, ms = _event_ms(lambda i: hip_ops.fp8_gemm_1x128_128x1(gtq, gts, xtq, xts), reps, 2)
+        us["wgrad_gemm"] = ms / reps * 1e3
+        flop = 2 * tokens * n * k
+        out[name] = {
+            "transpose_us": us["transpose"],
+            "transpose_GBps": 2 * n * k / us["transpose"] / 1e3,  # 1 B read + 1 B written per element
+            "quant_grad_transposed_us": us["quant_grad_t"],
+            "quant_grad_transposed_GBps": tokens * n * (3 + 4 / 128) / us["quant_grad_t"] / 1e3,
+            "quant_x_transposed_us": us["quant_x_t"],
+            "quant_x_transposed_GBps": tokens * k * (3 + 4 / 128) / us["quant_x_t"] / 1e3,
+            "dgrad_gemm_us": us["dgrad_gemm"],
+            "dgrad_gemm_TFLOPs": flop / us["dgrad_gemm"] / 1e6,
+            "wgrad_gemm_us": us["wgrad_gemm"],
+            "wgrad_gemm_TFLOPs": flop / us["wgrad_gemm"] / 1e6,
+            "wgrad_frac_of_fp8_mfma_peak": flop / us["wgrad_gemm"] / 1e6 / FP8_MFMA_PEAK_TFLOPS,
+        }
+        del x, g, wq, ws, gtq, gts, xtq, xts
+    return out
+
+
 def calibrate_copy(device, nbytes: int = 256 << 20, reps: int = 4) -> None:
     """A plain copy of known size through copy_segments_kernel: reads `nbytes`
     and writes `nbytes` per launch."""
@@ -411,6 +462,10 @@ def main() -> None:
         torch.cuda.empty_cache()
         secondary["fp8_linear_forward_8192_tokens"] = {
             name: {k: round(v, 4) for k, v in d.items()} for name, d in bench_fp8_linear(device).items()
+        }
+        torch.cuda.empty_cache()
+        secondary["fp8_linear_backward_8192_tokens"] = {
+            name: {k: round(v, 4) for k, v in d.items()} for name, d in bench_fp8_linear_backward(device).items()
         }
         result["secondary"] = secondary
     print(json.dumps(result))

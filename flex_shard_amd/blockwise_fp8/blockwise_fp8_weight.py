@@ -134,12 +134,28 @@ class BlockwiseFp8Weight(torch.Tensor):
     def __tensor_unflatten__(cls, inner_tensors, metadata, outer_size, outer_stride):
         return cls(inner_tensors["_data"], inner_tensors["_recip_scale"], metadata["block_size"], metadata["orig_dtype"])
 
+    def _map_inner(self, fn) -> "BlockwiseFp8Weight":
+        return BlockwiseFp8Weight(
+            fn(self._data), fn(self._recip_scale), self._block_size, self._orig_dtype, requires_grad=False
+        )
+
     @classmethod
     def __torch_dispatch__(cls, func, types, args=(), kwargs=None):
+        # Autograd needs to alias and detach the wrapper to save it for a
+        # backward pass (reference: blockwise_quant/weight.py:96-108); every
+        # other operator would silently compute on the wrapper's fake storage.
+        if func == torch.ops.aten.alias.default:
+            from torch.utils._python_dispatch import return_and_correct_aliasing
+
+            return return_and_correct_aliasing(func, args, kwargs or {}, args[0]._map_inner(func))
+        if func == torch.ops.aten.detach.default:
+            return args[0]._map_inner(torch.Tensor.detach)
         raise NotImplementedError(
             f"BlockwiseFp8Weight does not implement {func}; call dequantize() or pass fp8_data / recip_scale "
             "to an FP8 GEMM."
         )
+
+    __torch_function__ = torch._C._disabled_torch_function_impl
 
     def __repr__(self) -> str:  # the default repr would dispatch
         return (

@@ -123,17 +123,23 @@ struct Fp8GemmParams {
   const uint8_t* xq;
   const float* xs;   // [k / 128][m]
   const uint8_t* wq;
-  const float* ws;   // [ceil(n / 128)][ws_cols]
+  const float* ws;   // block scales: element (output-column block cb, k-block kb) at ws[cb * ws_cb + kb * ws_kb]
+  const float* cs;   // per-column scales [k / 128][n] (the other kernel variant)
   uint16_t* out;
   int64_t m, n, k;
-  int64_t ldxq, ldwq, ldo, ws_cols;
+  int64_t ldxq, ldwq, ldo, ws_cb, ws_kb;
   GemmParams schedule;  // tile order only
 };
 
 typedef int v8i32 __attribute__((ext_vector_type(8)));
 
+// kColumnScales = false: the second operand carries one scale per 128 x 128
+// tile (a prequantized weight, either orientation).  true: one scale per
+// output column and k-block (an operand quantized in 128 x 1 runs).
+template <bool kColumnScales>
 __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(const Fp8GemmParams p) {
   using Cfg = Fp8Gemm;
+  constexpr int kLoadsPerKTile = Cfg::kLoadsA + Cfg::kLoadsB + (kColumnScales ? 2 : 1);
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds_bytes[];
   constexpr int TM = Cfg::TM, TN = Cfg::TN;
   const int tid = threadIdx.x;
@@ -203,7 +209,6 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
   // wave's 128 columns.
   const int64_t wcol = n0 + wn * Cfg::kWaveN;
   const int64_t wblock = (wcol < p.n ? wcol : p.n - 1) / 128;
-  const float* ws_row = uniform_ptr(p.ws + wblock * p.ws_cols);  // scalar loads: no vector-memory wait
 
   f32x16 acc[TM][TN];
 #pragma unroll
@@ -223,19 +228,29 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
   const uint32_t scale_lds0 = lds_base + static_cast<uint32_t>(Cfg::kScaleOffset + wave * 256);
   const int64_t scale_row0 = m0 + wm * Cfg::kWaveM + lane;
   const uint32_t scale_voff = static_cast<uint32_t>((scale_row0 < p.m ? scale_row0 : p.m - 1) * 4);
+  // Per-column scales of the workgroup's 256 columns take the same road, 64
+  // columns per wave, into [stage][256] floats of the weight-scale area.
+  const uint32_t cscale_lds0 = lds_base + static_cast<uint32_t>(Cfg::kWeightScaleOffset + wave * 256);
+  const int64_t cscale_col0 = n0 + wave * 64 + lane;
+  const uint32_t cscale_voff = static_cast<uint32_t>((cscale_col0 < p.n ? cscale_col0 : p.n - 1) * 4);
   auto issue_k_tile = [&](int64_t kt, int stage) {
     issue_tile_load(kt, stage * Cfg::kStageBytes);
     dma_touch_4(scale_voff, reinterpret_cast<const uint8_t*>(p.xs + kt * p.m), scale_lds0 + stage * 1024);
+    if (kColumnScales)
+      dma_touch_4(cscale_voff, reinterpret_cast<const uint8_t*>(p.cs + kt * p.n), cscale_lds0 + stage * 1024);
   };
-  // The weight scales of the wave's 128 columns, one per k-tile, are copied
+  // The block scales of the wave's 128 columns, one per k-tile, are copied
   // to LDS once (a load from global memory inside the loop would again wait
   // for the prefetched tiles).
   float* ws_lds = reinterpret_cast<float*>(lds_bytes + Cfg::kWeightScaleOffset + wave * Cfg::kMaxKTilesInLds * 4);
-  for (int64_t i = lane; i < ktiles; i += 64) ws_lds[i] = ws_row[i];  // ktiles <= kMaxKTilesInLds (host check)
+  if (!kColumnScales) {
+    const float* ws_row = p.ws + wblock * p.ws_cb;
+    for (int64_t i = lane; i < ktiles; i += 64) ws_lds[i] = ws_row[i * p.ws_kb];  // ktiles <= kMaxKTilesInLds (host check)
+  }
   issue_k_tile(0, 0);
   if (ktiles > 1) {
     issue_k_tile(1, 1);
-    wait_for_dma_loads_except<Cfg::kLoadsA + Cfg::kLoadsB + 1>();
+    wait_for_dma_loads_except<kLoadsPerKTile>();
   } else {
     wait_for_dma_loads();
   }
@@ -246,12 +261,16 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
     const int stage_off = stage * Cfg::kStageBytes;
     const int stage2 = stage >= 1 ? stage - 1 : Cfg::kStages - 1;  // (stage + 2) % 3
     if (kt + 2 < ktiles) issue_k_tile(kt + 2, stage2);  // its stage was released by the barrier that ended kt - 1
-    const float ws_now = ws_lds[kt];
     float s[TM];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
       s[i] = *reinterpret_cast<const float*>(lds_bytes + Cfg::kScaleOffset + stage * 1024 + wave * 256 +
-                                             (i * 32 + frag_row) * 4) * ws_now;
+                                             (i * 32 + frag_row) * 4);
+    if (!kColumnScales) {
+      const float ws_now = ws_lds[kt];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) s[i] *= ws_now;
+    }
     v8i32 bfrag[TN][2], afrag[TM][2];
 #pragma unroll
     for (int j = 0; j < TN; ++j)
@@ -263,18 +282,38 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
       for (int kh = 0; kh < 2; ++kh) afrag[i][kh] = read_frag(stage_off, 0, wm * (Cfg::kWaveM / 32) + i, kh);
     // The eight 32x32 blocks in turn: two MFMAs give a block's partial product
     // for this scale block; it is folded into the result (16 fused multiply-
-    // adds) while the next block's MFMAs run.
+    // adds) while the next block's MFMAs run.  With per-column scales the
+    // blocks go column block by column block, so that the sixteen column
+    // scales a lane needs are read from LDS once for both row blocks.
+    auto block_i = [&](int blk) { return kColumnScales ? blk % TM : blk / TN; };
+    auto block_j = [&](int blk) { return kColumnScales ? blk / TM : blk % TN; };
+    const uint8_t* cscale_lds = lds_bytes + Cfg::kWeightScaleOffset + stage * 1024 + (wn * Cfg::kWaveN + 4 * h) * 4;
     f32x16 part_prev;
+    f32x4 cscale[4];
+    auto fold = [&](int pi, int pj) {
+      if (kColumnScales) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          acc[pi][pj][r] = __builtin_fmaf(part_prev[r] * s[pi], cscale[r / 4][r % 4], acc[pi][pj][r]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[pi][pj][r] = __builtin_fmaf(part_prev[r], s[pi], acc[pi][pj][r]);
+      }
+    };
 #pragma unroll
     for (int blk = 0; blk < TM * TN; ++blk) {
-      const int i = blk / TN, j = blk % TN;
+      const int i = block_i(blk), j = block_j(blk);
       const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (kColumnScales && blk > 0 && block_i(blk - 1) == 0) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          cscale[b] = *reinterpret_cast<const f32x4*>(cscale_lds + (block_j(blk - 1) * 32 + 8 * b) * 4);
+      }
       f32x16 part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j][0], afrag[i][0], zero, 0, 0, 0, 0, 0, 0);
       part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j][1], afrag[i][1], part, 0, 0, 0, 0, 0, 0);
       if (blk > 0) {
-        const int pi = (blk - 1) / TN, pj = (blk - 1) % TN;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[pi][pj][r] = __builtin_fmaf(part_prev[r], s[pi], acc[pi][pj][r]);
+        const int pi = block_i(blk - 1), pj = block_j(blk - 1);
+        fold(pi, pj);
         // An empty statement that "uses" the folded block keeps the folds on
         // this side of the scheduling barrier (plain arithmetic may otherwise
         // be moved past it and end up after the last MFMA).
@@ -283,10 +322,9 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
       part_prev = part;
       __builtin_amdgcn_sched_barrier(0);  // MFMA pair, then the previous block's folds, in that order
     }
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[TM - 1][TN - 1][r] = __builtin_fmaf(part_prev[r], s[TM - 1], acc[TM - 1][TN - 1][r]);
+    fold(TM - 1, TN - 1);
     if (kt + 1 < ktiles) {  // k-tile kt + 1 has landed; kt + 2 may still be on its way
-      if (kt + 2 < ktiles) wait_for_dma_loads_except<Cfg::kLoadsA + Cfg::kLoadsB + 1>();
+      if (kt + 2 < ktiles) wait_for_dma_loads_except<kLoadsPerKTile>();
       else wait_for_dma_loads();
     }
     __syncthreads();
@@ -373,25 +411,58 @@ FSH_API int fsh_act_quant_1x128(const void* x_dev, int64_t rows, int64_t cols, i
   return check_launch("act_quant_1x128_kernel");
 }
 
+namespace fsh {
+namespace {
+
+// Shared checks and launch of the two FP8 GEMM variants.  `p` arrives with
+// the operands, sizes and scale tables filled in.
+int launch_fp8_gemm(Fp8GemmParams& p, bool column_scales, const char* who, void* stream) {
+  if (p.m < 0 || p.n < 0 || p.k < 0) return fail(FSH_EINVAL, "%s: negative size", who);
+  if (p.m == 0 || p.n == 0) return FSH_OK;
+  if (!p.xq || !p.xs || !p.wq || !p.out || (column_scales ? !p.cs : !p.ws)) return fail(FSH_EINVAL, "%s: null pointer", who);
+  if (p.k == 0 || p.k % 128 || p.k / 128 > Fp8Gemm::kMaxKTilesInLds)
+    return fail(FSH_ENOTSUP, "%s: k must be a positive multiple of 128 (pad the operands) and at most %d, got %lld", who,
+                128 * Fp8Gemm::kMaxKTilesInLds, (long long)p.k);
+  if (p.ldxq < p.k || p.ldwq < p.k || p.ldo < p.n)
+    return fail(FSH_EINVAL, "%s: a leading dimension is smaller than its row", who);
+  if (p.ldxq % 16 || p.ldwq % 16 || !aligned(p.xq, 16) || !aligned(p.wq, 16) || !aligned(p.out, 2))
+    return fail(FSH_ENOTSUP, "%s: operand rows must be 16-byte aligned", who);
+  if (static_cast<int64_t>(Fp8Gemm::BN) * p.ldwq >= (1LL << 31) || static_cast<int64_t>(Fp8Gemm::BM) * p.ldxq >= (1LL << 31) ||
+      p.m >= (1LL << 29) || p.n >= (1LL << 29))
+    return fail(FSH_ENOTSUP, "%s: a tile spans more than 2 GiB", who);
+  GemmParams& s = p.schedule;
+  memset(&s, 0, sizeof(s));
+  s.tiles_m = static_cast<int32_t>(ceil_div(p.m, (int64_t)Fp8Gemm::BM));
+  s.tiles_n = static_cast<int32_t>(ceil_div(p.n, (int64_t)Fp8Gemm::BN));
+  const int64_t tiles = static_cast<int64_t>(s.tiles_m) * s.tiles_n;
+  if (tiles > 0x3FFFFFFFLL) return fail(FSH_ENOTSUP, "%s: too many tiles", who);
+  s.tiles_per_matrix = static_cast<int32_t>(tiles);
+  s.work_items = tiles;
+  s.items_per_xcd = ceil_div(tiles, static_cast<int64_t>(kXcds));
+  static bool reserved = false;
+  if (!reserved) {
+    if (int rc = reserve_lds(&fp8_gemm_blockwise_kernel<false>, Fp8Gemm::kLdsBytes)) return rc;
+    if (int rc = reserve_lds(&fp8_gemm_blockwise_kernel<true>, Fp8Gemm::kLdsBytes)) return rc;
+    reserved = true;
+  }
+  const dim3 grid(static_cast<uint32_t>(s.items_per_xcd * kXcds)), block(Fp8Gemm::kThreads);
+  if (column_scales)
+    hipLaunchKernelGGL(fp8_gemm_blockwise_kernel<true>, grid, block, Fp8Gemm::kLdsBytes, static_cast<hipStream_t>(stream), p);
+  else
+    hipLaunchKernelGGL(fp8_gemm_blockwise_kernel<false>, grid, block, Fp8Gemm::kLdsBytes, static_cast<hipStream_t>(stream), p);
+  return check_launch("fp8_gemm_blockwise_kernel");
+}
+
+}  // namespace
+}  // namespace fsh
+
 FSH_API int fsh_fp8_gemm_1x128_128x128(const void* xq_dev, const float* xs_dev, const void* wq_dev,
                                        const float* ws_dev, void* out_dev, int64_t m, int64_t n, int64_t k,
                                        int64_t ldxq, int64_t ldwq, int64_t ldo, int64_t ws_cols, void* stream) {
   using namespace fsh;
-  if (m < 0 || n < 0 || k < 0) return fail(FSH_EINVAL, "fsh_fp8_gemm_1x128_128x128: negative size");
-  if (m == 0 || n == 0) return FSH_OK;
-  if (!xq_dev || !xs_dev || !wq_dev || !ws_dev || !out_dev)
-    return fail(FSH_EINVAL, "fsh_fp8_gemm_1x128_128x128: null pointer");
-  if (k == 0 || k % 128 || k / 128 > Fp8Gemm::kMaxKTilesInLds)
-    return fail(FSH_ENOTSUP,
-                "fsh_fp8_gemm_1x128_128x128: k must be a positive multiple of 128 (pad the operands) and at most %d, got %lld",
-                128 * Fp8Gemm::kMaxKTilesInLds, (long long)k);
-  if (ldxq < k || ldwq < k || ldo < n || ws_cols < k / 128)
-    return fail(FSH_EINVAL, "fsh_fp8_gemm_1x128_128x128: a leading dimension is smaller than its row");
-  if (ldxq % 16 || ldwq % 16 || !aligned(xq_dev, 16) || !aligned(wq_dev, 16) || !aligned(out_dev, 2))
-    return fail(FSH_ENOTSUP, "fsh_fp8_gemm_1x128_128x128: operand rows must be 16-byte aligned");
-  if (static_cast<int64_t>(Fp8Gemm::BN) * ldwq >= (1LL << 31) || static_cast<int64_t>(Fp8Gemm::BM) * ldxq >= (1LL << 31) ||
-      m >= (1LL << 30))
-    return fail(FSH_ENOTSUP, "fsh_fp8_gemm_1x128_128x128: a tile spans more than 2 GiB");
+  if (k > 0 && ws_cols < k / 128)
+    return fail(FSH_EINVAL, "fsh_fp8_gemm_1x128_128x128: the weight scale table has %lld columns, k / 128 = %lld",
+                (long long)ws_cols, (long long)(k / 128));
   Fp8GemmParams p;
   memset(&p, 0, sizeof(p));
   p.xq = static_cast<const uint8_t*>(xq_dev);
@@ -400,21 +471,44 @@ FSH_API int fsh_fp8_gemm_1x128_128x128(const void* xq_dev, const float* xs_dev, 
   p.ws = ws_dev;
   p.out = static_cast<uint16_t*>(out_dev);
   p.m = m; p.n = n; p.k = k;
-  p.ldxq = ldxq; p.ldwq = ldwq; p.ldo = ldo; p.ws_cols = ws_cols;
-  GemmParams& s = p.schedule;
-  s.tiles_m = static_cast<int32_t>(ceil_div(m, (int64_t)Fp8Gemm::BM));
-  s.tiles_n = static_cast<int32_t>(ceil_div(n, (int64_t)Fp8Gemm::BN));
-  const int64_t tiles = static_cast<int64_t>(s.tiles_m) * s.tiles_n;
-  if (tiles > 0x3FFFFFFFLL) return fail(FSH_ENOTSUP, "fsh_fp8_gemm_1x128_128x128: too many tiles");
-  s.tiles_per_matrix = static_cast<int32_t>(tiles);
-  s.work_items = tiles;
-  s.items_per_xcd = ceil_div(tiles, static_cast<int64_t>(kXcds));
-  static bool reserved = false;
-  if (!reserved) {
-    if (int rc = reserve_lds(&fp8_gemm_blockwise_kernel, Fp8Gemm::kLdsBytes)) return rc;
-    reserved = true;
-  }
-  hipLaunchKernelGGL(fp8_gemm_blockwise_kernel, dim3(static_cast<uint32_t>(s.items_per_xcd * kXcds)),
-                     dim3(Fp8Gemm::kThreads), Fp8Gemm::kLdsBytes, static_cast<hipStream_t>(stream), p);
-  return check_launch("fp8_gemm_blockwise_kernel");
+  p.ldxq = ldxq; p.ldwq = ldwq; p.ldo = ldo;
+  p.ws_cb = ws_cols; p.ws_kb = 1;
+  return launch_fp8_gemm(p, false, "fsh_fp8_gemm_1x128_128x128", stream);
+}
+
+FSH_API int fsh_fp8_gemm_1x128_128x128_dgrad(const void* gq_dev, const float* gs_dev, const void* wtq_dev,
+                                             const float* ws_dev, void* out_dev, int64_t m, int64_t in_dim,
+                                             int64_t out_dim, int64_t ldgq, int64_t ldwt, int64_t ldo,
+                                             int64_t ws_cols, void* stream) {
+  using namespace fsh;
+  if (in_dim > 0 && ws_cols < ceil_div(in_dim, (int64_t)128))
+    return fail(FSH_EINVAL, "fsh_fp8_gemm_1x128_128x128_dgrad: the weight scale table has %lld columns, in_dim needs %lld",
+                (long long)ws_cols, (long long)ceil_div(in_dim, (int64_t)128));
+  Fp8GemmParams p;
+  memset(&p, 0, sizeof(p));
+  p.xq = static_cast<const uint8_t*>(gq_dev);
+  p.xs = gs_dev;
+  p.wq = static_cast<const uint8_t*>(wtq_dev);
+  p.ws = ws_dev;
+  p.out = static_cast<uint16_t*>(out_dev);
+  p.m = m; p.n = in_dim; p.k = out_dim;
+  p.ldxq = ldgq; p.ldwq = ldwt; p.ldo = ldo;
+  p.ws_cb = 1; p.ws_kb = ws_cols;  // the weight's table read across: (input block, output block)
+  return launch_fp8_gemm(p, false, "fsh_fp8_gemm_1x128_128x128_dgrad", stream);
+}
+
+FSH_API int fsh_fp8_gemm_1x128_128x1(const void* aq_dev, const float* as_dev, const void* bq_dev,
+                                     const float* bs_dev, void* out_dev, int64_t m, int64_t n, int64_t k,
+                                     int64_t ldaq, int64_t ldbq, int64_t ldo, void* stream) {
+  using namespace fsh;
+  Fp8GemmParams p;
+  memset(&p, 0, sizeof(p));
+  p.xq = static_cast<const uint8_t*>(aq_dev);
+  p.xs = as_dev;
+  p.wq = static_cast<const uint8_t*>(bq_dev);
+  p.cs = bs_dev;
+  p.out = static_cast<uint16_t*>(out_dev);
+  p.m = m; p.n = n; p.k = k;
+  p.ldxq = ldaq; p.ldwq = ldbq; p.ldo = ldo;
+  return launch_fp8_gemm(p, true, "fsh_fp8_gemm_1x128_128x1", stream);
 }

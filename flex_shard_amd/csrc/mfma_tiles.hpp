@@ -471,9 +471,10 @@ __device__ inline void dma_touch_4(uint32_t voffset, const uint8_t* base, uint32
 // of interest, those are complete once at most `younger` are outstanding.
 template <int younger>
 __device__ inline void wait_for_dma_loads_except() {
-  static_assert(younger == 2 || younger == 13, "one immediate per use");
+  static_assert(younger == 2 || younger == 13 || younger == 14, "one immediate per use");
   if (younger == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(13)" ::: "memory");
+  else if (younger == 13) asm volatile("s_waitcnt vmcnt(13)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(14)" ::: "memory");
 }
 
 constexpr int max_int(int a, int b) { return a > b ? a : b; }

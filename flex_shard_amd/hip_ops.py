@@ -31,7 +31,9 @@ from ._native import (
 __all__ = [
     "DT_BF16", "DT_F32", "EPS_FP32", "EPS_INPUT_DTYPE", "REDUCE_POSTDIV", "REDUCE_POSTMUL",
     "REDUCE_PREMUL", "REDUCE_SUM", "SRC_BF16", "SRC_F32", "SRC_F32_AS_BF16",
-    "QuantChunkSpec", "QuantPackPlan", "accumulate_grad", "copy_segments", "gemm_nt", "muon_apply", "muon_prepare",
+    "QuantChunkSpec", "QuantPackPlan", "accumulate_grad", "act_quant_128x1_transposed", "act_quant_1x128",
+    "copy_segments", "fp8_gemm_1x128_128x1", "fp8_gemm_1x128_128x128", "fp8_gemm_1x128_128x128_dgrad",
+    "fp8_transpose", "gemm_nt", "gemm_nt_group", "muon_apply", "muon_prepare", "newton_schulz_multi",
     "newton_schulz", "newton_schulz_workspace_bytes", "pack_segments", "quantize_pack",
     "reduce_rows", "stream_ptr", "unpack_dequant", "zero_segments",
 ]
@@ -465,7 +467,7 @@ def fp8_gemm_1x128_128x128(
     blocks = k // 128
     if xs.dtype != torch.float32 or not xs.is_contiguous() or tuple(xs.shape) != (blocks, m):
         raise ValueError(f"xs must be contiguous fp32 of shape {(blocks, m)}, got {tuple(xs.shape)}")
-    if ws.dtype != torch.float32 or ws.ndim != 2 or ws.stride(1) != 1 or ws.shape[0] != -(-n // 128) or ws.shape[1] < blocks:
+    if ws.dtype != torch.float32 or ws.ndim != 2 or not _unit_column_stride(ws) or ws.shape[0] != -(-n // 128) or ws.shape[1] < blocks:
         raise ValueError(f"ws must be fp32 [{-(-n // 128)}, >= {blocks}] with contiguous rows, got {tuple(ws.shape)}")
     if out is None:
         out = torch.empty((m, n), dtype=torch.bfloat16, device=xq.device)
@@ -477,6 +479,111 @@ def fp8_gemm_1x128_128x128(
         wq.stride(0), out.stride(0), ws.stride(0), stream_ptr(xq.device),
     )
     _native.check(status, "fsh_fp8_gemm_1x128_128x128")
+    return out
+
+
+def _unit_column_stride(t: torch.Tensor) -> bool:
+    return t.shape[1] <= 1 or t.stride(1) == 1  # the stride of a single column is arbitrary
+
+
+def _fp8_matrix(name: str, t: torch.Tensor) -> None:
+    if t.dtype not in (torch.float8_e4m3fn, torch.uint8) or t.ndim != 2 or t.stride(1) != 1:
+        raise ValueError(f"{name} must be a float8_e4m3fn matrix with contiguous rows")
+
+
+def fp8_transpose(src: torch.Tensor) -> torch.Tensor:
+    """Transposed copy of a float8_e4m3fn (byte) matrix ``[rows, cols]``: returns
+    ``[cols, rows rounded up to 128]`` whose pad columns are zero.  ``cols`` and
+    the row stride must be multiples of 16."""
+    _require_gpu(src)
+    _fp8_matrix("src", src)
+    rows, cols = src.shape
+    ld_dst = -(-rows // 128) * 128
+    dst = torch.empty((cols, ld_dst), dtype=src.dtype, device=src.device)
+    if rows == 0 or cols == 0:
+        return dst
+    status = _native.lib().fsh_fp8_transpose(
+        src.data_ptr(), rows, cols, src.stride(0), dst.data_ptr(), ld_dst, stream_ptr(src.device)
+    )
+    _native.check(status, "fsh_fp8_transpose")
+    return dst
+
+
+def act_quant_128x1_transposed(x: torch.Tensor, *, eps_fp32: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
+    """Quantize every run of 128 consecutive rows of each column of the bf16
+    matrix ``x`` to float8_e4m3fn and return the bytes transposed: ``q`` is
+    ``[cols, rows rounded up to 128]`` (pad zero), the reciprocal scales are a
+    ``[rows / 128, cols]`` fp32 table.  Same arithmetic and ``eps_fp32`` rule as
+    :func:`act_quant_1x128`."""
+    _require_gpu(x)
+    if x.dtype != torch.bfloat16 or x.ndim != 2 or x.stride(1) != 1:
+        raise ValueError("x must be a bf16 matrix with contiguous rows")
+    rows, cols = x.shape
+    padded = -(-rows // 128) * 128
+    q = torch.empty((cols, padded), dtype=torch.float8_e4m3fn, device=x.device)
+    scales = torch.empty((padded // 128, cols), dtype=torch.float32, device=x.device)
+    if rows == 0 or cols == 0:
+        return q, scales
+    status = _native.lib().fsh_act_quant_128x1_transposed(
+        x.data_ptr(), rows, cols, x.stride(0), q.data_ptr(), padded, scales.data_ptr(),
+        EPS_FP32 if eps_fp32 else EPS_INPUT_DTYPE, stream_ptr(x.device),
+    )
+    _native.check(status, "fsh_act_quant_128x1_transposed")
+    return q, scales
+
+
+def fp8_gemm_1x128_128x128_dgrad(
+    gq: torch.Tensor, gs: torch.Tensor, wtq: torch.Tensor, ws: torch.Tensor, in_dim: int | None = None
+) -> torch.Tensor:
+    """``out[i, j] = bf16(sum_ob dot(gq[i, ob], wtq[j, ob]) * gs[ob, i] * ws[ob, j // 128])``:
+    the input gradient of a linear whose weight has scales ``ws`` ``[out / 128,
+    >= in / 128]``.  ``gq`` [m, out] with ``gs`` [out / 128, m] from
+    :func:`act_quant_1x128`, ``wtq`` [in, out] from :func:`fp8_transpose`; ``out``
+    (the contraction) a multiple of 128.  Returns ``[m, in_dim]``."""
+    _require_gpu(gq, gs, wtq, ws)
+    _fp8_matrix("gq", gq)
+    _fp8_matrix("wtq", wtq)
+    m, out_dim = gq.shape
+    in_dim = wtq.shape[0] if in_dim is None else in_dim
+    if wtq.shape[1] != out_dim or in_dim > wtq.shape[0]:
+        raise ValueError(f"shapes do not match: gq {tuple(gq.shape)}, wtq {tuple(wtq.shape)}, in_dim {in_dim}")
+    blocks = out_dim // 128
+    if gs.dtype != torch.float32 or not gs.is_contiguous() or tuple(gs.shape) != (blocks, m):
+        raise ValueError(f"gs must be contiguous fp32 of shape {(blocks, m)}, got {tuple(gs.shape)}")
+    if ws.dtype != torch.float32 or ws.ndim != 2 or not _unit_column_stride(ws) or ws.shape[0] < blocks or ws.shape[1] < -(-in_dim // 128):
+        raise ValueError(f"ws must be fp32 [>= {blocks}, >= {-(-in_dim // 128)}] with contiguous rows, got {tuple(ws.shape)}")
+    out = torch.empty((m, in_dim), dtype=torch.bfloat16, device=gq.device)
+    status = _native.lib().fsh_fp8_gemm_1x128_128x128_dgrad(
+        gq.data_ptr(), gs.data_ptr(), wtq.data_ptr(), ws.data_ptr(), out.data_ptr(), m, in_dim, out_dim,
+        gq.stride(0), wtq.stride(0), out.stride(0), ws.stride(0), stream_ptr(gq.device),
+    )
+    _native.check(status, "fsh_fp8_gemm_1x128_128x128_dgrad")
+    return out
+
+
+def fp8_gemm_1x128_128x1(
+    aq: torch.Tensor, a_scales: torch.Tensor, bq: torch.Tensor, b_scales: torch.Tensor
+) -> torch.Tensor:
+    """``out[i, j] = bf16(sum_kb dot(aq[i, kb], bq[j, kb]) * a_scales[kb, i] * b_scales[kb, j])``
+    for two operands quantized in runs of 128 along the contraction
+    (:func:`act_quant_128x1_transposed`)."""
+    _require_gpu(aq, a_scales, bq, b_scales)
+    _fp8_matrix("aq", aq)
+    _fp8_matrix("bq", bq)
+    k = aq.shape[1]
+    if bq.shape[1] != k:
+        raise ValueError(f"inner dimensions differ: aq {tuple(aq.shape)} vs bq {tuple(bq.shape)}")
+    m, n = aq.shape[0], bq.shape[0]
+    blocks = k // 128
+    for name, t, size in (("a_scales", a_scales, aq.shape[0]), ("b_scales", b_scales, bq.shape[0])):
+        if t.dtype != torch.float32 or not t.is_contiguous() or tuple(t.shape) != (blocks, size):
+            raise ValueError(f"{name} must be contiguous fp32 of shape {(blocks, size)}, got {tuple(t.shape)}")
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=aq.device)
+    status = _native.lib().fsh_fp8_gemm_1x128_128x1(
+        aq.data_ptr(), a_scales.data_ptr(), bq.data_ptr(), b_scales.data_ptr(), out.data_ptr(), m, n, k,
+        aq.stride(0), bq.stride(0), out.stride(0), stream_ptr(aq.device),
+    )
+    _native.check(status, "fsh_fp8_gemm_1x128_128x1")
     return out
 
 

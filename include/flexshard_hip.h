@@ -271,6 +271,56 @@ int fsh_fp8_gemm_1x128_128x128(const void* xq_dev, const float* xs_dev, const vo
                                const float* ws_dev, void* out_dev, int64_t m, int64_t n, int64_t k,
                                int64_t ldxq, int64_t ldwq, int64_t ldo, int64_t ws_cols, void* stream);
 
+/* ------------------------------------------------------------------------
+ * 9. Backward products of the same linear layer.  Replace the device work of
+ * blockwise_fp8/fp8_blockwise_linear.py:93-162 (Fp8BlockwiseGemms.backward):
+ *
+ * input gradient (:107-126)   grad_x = grad_out . W: fsh_act_quant_1x128 on
+ *   grad_out (runs along the output index), fsh_fp8_transpose of the weight
+ *   bytes (replaces _as_column_major_2d at :113; the scales are read across,
+ *   no copy), fsh_fp8_gemm_1x128_128x128_dgrad.
+ * weight gradient (:127-161)  grad_w = grad_out^T . x: both operands through
+ *   fsh_act_quant_128x1_transposed (replaces torchao's
+ *   triton_fp8_blockwise_act_quant_transposed_lhs at :134 and
+ *   triton_fp8_blockwise_act_quant_rhs at :139; runs of 128 tokens), then
+ *   fsh_fp8_gemm_1x128_128x1 (replaces triton_fp8_gemm_1x128_128x1 at :144).
+ *
+ * fsh_fp8_transpose: dst[c][r] = src[r][c] for a [rows, cols] byte matrix;
+ * dst is [cols, ld_dst] with rows <= ld_dst <= rows rounded up to 128, the
+ * columns from `rows` on written as zero.
+ *
+ * fsh_act_quant_128x1_transposed: x is [rows, cols] bf16 with row stride ldx.
+ * Every run of 128 consecutive rows of a column (the last run zero-padded) is
+ * quantized like a weight tile (see section 8).  q_dev is [cols, ldq] bytes,
+ * q[c][r], ldq = rows rounded up to 128 with the pad written as zero;
+ * scales_dev is the [ldq / 128, cols] table of 1.0f / scale.
+ *
+ * fsh_fp8_gemm_1x128_128x128_dgrad:
+ *   out[i][j] = bf16( sum over ob of dot(gq[i][ob], wtq[j][ob])
+ *                                  * (gs[ob][i] * ws[ob][j / 128]) ),
+ * gq [m, out_dim] and its [out_dim / 128, m] scales from fsh_act_quant_1x128,
+ * wtq [in_dim, out_dim] the transposed weight bytes, ws the weight's own
+ * [out_dim / 128, ws_cols] table, out [m, in_dim] bf16.  out_dim (the
+ * contraction length) must be a multiple of 128.
+ *
+ * fsh_fp8_gemm_1x128_128x1:
+ *   out[i][j] = bf16( sum over kb of dot(aq[i][kb], bq[j][kb])
+ *                                  * (as[kb][i] * bs[kb][j]) ),
+ * aq [m, k], bq [n, k] bytes and their [k / 128, m] and [k / 128, n] tables
+ * (both as fsh_act_quant_128x1_transposed writes them), out [m, n] bf16.
+ * ---------------------------------------------------------------------- */
+int fsh_fp8_transpose(const void* src_dev, int64_t rows, int64_t cols, int64_t ld_src, void* dst_dev,
+                      int64_t ld_dst, void* stream);
+int fsh_act_quant_128x1_transposed(const void* x_dev, int64_t rows, int64_t cols, int64_t ldx, void* q_dev,
+                                   int64_t ldq, float* scales_dev, int32_t eps_mode, void* stream);
+int fsh_fp8_gemm_1x128_128x128_dgrad(const void* gq_dev, const float* gs_dev, const void* wtq_dev,
+                                     const float* ws_dev, void* out_dev, int64_t m, int64_t in_dim,
+                                     int64_t out_dim, int64_t ldgq, int64_t ldwt, int64_t ldo,
+                                     int64_t ws_cols, void* stream);
+int fsh_fp8_gemm_1x128_128x1(const void* aq_dev, const float* as_dev, const void* bq_dev,
+                             const float* bs_dev, void* out_dev, int64_t m, int64_t n, int64_t k,
+                             int64_t ldaq, int64_t ldbq, int64_t ldo, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

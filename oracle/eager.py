@@ -107,6 +107,80 @@ def fp8_gemm_1x128_128x128(
     return acc.to(out_dtype)
 
 
+def act_quant_128x1_transposed(
+    x: torch.Tensor, block: int = 128, fp8_dtype: torch.dtype = torch.float8_e4m3fn
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """Token-run quantizers of blockwise_fp8/fp8_blockwise_linear.py:134-143:
+    torchao's ``triton_fp8_blockwise_act_quant_transposed_lhs`` (output
+    ``[cols, rows]`` row-major, scales per column and run of ``block`` rows) and
+    ``triton_fp8_blockwise_act_quant_rhs`` (output ``[rows, cols]`` column-major
+    = the same bytes, scales ``[rows / block, cols]``).  Same provenance, same
+    per-run arithmetic and the same PARITY UNPINNED note as
+    ``act_quant_1x128``; pinned through the tile quantizer (a run is a
+    one-column tile) and the identity with ``act_quant_1x128`` of the
+    transposed matrix.  Returns the bytes transposed, ``[cols, rows padded to
+    whole runs]`` (pad zero), and the reciprocal scales ``[runs, cols]``."""
+    if x.ndim != 2:
+        raise ValueError(f"expects a 2D matrix, got {tuple(x.shape)}")
+    rows, cols = x.shape
+    runs = -(-rows // block)
+    fp8_max = torch.finfo(fp8_dtype).max
+    quant = torch.zeros((cols, runs * block), dtype=fp8_dtype)
+    recip = torch.empty((runs, cols), dtype=torch.float32)
+    for run in range(runs):
+        piece = x[run * block : (run + 1) * block].to(torch.float32)  # [<= block, cols]
+        amax = piece.abs().amax(dim=0).clamp(min=EPS).to(torch.float64)
+        scale = (fp8_max / amax).to(torch.float32)
+        q = (piece * scale[None, :]).clamp(-fp8_max, fp8_max).to(fp8_dtype)
+        quant[:, run * block : run * block + piece.shape[0]] = q.t()
+        recip[run] = 1.0 / scale
+    return quant, recip
+
+
+def fp8_gemm_1x128_128x1(
+    aq: torch.Tensor, a_scales: torch.Tensor, bq: torch.Tensor, b_scales: torch.Tensor, block: int = 128,
+    out_dtype: torch.dtype = torch.bfloat16,
+) -> torch.Tensor:
+    """Scaled product of blockwise_fp8/fp8_blockwise_linear.py:144-155
+    (torchao's ``triton_fp8_gemm_1x128_128x1``; PARITY UNPINNED against
+    torchao, as above): both operands carry one scale per row and k-block.
+    ``aq`` [m, k], ``bq`` [n, k], ``a_scales`` [k / block, m], ``b_scales``
+    [k / block, n]; fp32 accumulation in k order, one cast."""
+    m, k = aq.shape
+    n = bq.shape[0]
+    acc = torch.zeros((m, n), dtype=torch.float32)
+    for kb in range(k // block):
+        a = aq[:, kb * block : (kb + 1) * block].to(torch.float32)
+        b = bq[:, kb * block : (kb + 1) * block].to(torch.float32)
+        acc += (a @ b.t()) * a_scales[kb].to(torch.float32)[:, None] * b_scales[kb].to(torch.float32)[None, :]
+    return acc.to(out_dtype)
+
+
+def fp8_linear_backward(
+    grad_out: torch.Tensor, x: torch.Tensor, wq: torch.Tensor, ws: torch.Tensor, block: int = 128,
+    out_dtype: torch.dtype = torch.bfloat16,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """``Fp8BlockwiseGemms.backward`` (blockwise_fp8/fp8_blockwise_linear.py:93-162)
+    for a 2D weight ``wq`` [out, in] with tile scales ``ws``: returns
+    ``(grad_x [tokens, in], grad_weight [out, in])``.
+
+    grad_x (:107-126): grad_out zero-padded to whole runs of the output index,
+    quantized 1 x block, times the weight read as ``[out, in]`` with its scales
+    (the column-major copies of :113-114 change layout, not values).
+    grad_weight (:127-161): both operands zero-padded to whole runs of tokens
+    and quantized along the tokens; 1 x block times block x 1 product."""
+    out_dim, in_dim = wq.shape
+    pad_out, pad_in = -(-out_dim // block) * block, -(-in_dim // block) * block
+    wq_padded = torch.zeros((pad_out, pad_in), dtype=wq.dtype)
+    wq_padded.view(torch.uint8)[:out_dim, :in_dim] = wq.view(torch.uint8)
+    gq, gs = act_quant_1x128(grad_out, block, wq.dtype)  # pads the output index itself
+    grad_x = fp8_gemm_1x128_128x128(gq, gs, wq_padded.t().contiguous(), ws.t().contiguous(), block, out_dtype)
+    gtq, gts = act_quant_128x1_transposed(grad_out, block, wq.dtype)
+    xtq, xts = act_quant_128x1_transposed(x, block, wq.dtype)
+    grad_w = fp8_gemm_1x128_128x1(gtq, gts, xtq, xts, block, out_dtype)
+    return grad_x[:, :in_dim].contiguous(), grad_w[:out_dim, :in_dim].contiguous()
+
+
 def accumulate_microbatches(grads: list[torch.Tensor]) -> torch.Tensor:
     """flex_shard/bucket_runtime.py:931-933 -- each microbatch's bf16 grad is
     cast to the fp32 accumulation dtype and added in arrival order."""

@@ -121,5 +121,5 @@ def test_forward_of_the_prequantized_linear(device):
         Fp8BlockwiseGemms(block_size=64).forward(x.to(device), flat)
     with pytest.raises(ValueError, match="input dim"):
         gemms.forward(x.to(device)[:, :128].contiguous(), flat)
-    with pytest.raises(NotImplementedError, match="not built"):
-        gemms.backward(None, None, flat, True, True)
+    with pytest.raises(ValueError, match="block_size"):
+        Fp8BlockwiseGemms(block_size=64).backward(x.to(device), x.to(device), flat, True, True)

@@ -1,0 +1,237 @@
+"""GPU parity of the backward products of the prequantized-weight linear: the
+byte transpose and the token-run quantizer are bit-exact against the oracle,
+the two scaled FP8 GEMMs are within one bf16 rounding plus summation-order
+noise of the oracle's fp32 result (relative 2^-7) and exact where the
+arithmetic is exact."""
+
+import pytest
+import torch
+
+from flex_shard_amd import hip_ops
+from flex_shard_amd.blockwise_fp8 import (
+    BlockwiseFp8Weight,
+    FlexShardFloat8BlockwiseLinear,
+    Fp8BlockwiseGemms,
+    prequantized_linear,
+)
+from oracle import eager
+
+pytestmark = pytest.mark.gpu
+E4M3 = torch.float8_e4m3fn
+RTOL = 2.0**-7
+
+
+def _bits(t):
+    return t.contiguous().view(torch.int32)
+
+
+def _close(got, want):
+    return torch.allclose(got.cpu().float(), want, rtol=RTOL, atol=1e-3 * want.abs().max().item())
+
+
+def _small_int_fp8(shape, gen, high=1):
+    return torch.randint(-high, high + 1, shape, generator=gen).to(torch.float32).to(E4M3)
+
+
+@pytest.mark.parametrize("rows,cols", [(128, 128), (384, 256), (130, 144), (1, 16), (500, 1040), (4096, 1024)])
+def test_transpose_is_exact(device, rows, cols):
+    gen = torch.Generator().manual_seed(rows + cols)
+    src = torch.randint(0, 256, (rows, cols), generator=gen, dtype=torch.uint8)
+    got = hip_ops.fp8_transpose(src.to(device)).cpu()
+    padded = -(-rows // 128) * 128
+    assert got.shape == (cols, padded)
+    assert torch.equal(got[:, :rows], src.t())
+    assert (got[:, rows:] == 0).all()
+
+
+def test_transpose_of_a_strided_view_and_errors(device):
+    gen = torch.Generator().manual_seed(1)
+    wide = torch.randint(0, 256, (200, 512), generator=gen, dtype=torch.uint8).to(device)
+    view = wide[:, 64:320].view(E4M3)
+    got = hip_ops.fp8_transpose(view)
+    assert got.dtype == E4M3 and torch.equal(got.view(torch.uint8)[:, :200].cpu(), wide[:, 64:320].t().cpu())
+    with pytest.raises(RuntimeError, match="multiples of 16"):
+        hip_ops.fp8_transpose(wide[:, :40])
+    with pytest.raises(ValueError, match="contiguous rows"):
+        hip_ops.fp8_transpose(wide.t())
+    assert hip_ops.fp8_transpose(wide[:0]).shape == (512, 0)
+
+
+@pytest.mark.parametrize("rows,cols", [(128, 128), (256, 384), (130, 136), (77, 8), (1000, 520), (4096, 256), (1, 128)])
+def test_token_run_quantizer_is_bit_exact(device, rows, cols):
+    gen = torch.Generator().manual_seed(rows * 5 + cols)
+    x = (torch.randn(rows, cols, generator=gen) * 0.5).bfloat16()
+    x[torch.rand(rows, cols, generator=gen) < 0.002] *= 60  # outliers
+    if rows >= 256:
+        x[128:256, cols // 2] = 0  # an all-zero run
+    x[0, 0] = 0.0
+    x[rows - 1, cols - 1] = 3.0e38  # the largest magnitudes saturate nothing: amax scales them to 448
+    x[rows // 2, 1] = 1e-40  # a subnormal input
+    q, s = hip_ops.act_quant_128x1_transposed(x.to(device))
+    oq, os_ = eager.act_quant_128x1_transposed(x)
+    assert q.shape == oq.shape and s.shape == os_.shape
+    assert torch.equal(q.cpu().view(torch.uint8), oq.view(torch.uint8))
+    assert torch.equal(_bits(s.cpu()), _bits(os_))
+
+
+def test_token_run_quantizer_strided_rows_and_eps_switch(device):
+    gen = torch.Generator().manual_seed(4)
+    wide = torch.randn(300, 640, generator=gen).bfloat16().to(device)
+    view = wide[:, 128:512]
+    q, s = hip_ops.act_quant_128x1_transposed(view)
+    oq, os_ = eager.act_quant_128x1_transposed(view.cpu())
+    assert torch.equal(q.cpu().view(torch.uint8), oq.view(torch.uint8)) and torch.equal(_bits(s.cpu()), _bits(os_))
+    zeros = torch.zeros(128, 8, dtype=torch.bfloat16, device=device)
+    _, s32 = hip_ops.act_quant_128x1_transposed(zeros)
+    _, s16 = hip_ops.act_quant_128x1_transposed(zeros, eps_fp32=False)
+    assert (_bits(s32.cpu()) == 0x2720D7C5).all() and (_bits(s16.cpu()) == 0x27212492).all()
+    with pytest.raises(RuntimeError, match="multiples of 8"):
+        hip_ops.act_quant_128x1_transposed(torch.zeros(128, 12, dtype=torch.bfloat16, device=device))
+
+
+@pytest.mark.parametrize("m,n,k", [(128, 256, 128), (70, 200, 384), (300, 520, 256), (1, 8, 128), (129, 257, 1024)])
+def test_column_scaled_gemm_integer_products_are_exact(device, m, n, k):
+    gen = torch.Generator().manual_seed(m + n + k + 1)
+    aq, bq = _small_int_fp8((m, k), gen), _small_int_fp8((n, k), gen)
+    a_s = torch.exp2(torch.randint(-2, 3, (k // 128, m), generator=gen).float())
+    b_s = torch.exp2(torch.randint(-2, 3, (k // 128, n), generator=gen).float())
+    want = eager.fp8_gemm_1x128_128x1(aq, a_s, bq, b_s, out_dtype=torch.float32)
+    got = hip_ops.fp8_gemm_1x128_128x1(aq.to(device), a_s.to(device), bq.to(device), b_s.to(device))
+    assert torch.equal(got.cpu(), want.bfloat16())
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 512, 512), (200, 384, 256), (1024, 1032, 2048), (77, 130, 128)])
+def test_column_scaled_gemm_matches_the_oracle(device, m, n, k):
+    gen = torch.Generator().manual_seed(m * 3 + n + k + 1)
+    a = torch.randn(k, m, generator=gen).bfloat16()
+    b = (torch.randn(k, n, generator=gen) * 0.02).bfloat16()
+    aq, a_s = eager.act_quant_128x1_transposed(a)
+    bq, b_s = eager.act_quant_128x1_transposed(b)
+    want = eager.fp8_gemm_1x128_128x1(aq, a_s, bq, b_s, out_dtype=torch.float32)
+    got = hip_ops.fp8_gemm_1x128_128x1(aq.to(device), a_s.to(device), bq.to(device), b_s.to(device))
+    assert _close(got, want)
+
+
+@pytest.mark.parametrize("tokens,out_dim,in_dim", [(128, 256, 256), (70, 384, 200), (300, 128, 520), (1000, 1024, 1024)])
+def test_input_gradient_product(device, tokens, out_dim, in_dim):
+    """Against the oracle, and bit for bit against the forward kernel fed with
+    explicitly transposed copies of the weight bytes AND scales (the kernel
+    reads the scale table across instead)."""
+    gen = torch.Generator().manual_seed(tokens + out_dim + in_dim)
+    w = (torch.randn(out_dim, in_dim, generator=gen) * 0.05).bfloat16()
+    g = (torch.randn(tokens, out_dim, generator=gen) * 0.01).bfloat16()
+    wq, ws = eager.quantize_blockwise(w, 128)
+    gq, gs = eager.act_quant_1x128(g)
+    in_pad = -(-in_dim // 16) * 16
+    wq_dev = torch.zeros(out_dim, in_pad, dtype=torch.uint8, device=device)
+    wq_dev[:, :in_dim] = wq.view(torch.uint8).to(device)
+    wt = hip_ops.fp8_transpose(wq_dev.view(E4M3))
+    got = hip_ops.fp8_gemm_1x128_128x128_dgrad(gq.to(device), gs.to(device), wt, ws.to(device), in_dim=in_dim)
+    assert got.shape == (tokens, in_dim)
+    want = eager.fp8_gemm_1x128_128x128(gq, gs, wq.t().contiguous(), ws.t().contiguous(), out_dtype=torch.float32)
+    assert _close(got, want)
+    same = hip_ops.fp8_gemm_1x128_128x128(gq.to(device), gs.to(device), wt[:in_dim], ws.t().contiguous().to(device))
+    assert torch.equal(got, same)
+
+
+def _case(gen, tokens, out_shape, in_dim, device):
+    out_dim = 1
+    for extent in out_shape:
+        out_dim *= extent
+    w = (torch.randn(out_dim, in_dim, generator=gen) * 0.05).bfloat16()
+    x = torch.randn(tokens, in_dim, generator=gen).bfloat16()
+    g = (torch.randn(tokens, out_dim, generator=gen) * 0.01).bfloat16()
+    wq, ws = eager.quantize_blockwise(w, 128)
+    weight = BlockwiseFp8Weight(wq.to(device).view(*out_shape, in_dim), ws.to(device), 128, orig_dtype=torch.bfloat16)
+    return w, x, g, wq, ws, weight
+
+
+@pytest.mark.parametrize(
+    "tokens,out_shape,in_dim", [(256, (256,), 384), (77, (200,), 136), (150, (2, 192), 256), (130, (72,), 100)]
+)
+def test_backward_of_the_prequantized_linear(device, tokens, out_shape, in_dim):
+    """Fp8BlockwiseGemms.backward against the oracle's restatement of the
+    reference's steps and, loosely, against the unquantized gradients; odd
+    token counts and widths exercise every padding branch, the stacked weight
+    returns a gradient of the parameter's shape."""
+    gen = torch.Generator().manual_seed(tokens * 3 + in_dim)
+    w, x, g, wq, ws, weight = _case(gen, tokens, out_shape, in_dim, device)
+    gemms = Fp8BlockwiseGemms(block_size=128)
+    grad_x, grad_w = gemms.backward(g.to(device), x.to(device), weight, True, True)
+    want_x, want_w = eager.fp8_linear_backward(g, x, wq, ws, out_dtype=torch.float32)
+    assert grad_x.shape == x.shape and grad_x.dtype == torch.bfloat16
+    assert grad_w.shape == weight.shape and grad_w.dtype == torch.bfloat16 and grad_w.is_contiguous()
+    assert _close(grad_x, want_x)
+    assert _close(grad_w.view(w.shape), want_w)
+    exact_x, exact_w = g.double() @ w.double(), g.double().t() @ x.double()
+    assert (grad_x.cpu().double() - exact_x).norm() <= 0.06 * exact_x.norm()
+    assert (grad_w.view(w.shape).cpu().double() - exact_w).norm() <= 0.06 * exact_w.norm()
+    only_x = gemms.backward(g.to(device), x.to(device), weight, True, False)
+    only_w = gemms.backward(g.to(device), x.to(device), weight, False, True)
+    assert only_x[1] is None and only_w[0] is None
+    assert torch.equal(only_x[0], grad_x) and torch.equal(only_w[1], grad_w)
+    with pytest.raises(ValueError, match="grad_output"):
+        gemms.backward(g.to(device)[:, :8], x.to(device), weight, True, True)
+    with pytest.raises(ValueError, match="activation"):
+        gemms.backward(g.to(device), x.to(device)[:-1], weight, True, True)
+
+
+def test_autograd_through_the_prequantized_linear(device):
+    gen = torch.Generator().manual_seed(11)
+    w, x, g, wq, ws, _ = _case(gen, 96, (256,), 128, device)
+    weight = BlockwiseFp8Weight(wq.to(device), ws.to(device), 128, orig_dtype=torch.bfloat16, requires_grad=True)
+    bias = torch.randn(256, generator=gen).bfloat16().to(device).requires_grad_()
+    x_dev = x.to(device).view(4, 24, 128).requires_grad_()
+    out = prequantized_linear(x_dev, weight, bias)
+    assert out.shape == (4, 24, 256)
+    out.backward(g.to(device).view(4, 24, 256))
+    gemms = Fp8BlockwiseGemms(block_size=128)
+    want_x, want_w = gemms.backward(g.to(device), x.to(device), weight.detach(), True, True)
+    assert torch.equal(x_dev.grad.view(96, 128), want_x)
+    assert torch.equal(weight.grad, want_w)
+    assert torch.equal(bias.grad, g.to(device).sum(dim=0))
+    plain = gemms.forward(x.to(device), weight.detach())
+    assert torch.equal(out.detach().view(96, 256), plain + bias.detach())
+
+    linear = torch.nn.Linear(128, 256, bias=False, device=device, dtype=torch.bfloat16)
+    module = FlexShardFloat8BlockwiseLinear.from_float(linear)
+    with pytest.raises(TypeError, match="BlockwiseFp8Weight"):
+        module(x.to(device))
+    module._parameters["weight"] = weight  # what an FP8 unshard installs for the span of a forward/backward
+    assert torch.equal(module(x.to(device)).detach(), plain)
+
+
+def test_llama_sized_gradients_on_sampled_entries(device):
+    """At the size the measurements quote (8192 tokens, a [4096, 14336]
+    weight gradient and its input gradient) a sample of output entries is
+    checked against fp64 dot products of the dequantized operands."""
+    gen = torch.Generator(device=device).manual_seed(5)
+    tokens, out_dim, in_dim = 8192, 4096, 14336
+    x = torch.randn(tokens, in_dim, generator=gen, device=device, dtype=torch.float32).bfloat16()
+    g = (torch.randn(tokens, out_dim, generator=gen, device=device, dtype=torch.float32) * 0.01).bfloat16()
+    wq = torch.randint(0, 256, (out_dim, in_dim), generator=gen, device=device, dtype=torch.uint8)
+    wq[(wq & 0x7F) == 0x7F] = 0x3C  # no NaN encodings
+    ws = torch.rand(out_dim // 128, in_dim // 128, generator=gen, device=device) * 1e-3 + 1e-4
+    weight = BlockwiseFp8Weight(wq.view(E4M3), ws, 128, orig_dtype=torch.bfloat16)
+    grad_x, grad_w = Fp8BlockwiseGemms(block_size=128).backward(g, x, weight, True, True)
+
+    gq, gs = hip_ops.act_quant_1x128(g)
+    gtq, gts = hip_ops.act_quant_128x1_transposed(g)
+    xtq, xts = hip_ops.act_quant_128x1_transposed(x)
+    cpu_gen = torch.Generator().manual_seed(6)
+    rows = torch.randint(0, tokens, (64,), generator=cpu_gen).tolist()
+    cols = torch.randint(0, in_dim, (64,), generator=cpu_gen).tolist()
+    outs = torch.randint(0, out_dim, (64,), generator=cpu_gen).tolist()
+    for t, i, o in zip(rows, cols, outs):
+        # grad_x[t, i] = sum_o deq(g)[t, o] * deq(w)[o, i]
+        g_row = (gq[t].double().view(-1, 128) * gs[:, t].double()[:, None]).view(-1)
+        w_col = wq.view(E4M3)[:, i].double() * ws[:, i // 128].double().repeat_interleave(128)
+        want = float(g_row @ w_col)
+        scale = float(g_row.abs() @ w_col.abs())
+        assert abs(float(grad_x[t, i]) - want) <= RTOL * abs(want) + 1e-5 * scale
+        # grad_w[o, i] = sum_t deq(g^T)[o, t] * deq(x^T)[i, t]
+        g_col = (gtq[o].double().view(-1, 128) * gts[:, o].double()[:, None]).view(-1)
+        x_col = (xtq[i].double().view(-1, 128) * xts[:, i].double()[:, None]).view(-1)
+        want = float(g_col @ x_col)
+        scale = float(g_col.abs() @ x_col.abs())
+        assert abs(float(grad_w[o, i]) - want) <= RTOL * abs(want) + 1e-5 * scale
