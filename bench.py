@@ -265,8 +265,29 @@ def bench_muon(device, reps=3):
     _, ms = _event_ms(lambda i: opt.step(grads), reps, 1)
     per = ms / reps
     flops = opt.flops_per_step()
+    # The orthogonalization alone (normalization + 5 iterations on all 48
+    # matrices, one fsh_newton_schulz_multi call), without the momentum and
+    # update kernels around it: inputs restored outside the timed region.
+    from flex_shard_amd import hip_ops
+
+    problems = [(opt._batch[shape], opt._workspace[shape]) for shape in opt._groups]
+    saved = [torch.stack([grads[i] for i in opt._groups[shape]]) for shape in opt._groups]
+    ns_ms = 0.0
+    for rep in range(reps + 1):
+        for (batch, _), keep in zip(problems, saved):
+            batch.copy_(keep)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        hip_ops.newton_schulz_multi(problems, opt.ns_coefficients, opt.ns_steps, opt.eps)
+        stop.record()
+        torch.cuda.synchronize()
+        if rep:  # the first call is a warm-up
+            ns_ms += start.elapsed_time(stop)
+    ns_per = ns_ms / reps
     return {"step_ms": per, "ns_flop": flops, "ns_TFLOPs": flops / per / 1e9,
-            "frac_of_bf16_mfma_peak": flops / per / 1e9 / BF16_MFMA_PEAK_TFLOPS}
+            "frac_of_bf16_mfma_peak": flops / per / 1e9 / BF16_MFMA_PEAK_TFLOPS,
+            "newton_schulz_only_ms": ns_per, "newton_schulz_only_TFLOPs": flops / ns_per / 1e9,
+            "newton_schulz_only_frac_of_bf16_mfma_peak": flops / ns_per / 1e9 / BF16_MFMA_PEAK_TFLOPS}
 
 
 def bench_fp8_linear(device, tokens: int = 8192, reps: int = 10):
