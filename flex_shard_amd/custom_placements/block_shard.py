@@ -19,7 +19,6 @@ from dataclasses import dataclass
 from typing import TYPE_CHECKING, Any
 
 import torch
-import torch.distributed as dist
 import torch.nn as nn
 
 from ..placement_contract import (
@@ -35,8 +34,10 @@ from ..placement_contract import (
 from ..profiling import record_comm, record_copy_in, record_copy_out, record_range
 from ._copy_kernels import SegmentPackDescriptor
 from .utils import (
+    all_gather_rows,
     copy_tensor_to_dtype,
     foreach_copy_,
+    group_size,
     pack_segments_into_flat_buffer_if_supported,
     pack_tensors_into_flat_buffer_with_scratch,
     reduce_scatter_grads,
@@ -463,10 +464,10 @@ class BucketedBlockShard(Placement):
         else:
             bucket = send.new_empty(layout.global_numel)
             prepared.buffers.insert(1, bucket)
-        world_size = dist.get_world_size(state.pg)
+        world_size = group_size(state.pg)
         target = bucket if world_size * send.numel() == bucket.numel() else bucket.new_empty(world_size * send.numel())
         with record_comm("FlexShard::all_gather", state.debug_fqn):
-            work = dist.all_gather_into_tensor(target, send, group=state.pg, async_op=async_op)
+            work = all_gather_rows(target, send, state.pg, async_op=async_op)
         if target is not bucket:
             if work is not None:
                 work.wait()

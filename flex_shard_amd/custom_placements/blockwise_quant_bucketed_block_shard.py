@@ -22,7 +22,6 @@ from dataclasses import dataclass
 from typing import TYPE_CHECKING, Any
 
 import torch
-import torch.distributed as dist
 import torch.nn as nn
 
 from .. import hip_ops
@@ -41,6 +40,7 @@ from .quant_plan import ScaleRegion as _ScaleRegion
 from .quant_plan import align_up as _align_up
 from .quant_plan import ceil_div as _ceil_div
 from .quant_plan import matrix_shape as _matrix_shape
+from .utils import all_gather_rows
 
 if TYPE_CHECKING:
     from ..bucket_storage import ParamInfo
@@ -624,9 +624,7 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         state = self._unshard_state(prepared)
         local, gathered = prepared.buffers
         with record_comm("FlexShard::all_gather", state.debug_fqn):
-            return dist.all_gather_into_tensor(
-                output_tensor=gathered, input_tensor=local, group=state.pg, async_op=async_op
-            )
+            return all_gather_rows(gathered, local, state.pg, async_op=async_op)
 
     def finish_prepared_unshard(self, prepared: PlacementPreparedUnshard) -> PlacementUnshardResult:
         state = self._unshard_state(prepared)

@@ -167,7 +167,8 @@ def reduce_grads_on_one_rank(grads: torch.Tensor, reduction: "GradientReduction"
 
 
 class LocalReduceGroup:
-    """One-GPU stand-in for a reduce-scatter group of ``world_size`` ranks.
+    """One-GPU stand-in for the process group of ``world_size`` ranks: serves
+    the reduce-scatter of the gradient path and the all-gather of the unshard.
 
     ``contributions`` is a [world_size, world_size * segment] tensor: row r is
     the reduce-scatter input rank r would send (``world_size`` padded rank
@@ -182,6 +183,8 @@ class LocalReduceGroup:
         self._rank = rank
         self.contributions: torch.Tensor | None = None
         self.deposited: set[int] = set()
+        #: all-gather rows of the other ranks, by rank (see ``all_gather_rows``)
+        self.gather_rows: dict[int, torch.Tensor] = {}
 
     def size(self) -> int:
         return self._world_size
@@ -206,6 +209,39 @@ class LocalReduceGroup:
         assert self.contributions is not None
         self.contributions[rank].copy_(send_buf.reshape(-1))
         self.deposited.add(rank)
+
+
+def group_size(group: Any) -> int:
+    """Ranks of a process group or of its one-GPU stand-in."""
+    if isinstance(group, LocalReduceGroup):
+        return group.size()
+    return dist.get_world_size(group)
+
+
+def all_gather_rows(output: torch.Tensor, input: torch.Tensor, group: Any, *, async_op: bool = False) -> Any | None:
+    """All-gather equal rows into ``output`` (``world_size`` rows back to back).
+
+    With a :class:`LocalReduceGroup` the exchange is local: this rank's
+    ``input`` lands in its row and every other rank's row is copied from
+    ``group.gather_rows`` (which the harness fills with what those ranks would
+    send; a one-rank group needs none).  With a ``torch.distributed`` group it
+    is one collective, as in the reference."""
+    if isinstance(group, LocalReduceGroup):
+        world, rank = group.size(), group.rank()
+        if output.numel() != world * input.numel():
+            raise ValueError(f"all-gather output has {output.numel()} elements, expected {world} x {input.numel()}")
+        missing = sorted(set(range(world)) - {rank} - set(group.gather_rows))
+        if missing:
+            raise ValueError(f"LocalReduceGroup is missing the all-gather rows of ranks {missing}.")
+        rows = output.view(world, input.numel())
+        rows[rank].copy_(input.reshape(-1))
+        for other, row in group.gather_rows.items():
+            if other != rank:
+                rows[other].copy_(row.reshape(-1))
+        return None
+    if group is None:
+        raise ValueError("all_gather_rows needs a process group (or a LocalReduceGroup on one GPU); got None.")
+    return dist.all_gather_into_tensor(output, input, group=group, async_op=async_op)
 
 
 def _local_reduce(output: torch.Tensor, group: LocalReduceGroup, reduction: "GradientReduction") -> None:
@@ -237,7 +273,8 @@ def reduce_scatter_grads(output: torch.Tensor, input: torch.Tensor, reduction: "
     """Reduce-scatter packed gradients into ``output`` as ``reduction`` asks.
 
     With a :class:`LocalReduceGroup` the reduction runs on this GPU (``input``
-    is deposited as this rank's contribution unless already present); with a
+    is deposited as this rank's contribution unless already present) and
+    consumes the deposits; with a
     ``torch.distributed`` group it is one collective, as in the reference."""
     if isinstance(group, LocalReduceGroup):
         if group.rank() not in group.deposited:
@@ -246,6 +283,7 @@ def reduce_scatter_grads(output: torch.Tensor, input: torch.Tensor, reduction: "
         if missing:
             raise ValueError(f"LocalReduceGroup is missing the contributions of ranks {missing}.")
         _local_reduce(output, group, reduction)
+        group.deposited.clear()  # consumed: the next reduction needs fresh contributions
         return
     if group is None:
         raise ValueError(
@@ -284,10 +322,12 @@ def pack_segments_into_flat_buffer_if_supported(
 
 __all__ = [
     "LocalReduceGroup",
+    "all_gather_rows",
     "copy_tensor_to_dtype",
     "copy_tensors_into_flat_buffer",
     "foreach_copy_",
     "gradient_reduce_plan",
+    "group_size",
     "make_segment_pack_descriptor_if_supported",
     "pack_segments_into_flat_buffer_if_supported",
     "pack_tensors_into_flat_buffer",

@@ -1,0 +1,165 @@
+"""The placements under a real forward and backward on one GPU: the stream
+hand-off (side-stream unshard and gradient reduction, event ordering, buffer
+release), persistent unsharded parameters and their refill, reshard, and the
+accumulation of the reduced shards -- checked bit for bit against the same
+kernels called directly on the current stream."""
+
+import pytest
+import torch
+import torch.nn as nn
+
+from flex_shard_amd import Fp8BucketedBlockShard, GradientReduction, LocalReduceGroup
+from flex_shard_amd.blockwise_fp8 import (
+    BlockwiseFp8Weight,
+    Fp8BlockwiseGemms,
+    convert_to_flex_shard_float8_blockwise_linear,
+    make_blockwise_fp8_weight,
+    prequantized_linear,
+)
+from flex_shard_amd.custom_placements.fp8_bucketed_block_shard import _quantize_dense_weight_to_blockwise_fp8
+from flex_shard_amd.flex_shard import BucketCommContext, BucketRuntime, StreamHandoff, begin_bucket_unshard
+from flex_shard_amd.testing import FakeMesh, local_rows, make_param_infos
+
+pytestmark = pytest.mark.gpu
+
+
+def _mlp(device, gen):
+    model = nn.Sequential(nn.Linear(256, 384, bias=False), nn.Linear(384, 256, bias=False))
+    with torch.no_grad():
+        for p in model.parameters():
+            p.copy_(torch.randn(p.shape, generator=gen) * 0.05)
+    return model.to(device=device, dtype=torch.bfloat16)
+
+
+def _direct(weights, x, grad_out):
+    """Forward and backward of the two-layer MLP with the kernels called
+    directly: returns (out, grad_x, [grad_w0, grad_w1]) in bf16."""
+    gemms = Fp8BlockwiseGemms(128)
+    quantized = []
+    for w in weights:
+        q, s = _quantize_dense_weight_to_blockwise_fp8(w, 128, torch.float8_e4m3fn)
+        quantized.append(BlockwiseFp8Weight(q, s, 128))
+    hidden = gemms.forward(x, quantized[0])
+    out = gemms.forward(hidden, quantized[1])
+    grad_hidden, grad_w1 = gemms.backward(grad_out, hidden, quantized[1], True, True)
+    grad_x, grad_w0 = gemms.backward(grad_hidden, x, quantized[0], True, True)
+    return out, grad_x, [grad_w0, grad_w1]
+
+
+def test_one_rank_bucket_under_hooks(device):
+    gen = torch.Generator().manual_seed(0)
+    model = _mlp(device, gen)
+    full = [p.detach().clone() for p in model.parameters()]
+    convert_to_flex_shard_float8_blockwise_linear(model)
+    group = LocalReduceGroup(1, 0)
+    mesh = FakeMesh(1, 0, group)
+    placement = Fp8BucketedBlockShard(world_size=1, weight_factory=make_blockwise_fp8_weight)
+    context = BucketCommContext.create(device)
+    runtime = BucketRuntime.shard_module_params(model, ["0.weight", "1.weight"], placement, mesh, context)
+    runtime.install_hooks(model)
+    assert all(torch.equal(s.view(w.shape), w) for s, w in zip(runtime.sharded_params, full))
+
+    x = torch.randn(96, 256, generator=gen).bfloat16().to(device).requires_grad_()
+    grad_out = (torch.randn(96, 256, generator=gen) * 0.01).bfloat16().to(device)
+    for step in range(3):
+        if step:  # an "optimizer step" on the local shards: the next unshard must refill from them
+            with torch.no_grad():
+                for p in runtime.sharded_params:
+                    p.mul_(0.5)
+                    p.grad = None
+                x.grad = None
+        out = model(x)
+        # between forward and backward the modules hold the shards and the full weights' storage is freed
+        assert model[0]._parameters["weight"] is runtime.sharded_params[0]
+        assert all(b.untyped_storage().size() == 0 for b in runtime.persistent_buffers)
+        buffers, unsharded = list(runtime.persistent_buffers), list(runtime.unsharded_params)
+        out.backward(grad_out)
+        context.wait_and_clear_reduce_grad_states()
+        assert not context.reduce_grad_states and not runtime.is_unsharded
+        assert all(a is b for a, b in zip(buffers, runtime.persistent_buffers))
+        assert all(a is b for a, b in zip(unsharded, runtime.unsharded_params))
+        weights = [w * (0.5**step) for w in full]
+        want_out, want_gx, want_gw = _direct(weights, x.detach(), grad_out)
+        assert torch.equal(out.detach(), want_out)
+        assert torch.equal(x.grad, want_gx)
+        for p, g in zip(runtime.sharded_params, want_gw):
+            # reduced in fp32, stored in the sharded parameter's own dtype
+            assert p.grad.dtype == torch.bfloat16 and torch.equal(p.grad.view(g.shape), g)
+    torch.cuda.synchronize()
+
+
+def test_rank_zero_of_two_driven_by_hand(device):
+    """Rank 0 of a 2-rank mesh: the other rank's all-gather row and its
+    reduce-scatter contribution are deposited in the one-GPU group; the unshard
+    runs on the side stream, the reduction on the reduce stream."""
+    gen = torch.Generator().manual_seed(1)
+    model = _mlp(device, gen)
+    full = [p.detach().clone() for p in model.parameters()]
+    named = [("0.weight", nn.Parameter(full[0])), ("1.weight", nn.Parameter(full[1]))]
+    convert_to_flex_shard_float8_blockwise_linear(model)
+    placement = Fp8BucketedBlockShard(world_size=2, weight_factory=make_blockwise_fp8_weight)
+    group = LocalReduceGroup(2, 0)
+    mesh0, mesh1 = FakeMesh(2, 0, group), FakeMesh(2, 1, None)
+    # what rank 1 would send: its quantized, packed payload
+    infos1 = make_param_infos(named, placement, mesh1)
+    for info in infos1:
+        info.reduce_dtype = torch.float32  # the runtime's default mixed-precision policy
+    prepared1 = placement.prepare_unshard_bucket([local_rows(p, i) for (_, p), i in zip(named, infos1)], infos1, mesh1, None)
+    group.gather_rows[1] = prepared1.buffers[0]
+
+    context = BucketCommContext.create(device)
+    runtime = BucketRuntime.shard_module_params(
+        model, ["0.weight", "1.weight"], placement, mesh0, context, GradientReduction()
+    )
+    assert sum(p.numel() for p in runtime.sharded_params) < sum(w.numel() for w in full)
+    handle = runtime.begin_unshard()
+    runtime.finish_unshard(handle)
+    with pytest.raises(RuntimeError, match="only be finished once"):
+        handle.finish()
+    runtime._swap_in_params(runtime.unsharded_params)
+    x = torch.randn(64, 256, generator=gen).bfloat16().to(device)
+    grad_out = (torch.randn(64, 256, generator=gen) * 0.01).bfloat16().to(device)
+    out = model(x)
+    want_out, _, want_gw = _direct(full, x, grad_out)
+    assert torch.equal(out.detach(), want_out)
+    out.backward(grad_out)
+    grads0 = [p.grad for p in runtime.unsharded_params]
+    assert all(g.dtype == torch.float32 for g in grads0)
+    assert all(torch.equal(g, w.float()) for g, w in zip(grads0, want_gw))
+    # rank 1's contribution: other gradients, laid out as its reduce-scatter input
+    grads1 = [torch.randn(g.shape, generator=gen).to(device) for g in grads0]
+    send1 = placement.prepare_reduce_grad(grads1, infos1, mesh1, None).buffers[0]
+    group.deposit(1, send1)
+    runtime.reduce_grads()
+    runtime.reshard()
+    context.wait_and_clear_reduce_grad_states()
+    for param, info, g0, g1 in zip(runtime.sharded_params, runtime.infos, grads0, grads1):
+        # pre-multiplied sum in rank order in fp32, stored in the sharded parameter's dtype
+        want = local_rows(nn.Parameter((g0 * 0.5 + g1 * 0.5).bfloat16()), info)
+        assert param.grad.shape == info.local_shape and torch.equal(param.grad, want)
+    torch.cuda.synchronize()
+
+
+def test_unshard_buffers_are_released_through_both_streams(device):
+    gen = torch.Generator().manual_seed(2)
+    weight = nn.Parameter((torch.randn(256, 256, generator=gen) * 0.05).bfloat16().to(device))
+    placement = Fp8BucketedBlockShard(world_size=1, weight_factory=make_blockwise_fp8_weight)
+    mesh = FakeMesh(1, 0, LocalReduceGroup(1, 0))
+    infos = make_param_infos([("w", weight)], placement, mesh)
+    side = torch.cuda.Stream(device)
+    handle = begin_bucket_unshard([weight.detach()], infos, mesh, side)
+    assert handle.prepared.buffers  # payload and gathered rows, allocated on the side stream
+    handle.release_buffers()
+    assert not handle.prepared.buffers
+    handle = begin_bucket_unshard([weight.detach()], infos, mesh, side)
+    result = handle.finish()
+    assert not handle.prepared.buffers and not result.buffers and len(result.persistent_buffers) == 1
+    q, s = _quantize_dense_weight_to_blockwise_fp8(weight.detach(), 128, torch.float8_e4m3fn)
+    got = result.full_params[0]
+    assert torch.equal(got.fp8_data.view(torch.uint8), q.view(torch.uint8)) and torch.equal(got.recip_scale, s)
+    kept = [torch.ones(4, device=device)]
+    handoff = StreamHandoff(kept, (side, torch.cuda.current_stream(device)))
+    handoff.release_after_current_stream()
+    handoff.release_after_current_stream()  # idempotent
+    assert not kept
+    torch.cuda.synchronize()
