@@ -98,23 +98,27 @@ __global__ __launch_bounds__(kActThreads) void act_quant_1x128_kernel(const ActQ
 }
 
 // ----------------------------------------------------------------- FP8 GEMM
-// 128 x 256 output tile per workgroup, four waves of 64 x 128 (two by four
-// 32x32 blocks).  Operand tiles are 128 bytes per row and k-tile and travel
-// global -> LDS directly, 16-byte chunk c of row r in slot c ^ (r & 7), into
-// one of three stages.  A lane feeds the matrix core bytes [32 h, 32 h + 32) of each half
-// of its row (h = lane / 32), i.e. chunks 2h and 2h+1 of a 64-byte half.
+// 256 x 256 output tile per workgroup, four waves of 128 x 128 (four by four
+// 32x32 blocks): 262 flop per operand byte, which is what keeps the request
+// rate to L2 within reach at FP8 speed (a 128 x 256 tile needs 50 % more
+// operand bytes per flop).  Operand tiles are 128 bytes per row and k-tile and
+// travel global -> LDS directly, 16-byte chunk c of row r in slot c ^ ((r >> 1) & 7),
+// into one of two 64 KB stages.  A lane feeds the matrix core bytes
+// [32 h, 32 h + 32) of each half of its row (h = lane / 32), i.e. chunks 2h
+// and 2h+1 of a 64-byte half.
 struct Fp8Gemm {
-  static constexpr int BM = 128, BN = 256, BK = 128, WM = 2, WN = 2, TM = 2, TN = 4;
-  static constexpr int kThreads = 256, kWaveM = 64, kWaveN = 128;
+  static constexpr int BM = 256, BN = 256, BK = 128, WM = 2, WN = 2, TM = 4, TN = 4;
+  static constexpr int kThreads = 256, kWaveM = 128, kWaveN = 128;
   static constexpr int kRowBytes = 128;
-  static constexpr int kABytes = BM * kRowBytes;               // 16 KB
-  static constexpr int kStageBytes = (BM + BN) * kRowBytes;    // 48 KB
-  static constexpr int kLoadsA = BM / 8 / 4, kLoadsB = BN / 8 / 4;  // per wave: 4 and 8
+  static constexpr int kABytes = BM * kRowBytes;               // 32 KB
+  static constexpr int kStageBytes = (BM + BN) * kRowBytes;    // 64 KB
+  static constexpr int kLoadsA = BM / 8 / 4, kLoadsB = BN / 8 / 4;  // per wave: 8 and 8
   static constexpr int kPitch = kWaveN * 2 + 8;                // epilogue staging, bytes
   static constexpr int kRegion = kWaveM * kPitch;              // per wave
-  static constexpr int kStages = 3;
-  static constexpr int kScaleOffset = kStages * kStageBytes;   // [stage][wave][64] activation scales
-  static constexpr int kWeightScaleOffset = kScaleOffset + kStages * 1024;  // [wave][256] weight scales
+  static constexpr int kStages = 2;
+  static constexpr int kScaleStageBytes = 4 * kWaveM * 4;      // per stage: [wave][128] row scales
+  static constexpr int kScaleOffset = kStages * kStageBytes;
+  static constexpr int kWeightScaleOffset = kScaleOffset + kStages * kScaleStageBytes;  // [wave][256] block scales
   static constexpr int kMaxKTilesInLds = 256;
   static constexpr int kLdsBytes = max_int(kWeightScaleOffset + 4 * kMaxKTilesInLds * 4, 4 * kRegion);
 };
@@ -139,7 +143,7 @@ typedef int v8i32 __attribute__((ext_vector_type(8)));
 template <bool kColumnScales>
 __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(const Fp8GemmParams p) {
   using Cfg = Fp8Gemm;
-  constexpr int kLoadsPerKTile = Cfg::kLoadsA + Cfg::kLoadsB + (kColumnScales ? 2 : 1);
+  static_assert(Cfg::kStages == 2, "the loop below alternates between two stages");
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds_bytes[];
   constexpr int TM = Cfg::TM, TN = Cfg::TN;
   const int tid = threadIdx.x;
@@ -158,7 +162,7 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
   // lane l fills slot l & 7 of row l >> 3 there.  Rows past the matrix are
   // read from its last row (their products are never stored).
   const int fill_row = lane >> 3;
-  const int fill_chunk = (lane & 7) ^ fill_row;
+  const int fill_chunk = (lane & 7) ^ (((8 * wave + fill_row) >> 1) & 7);
   uint32_t a_voff[Cfg::kLoadsA], b_voff[Cfg::kLoadsB];
 #pragma unroll
   for (int q = 0; q < Cfg::kLoadsA; ++q) {
@@ -188,14 +192,14 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
   };
 
   // Fragment side: row = lane & 31 of a 32-row block; chunks 4 kh + 2 h and
-  // 4 kh + 2 h + 1 of the row (kh = 64-byte half), each in slot chunk ^ (row & 7).
+  // 4 kh + 2 h + 1 of the row (kh = 64-byte half), each in slot chunk ^ ((row >> 1) & 7).
   const int frag_row = lane & 31, h = lane >> 5;
   uint32_t frag_off[2][2];
 #pragma unroll
   for (int kh = 0; kh < 2; ++kh)
 #pragma unroll
     for (int c = 0; c < 2; ++c)
-      frag_off[kh][c] = static_cast<uint32_t>(frag_row * Cfg::kRowBytes + (((4 * kh + 2 * h + c) ^ (frag_row & 7)) * 16));
+      frag_off[kh][c] = static_cast<uint32_t>(frag_row * Cfg::kRowBytes + (((4 * kh + 2 * h + c) ^ ((frag_row >> 1) & 7)) * 16));
   auto read_frag = [&](int stage_off, int operand_off, int block, int kh) -> v8i32 {
     const uint8_t* base = lds_bytes + stage_off + operand_off + block * 32 * Cfg::kRowBytes;
     const u32x4 lo = *reinterpret_cast<const u32x4*>(base + frag_off[kh][0]);
@@ -218,75 +222,70 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  // Three stages: the operands of k-tiles kt + 1 and kt + 2 are in flight
-  // while kt is multiplied (a k-tile is under a microsecond of MFMA work, a
-  // miss to HBM takes two).  The activation scales ride the same global->LDS
-  // path (one 4-byte-per-lane request per wave and k-tile for the wave's 64
-  // rows): a compiler-visible load here would make the compiler wait for
-  // everything in flight, the prefetched tiles included.  Requests complete
-  // in order, so "at most 13 outstanding" means all but the youngest tile's.
-  const uint32_t scale_lds0 = lds_base + static_cast<uint32_t>(Cfg::kScaleOffset + wave * 256);
-  const int64_t scale_row0 = m0 + wm * Cfg::kWaveM + lane;
-  const uint32_t scale_voff = static_cast<uint32_t>((scale_row0 < p.m ? scale_row0 : p.m - 1) * 4);
+  // Two stages: the operands of k-tile kt + 1 are in flight while kt is
+  // multiplied.  The row scales ride the same global->LDS path (two 4-byte-
+  // per-lane requests per wave and k-tile for the wave's 128 rows): a
+  // compiler-visible load here would make the compiler wait for everything in
+  // flight, the prefetched tile included.
+  const uint32_t scale_lds0 = lds_base + static_cast<uint32_t>(Cfg::kScaleOffset + wave * Cfg::kWaveM * 4);
+  uint32_t scale_voff[2];
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    const int64_t row = m0 + wm * Cfg::kWaveM + half * 64 + lane;
+    scale_voff[half] = static_cast<uint32_t>((row < p.m ? row : p.m - 1) * 4);
+  }
   // Per-column scales of the workgroup's 256 columns take the same road, 64
-  // columns per wave, into [stage][256] floats of the weight-scale area.
+  // columns per wave, into [stage][256] floats of the block-scale area.
   const uint32_t cscale_lds0 = lds_base + static_cast<uint32_t>(Cfg::kWeightScaleOffset + wave * 256);
   const int64_t cscale_col0 = n0 + wave * 64 + lane;
   const uint32_t cscale_voff = static_cast<uint32_t>((cscale_col0 < p.n ? cscale_col0 : p.n - 1) * 4);
   auto issue_k_tile = [&](int64_t kt, int stage) {
     issue_tile_load(kt, stage * Cfg::kStageBytes);
-    dma_touch_4(scale_voff, reinterpret_cast<const uint8_t*>(p.xs + kt * p.m), scale_lds0 + stage * 1024);
+    const uint8_t* xs_row = reinterpret_cast<const uint8_t*>(p.xs + kt * p.m);
+    dma_touch_4(scale_voff[0], xs_row, scale_lds0 + stage * Cfg::kScaleStageBytes);
+    dma_touch_4(scale_voff[1], xs_row, scale_lds0 + stage * Cfg::kScaleStageBytes + 256);
     if (kColumnScales)
       dma_touch_4(cscale_voff, reinterpret_cast<const uint8_t*>(p.cs + kt * p.n), cscale_lds0 + stage * 1024);
   };
   // The block scales of the wave's 128 columns, one per k-tile, are copied
   // to LDS once (a load from global memory inside the loop would again wait
-  // for the prefetched tiles).
+  // for the prefetched tile).
   float* ws_lds = reinterpret_cast<float*>(lds_bytes + Cfg::kWeightScaleOffset + wave * Cfg::kMaxKTilesInLds * 4);
   if (!kColumnScales) {
     const float* ws_row = p.ws + wblock * p.ws_cb;
     for (int64_t i = lane; i < ktiles; i += 64) ws_lds[i] = ws_row[i * p.ws_kb];  // ktiles <= kMaxKTilesInLds (host check)
   }
   issue_k_tile(0, 0);
-  if (ktiles > 1) {
-    issue_k_tile(1, 1);
-    wait_for_dma_loads_except<kLoadsPerKTile>();
-  } else {
-    wait_for_dma_loads();
-  }
+  wait_for_dma_loads();
   __syncthreads();
 
   int stage = 0;
   for (int64_t kt = 0; kt < ktiles; ++kt) {
     const int stage_off = stage * Cfg::kStageBytes;
-    const int stage2 = stage >= 1 ? stage - 1 : Cfg::kStages - 1;  // (stage + 2) % 3
-    if (kt + 2 < ktiles) issue_k_tile(kt + 2, stage2);  // its stage was released by the barrier that ended kt - 1
+    if (kt + 1 < ktiles) issue_k_tile(kt + 1, stage ^ 1);  // its stage was released by the barrier that ended kt - 1
     float s[TM];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
-      s[i] = *reinterpret_cast<const float*>(lds_bytes + Cfg::kScaleOffset + stage * 1024 + wave * 256 +
-                                             (i * 32 + frag_row) * 4);
+      s[i] = *reinterpret_cast<const float*>(lds_bytes + Cfg::kScaleOffset + stage * Cfg::kScaleStageBytes +
+                                             (wave * Cfg::kWaveM + i * 32 + frag_row) * 4);
     if (!kColumnScales) {
       const float ws_now = ws_lds[kt];
 #pragma unroll
       for (int i = 0; i < TM; ++i) s[i] *= ws_now;
     }
-    v8i32 bfrag[TN][2], afrag[TM][2];
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int kh = 0; kh < 2; ++kh) bfrag[j][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32) + j, kh);
+    // The A fragments of the wave's four row blocks stay in registers for the
+    // whole k-tile; the B fragments are read one column block ahead.
+    v8i32 afrag[TM][2], bfrag[2][2];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int kh = 0; kh < 2; ++kh) afrag[i][kh] = read_frag(stage_off, 0, wm * (Cfg::kWaveM / 32) + i, kh);
-    // The eight 32x32 blocks in turn: two MFMAs give a block's partial product
-    // for this scale block; it is folded into the result (16 fused multiply-
-    // adds) while the next block's MFMAs run.  With per-column scales the
-    // blocks go column block by column block, so that the sixteen column
-    // scales a lane needs are read from LDS once for both row blocks.
-    auto block_i = [&](int blk) { return kColumnScales ? blk % TM : blk / TN; };
-    auto block_j = [&](int blk) { return kColumnScales ? blk / TM : blk % TN; };
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh) bfrag[0][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32), kh);
+    // The sixteen 32x32 blocks, column block by column block: two MFMAs give
+    // a block's partial product for this scale block; it is folded into the
+    // result (16 fused multiply-adds, or multiply + fused multiply-add with
+    // per-column scales) while the next block's MFMAs run.
     const uint8_t* cscale_lds = lds_bytes + Cfg::kWeightScaleOffset + stage * 1024 + (wn * Cfg::kWaveN + 4 * h) * 4;
     f32x16 part_prev;
     f32x4 cscale[4];
@@ -302,17 +301,22 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
     };
 #pragma unroll
     for (int blk = 0; blk < TM * TN; ++blk) {
-      const int i = block_i(blk), j = block_j(blk);
+      const int i = blk % TM, j = blk / TM;
       const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      if (kColumnScales && blk > 0 && block_i(blk - 1) == 0) {
+      if (i == 0 && j + 1 < TN) {  // next column block's B fragments
+#pragma unroll
+        for (int kh = 0; kh < 2; ++kh)
+          bfrag[(j + 1) & 1][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32) + j + 1, kh);
+      }
+      if (kColumnScales && blk > 0 && (blk - 1) % TM == 0) {
 #pragma unroll
         for (int b = 0; b < 4; ++b)
-          cscale[b] = *reinterpret_cast<const f32x4*>(cscale_lds + (block_j(blk - 1) * 32 + 8 * b) * 4);
+          cscale[b] = *reinterpret_cast<const f32x4*>(cscale_lds + (((blk - 1) / TM) * 32 + 8 * b) * 4);
       }
-      f32x16 part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j][0], afrag[i][0], zero, 0, 0, 0, 0, 0, 0);
-      part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j][1], afrag[i][1], part, 0, 0, 0, 0, 0, 0);
+      f32x16 part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j & 1][0], afrag[i][0], zero, 0, 0, 0, 0, 0, 0);
+      part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j & 1][1], afrag[i][1], part, 0, 0, 0, 0, 0, 0);
       if (blk > 0) {
-        const int pi = block_i(blk - 1), pj = block_j(blk - 1);
+        const int pi = (blk - 1) % TM, pj = (blk - 1) / TM;
         fold(pi, pj);
         // An empty statement that "uses" the folded block keeps the folds on
         // this side of the scheduling barrier (plain arithmetic may otherwise
@@ -323,12 +327,9 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
       __builtin_amdgcn_sched_barrier(0);  // MFMA pair, then the previous block's folds, in that order
     }
     fold(TM - 1, TN - 1);
-    if (kt + 1 < ktiles) {  // k-tile kt + 1 has landed; kt + 2 may still be on its way
-      if (kt + 2 < ktiles) wait_for_dma_loads_except<kLoadsPerKTile>();
-      else wait_for_dma_loads();
-    }
+    if (kt + 1 < ktiles) wait_for_dma_loads();  // k-tile kt + 1 has landed
     __syncthreads();
-    stage = stage + 1 == Cfg::kStages ? 0 : stage + 1;
+    stage ^= 1;
   }
 
   // Epilogue: bf16 finals to the wave's staging region as [row][col], then

@@ -351,10 +351,14 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_nt_interior_kernel(const G
 // no ds_write, and the loads of tile t+1 are waited for only at the end of
 // tile t.  A wave-level load fills 1 KB of LDS = 8 tile rows of 128 bytes
 // with no padding, so bank conflicts are avoided by an XOR swizzle instead:
-// the 16-byte chunk c of row r is stored in slot c ^ (r & 7) of its row, done
-// on the global side by letting the lane that fills slot s of row r fetch
-// chunk s ^ (r & 7).  Eight neighbouring lanes of a fragment read then hit
-// eight different slots.
+// the 16-byte chunk c of row r is stored in slot c ^ ((r >> 1) & 7) of its
+// row, done on the global side by letting the lane that fills slot s of row r
+// fetch chunk s ^ ((r >> 1) & 7).  The LDS has 64 banks of 4 bytes and serves
+// a 16-byte-per-lane read sixteen lanes at a time; rows are 128 bytes, so the
+// sixteen rows of such a group alternate between the two halves of the bank
+// window and, within a half, take eight different slots.  (XOR with r & 7
+// spreads only eight lanes and costs a two-way conflict on every fragment
+// read: 8 instead of 4 cycles by the bank-conflict counter.)
 //
 // These loads and their waits are inline asm, which the compiler neither
 // reorders nor counts; everything else in the loop is compiler-visible and is
@@ -423,7 +427,7 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   // Load side.  Wave-level load q (0..7) of this wave fills tile rows
   // [32 q + 8 wave, +8); lane l fills slot l & 7 of row l >> 3 there.
   const int fill_row = lane >> 3;
-  const int fill_chunk = (lane & 7) ^ fill_row;
+  const int fill_chunk = (lane & 7) ^ (((8 * wave + fill_row) >> 1) & 7);
   // M0 takes the LDS byte address relative to the workgroup's allocation.
   typedef __attribute__((address_space(3))) uint8_t* lds_address;
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_address)lds_bytes));
@@ -449,10 +453,11 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   };
 
   // Fragment side.  Lane l reads row l & 31 of a 32-row block, k chunk
-  // 2 ks + (l >> 5); its slot is that chunk XOR (row & 7), i.e. the ks = 0
-  // address with bits 5..6 flipped by ks.
+  // 2 ks + (l >> 5); its slot is that chunk XOR ((row >> 1) & 7), i.e. the
+  // ks = 0 address with bits 5..6 flipped by ks.
   const int frag_row = lane & 31;
-  const uint32_t frag_base = static_cast<uint32_t>(frag_row * Cfg::kRowBytes + (((lane >> 5) ^ (frag_row & 7)) * 16));
+  const uint32_t frag_base =
+      static_cast<uint32_t>(frag_row * Cfg::kRowBytes + (((lane >> 5) ^ ((frag_row >> 1) & 7)) * 16));
   uint32_t a_frag[KS], b_frag[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
