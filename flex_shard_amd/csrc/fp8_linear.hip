@@ -273,60 +273,69 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
 #pragma unroll
       for (int i = 0; i < TM; ++i) s[i] *= ws_now;
     }
-    // The A fragments of the wave's four row blocks stay in registers for the
-    // whole k-tile; the B fragments are read one column block ahead.
+    // Fragments are read in the order the blocks need them: the first column
+    // block's B and the first row block's A before the first MFMA, the other
+    // A row blocks under the MFMAs of the first column block (they stay for
+    // the whole k-tile), each further B column block while the previous one is
+    // multiplied.
     v8i32 afrag[TM][2], bfrag[2][2];
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int kh = 0; kh < 2; ++kh) afrag[i][kh] = read_frag(stage_off, 0, wm * (Cfg::kWaveM / 32) + i, kh);
-#pragma unroll
     for (int kh = 0; kh < 2; ++kh) bfrag[0][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32), kh);
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh) afrag[0][kh] = read_frag(stage_off, 0, wm * (Cfg::kWaveM / 32), kh);
     // The sixteen 32x32 blocks, column block by column block: two MFMAs give
     // a block's partial product for this scale block; it is folded into the
     // result (16 fused multiply-adds, or multiply + fused multiply-add with
-    // per-column scales) while the next block's MFMAs run.
+    // per-column scales) while the next block's MFMAs run.  A wave issues in
+    // order and an MFMA keeps the matrix core busy for 64 cycles = 16 vector
+    // instructions, so half of a fold goes behind each of the two MFMAs; all
+    // of it behind the second one would hold up the next block's first MFMA.
     const uint8_t* cscale_lds = lds_bytes + Cfg::kWeightScaleOffset + stage * 1024 + (wn * Cfg::kWaveN + 4 * h) * 4;
     f32x16 part_prev;
     f32x4 cscale[4];
-    auto fold = [&](int pi, int pj) {
-      if (kColumnScales) {
+    auto fold_half = [&](int pi, int pj, int half) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
+      for (int r = 8 * half; r < 8 * half + 8; ++r) {
+        if (kColumnScales)
           acc[pi][pj][r] = __builtin_fmaf(part_prev[r] * s[pi], cscale[r / 4][r % 4], acc[pi][pj][r]);
-      } else {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[pi][pj][r] = __builtin_fmaf(part_prev[r], s[pi], acc[pi][pj][r]);
+        else
+          acc[pi][pj][r] = __builtin_fmaf(part_prev[r], s[pi], acc[pi][pj][r]);
       }
     };
 #pragma unroll
     for (int blk = 0; blk < TM * TN; ++blk) {
       const int i = blk % TM, j = blk / TM;
+      const int pi = (blk + TM * TN - 1) % TM, pj = (blk + TM * TN - 1) % (TM * TN) / TM;  // previous block
       const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      if (i == 0 && j + 1 < TN) {  // next column block's B fragments
+      if (j == 0 && i + 1 < TM) {  // next row block's A fragments
+#pragma unroll
+        for (int kh = 0; kh < 2; ++kh) afrag[i + 1][kh] = read_frag(stage_off, 0, wm * (Cfg::kWaveM / 32) + i + 1, kh);
+      }
+      if (i == 1 && j + 1 < TN) {  // next column block's B fragments
 #pragma unroll
         for (int kh = 0; kh < 2; ++kh)
           bfrag[(j + 1) & 1][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32) + j + 1, kh);
       }
-      if (kColumnScales && blk > 0 && (blk - 1) % TM == 0) {
+      if (kColumnScales && blk > 0 && pi == 0) {
 #pragma unroll
-        for (int b = 0; b < 4; ++b)
-          cscale[b] = *reinterpret_cast<const f32x4*>(cscale_lds + (((blk - 1) / TM) * 32 + 8 * b) * 4);
+        for (int b = 0; b < 4; ++b) cscale[b] = *reinterpret_cast<const f32x4*>(cscale_lds + (pj * 32 + 8 * b) * 4);
       }
       f32x16 part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j & 1][0], afrag[i][0], zero, 0, 0, 0, 0, 0, 0);
+      if (blk > 0) fold_half(pi, pj, 0);
+      // The scheduling barriers fix this order; an empty statement that
+      // "uses" the folded block (below) keeps its arithmetic between them
+      // (plain arithmetic may otherwise be moved past a barrier).
+      __builtin_amdgcn_sched_barrier(0);
       part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j & 1][1], afrag[i][1], part, 0, 0, 0, 0, 0, 0);
       if (blk > 0) {
-        const int pi = (blk - 1) % TM, pj = (blk - 1) / TM;
-        fold(pi, pj);
-        // An empty statement that "uses" the folded block keeps the folds on
-        // this side of the scheduling barrier (plain arithmetic may otherwise
-        // be moved past it and end up after the last MFMA).
+        fold_half(pi, pj, 1);
         asm volatile("" : "+v"(acc[pi][pj]));
       }
       part_prev = part;
-      __builtin_amdgcn_sched_barrier(0);  // MFMA pair, then the previous block's folds, in that order
+      __builtin_amdgcn_sched_barrier(0);
     }
-    fold(TM - 1, TN - 1);
+    fold_half(TM - 1, TN - 1, 0);
+    fold_half(TM - 1, TN - 1, 1);
     if (kt + 1 < ktiles) wait_for_dma_loads();  // k-tile kt + 1 has landed
     __syncthreads();
     stage ^= 1;
