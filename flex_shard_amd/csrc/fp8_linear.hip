@@ -259,6 +259,16 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
   wait_for_dma_loads();
   __syncthreads();
 
+#ifdef FSH_TRACE
+  // Time per phase of the k loop, summed over the k-tiles (10 ns ticks).
+  uint64_t t_compute = 0, t_wait = 0, t_barrier = 0, t_mark = __builtin_amdgcn_s_memrealtime();
+  const uint64_t t_begin = t_mark;
+  auto lap = [&](uint64_t& sum) {
+    const uint64_t now = __builtin_amdgcn_s_memrealtime();
+    sum += now - t_mark;
+    t_mark = now;
+  };
+#endif
   int stage = 0;
   for (int64_t kt = 0; kt < ktiles; ++kt) {
     const int stage_off = stage * Cfg::kStageBytes;
@@ -283,29 +293,37 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
     for (int kh = 0; kh < 2; ++kh) bfrag[0][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32), kh);
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh) afrag[0][kh] = read_frag(stage_off, 0, wm * (Cfg::kWaveM / 32), kh);
-    // The sixteen 32x32 blocks, column block by column block: two MFMAs give
-    // a block's partial product for this scale block; it is folded into the
-    // result (16 fused multiply-adds, or multiply + fused multiply-add with
-    // per-column scales) while the next block's MFMAs run.  A wave issues in
-    // order and an MFMA keeps the matrix core busy for 64 cycles = 16 vector
-    // instructions, so half of a fold goes behind each of the two MFMAs; all
-    // of it behind the second one would hold up the next block's first MFMA.
+    // The sixteen 32x32 blocks, column block by column block: two MFMAs, back
+    // to back, give a block's partial product for this scale block.  It is
+    // folded into the result (16 fused multiply-adds, or multiply + fused
+    // multiply-add with per-column scales) two blocks later, behind that
+    // block's MFMAs: a fold that reads the product of the MFMA issued just
+    // before it waits for the matrix core to drain (measured: 122 against 100
+    // time units per block for the arrangement used here).
     const uint8_t* cscale_lds = lds_bytes + Cfg::kWeightScaleOffset + stage * 1024 + (wn * Cfg::kWaveN + 4 * h) * 4;
-    f32x16 part_prev;
+    constexpr int kBlocks = TM * TN;
+    f32x16 part[3];
     f32x4 cscale[4];
-    auto fold_half = [&](int pi, int pj, int half) {
+    auto fold = [&](int blk, const f32x16& product) {
+      const int pi = blk % TM, pj = blk / TM;
+      if (kColumnScales && pi == 0) {
 #pragma unroll
-      for (int r = 8 * half; r < 8 * half + 8; ++r) {
-        if (kColumnScales)
-          acc[pi][pj][r] = __builtin_fmaf(part_prev[r] * s[pi], cscale[r / 4][r % 4], acc[pi][pj][r]);
-        else
-          acc[pi][pj][r] = __builtin_fmaf(part_prev[r], s[pi], acc[pi][pj][r]);
+        for (int b = 0; b < 4; ++b) cscale[b] = *reinterpret_cast<const f32x4*>(cscale_lds + (pj * 32 + 8 * b) * 4);
       }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        if (kColumnScales)
+          acc[pi][pj][r] = __builtin_fmaf(product[r] * s[pi], cscale[r / 4][r % 4], acc[pi][pj][r]);
+        else
+          acc[pi][pj][r] = __builtin_fmaf(product[r], s[pi], acc[pi][pj][r]);
+      }
+      // An empty statement that "uses" the folded block keeps its arithmetic
+      // on this side of the next scheduling barrier.
+      asm volatile("" : "+v"(acc[pi][pj]));
     };
 #pragma unroll
-    for (int blk = 0; blk < TM * TN; ++blk) {
+    for (int blk = 0; blk < kBlocks; ++blk) {
       const int i = blk % TM, j = blk / TM;
-      const int pi = (blk + TM * TN - 1) % TM, pj = (blk + TM * TN - 1) % (TM * TN) / TM;  // previous block
       const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       if (j == 0 && i + 1 < TM) {  // next row block's A fragments
 #pragma unroll
@@ -316,30 +334,35 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
         for (int kh = 0; kh < 2; ++kh)
           bfrag[(j + 1) & 1][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32) + j + 1, kh);
       }
-      if (kColumnScales && blk > 0 && pi == 0) {
-#pragma unroll
-        for (int b = 0; b < 4; ++b) cscale[b] = *reinterpret_cast<const f32x4*>(cscale_lds + (pj * 32 + 8 * b) * 4);
-      }
-      f32x16 part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j & 1][0], afrag[i][0], zero, 0, 0, 0, 0, 0, 0);
-      if (blk > 0) fold_half(pi, pj, 0);
-      // The scheduling barriers fix this order; an empty statement that
-      // "uses" the folded block (below) keeps its arithmetic between them
-      // (plain arithmetic may otherwise be moved past a barrier).
+      f32x16 product = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j & 1][0], afrag[i][0], zero, 0, 0, 0, 0, 0, 0);
+      product = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j & 1][1], afrag[i][1], product, 0, 0, 0, 0, 0, 0);
+      part[blk % 3] = product;
       __builtin_amdgcn_sched_barrier(0);
-      part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j & 1][1], afrag[i][1], part, 0, 0, 0, 0, 0, 0);
-      if (blk > 0) {
-        fold_half(pi, pj, 1);
-        asm volatile("" : "+v"(acc[pi][pj]));
-      }
-      part_prev = part;
+      if (blk >= 2) fold(blk - 2, part[(blk - 2) % 3]);
       __builtin_amdgcn_sched_barrier(0);
     }
-    fold_half(TM - 1, TN - 1, 0);
-    fold_half(TM - 1, TN - 1, 1);
+    fold(kBlocks - 2, part[(kBlocks - 2) % 3]);
+    fold(kBlocks - 1, part[(kBlocks - 1) % 3]);
+#ifdef FSH_TRACE
+    asm volatile("" : "+v"(acc[TM - 1][TN - 1]));
+    lap(t_compute);
+#endif
     if (kt + 1 < ktiles) wait_for_dma_loads();  // k-tile kt + 1 has landed
+#ifdef FSH_TRACE
+    lap(t_wait);
+#endif
     __syncthreads();
+#ifdef FSH_TRACE
+    lap(t_barrier);
+#endif
     stage ^= 1;
   }
+#ifdef FSH_TRACE
+  if (p.schedule.trace && lane == 0) {
+    uint64_t* out = p.schedule.trace + (static_cast<int64_t>(blockIdx.x) * 4 + wave) * 8;
+    out[0] = t_begin; out[1] = t_compute; out[2] = t_wait; out[3] = t_barrier; out[4] = t_mark;
+  }
+#endif
 
   // Epilogue: bf16 finals to the wave's staging region as [row][col], then
   // 16-byte row stores, rows and 8-column groups past the matrix skipped.
@@ -442,6 +465,9 @@ int launch_fp8_gemm(Fp8GemmParams& p, bool column_scales, const char* who, void*
     return fail(FSH_ENOTSUP, "%s: a tile spans more than 2 GiB", who);
   GemmParams& s = p.schedule;
   memset(&s, 0, sizeof(s));
+#ifdef FSH_TRACE
+  if (const char* e = getenv("FSH_GEMM_TRACE")) s.trace = reinterpret_cast<uint64_t*>(strtoull(e, nullptr, 0));
+#endif
   s.tiles_m = static_cast<int32_t>(ceil_div(p.m, (int64_t)Fp8Gemm::BM));
   s.tiles_n = static_cast<int32_t>(ceil_div(p.n, (int64_t)Fp8Gemm::BN));
   const int64_t tiles = static_cast<int64_t>(s.tiles_m) * s.tiles_n;
