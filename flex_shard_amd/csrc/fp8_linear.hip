@@ -239,14 +239,31 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
   const uint32_t cscale_lds0 = lds_base + static_cast<uint32_t>(Cfg::kWeightScaleOffset + wave * 256);
   const int64_t cscale_col0 = n0 + wave * 64 + lane;
   const uint32_t cscale_voff = static_cast<uint32_t>((cscale_col0 < p.n ? cscale_col0 : p.n - 1) * 4);
-  auto issue_k_tile = [&](int64_t kt, int stage) {
-    issue_tile_load(kt, stage * Cfg::kStageBytes);
+  auto issue_scale_loads = [&](int64_t kt, int stage) {
     const uint8_t* xs_row = reinterpret_cast<const uint8_t*>(p.xs + kt * p.m);
     dma_touch_4(scale_voff[0], xs_row, scale_lds0 + stage * Cfg::kScaleStageBytes);
     dma_touch_4(scale_voff[1], xs_row, scale_lds0 + stage * Cfg::kScaleStageBytes + 256);
     if (kColumnScales)
       dma_touch_4(cscale_voff, reinterpret_cast<const uint8_t*>(p.cs + kt * p.n), cscale_lds0 + stage * 1024);
   };
+  auto issue_k_tile = [&](int64_t kt, int stage) {
+    issue_tile_load(kt, stage * Cfg::kStageBytes);
+    issue_scale_loads(kt, stage);
+  };
+  // One sixteenth of the next k-tile's requests; issued behind each block's
+  // MFMAs.  Sixteen 1 KB requests in a row keep the wave's instruction issue
+  // waiting on the memory pipeline (0.67 us per k-tile by measurement) while
+  // the matrix core runs dry.
+  auto issue_k_tile_part = [&](int64_t kt, int stage, int part) {
+    const int stage_off = stage * Cfg::kStageBytes;
+    const int q = part >> 1;
+    if (part & 1)
+      dma_load_16(b_voff[q], Bb + kt * Cfg::kRowBytes, stage_off + Cfg::kABytes + fill_lds + q * 4096);
+    else
+      dma_load_16(a_voff[q], Ab + kt * Cfg::kRowBytes, stage_off + fill_lds + q * 4096);
+    if (part == 0) issue_scale_loads(kt, stage);
+  };
+  static_assert(Cfg::kLoadsA == 8 && Cfg::kLoadsB == 8 && Cfg::TM * Cfg::TN == 16, "one request per block");
   // The block scales of the wave's 128 columns, one per k-tile, are copied
   // to LDS once (a load from global memory inside the loop would again wait
   // for the prefetched tile).
@@ -272,7 +289,7 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
   int stage = 0;
   for (int64_t kt = 0; kt < ktiles; ++kt) {
     const int stage_off = stage * Cfg::kStageBytes;
-    if (kt + 1 < ktiles) issue_k_tile(kt + 1, stage ^ 1);  // its stage was released by the barrier that ended kt - 1
+    const bool more = kt + 1 < ktiles;  // the next k-tile's stage was released by the barrier that ended kt - 1
     float s[TM];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -302,7 +319,10 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
     // time units per block for the arrangement used here).
     const uint8_t* cscale_lds = lds_bytes + Cfg::kWeightScaleOffset + stage * 1024 + (wn * Cfg::kWaveN + 4 * h) * 4;
     constexpr int kBlocks = TM * TN;
-    f32x16 part[3];
+    // Blocks between a product and its fold; the per-column variant has no
+    // registers left for a third product.
+    constexpr int kLag = kColumnScales ? 1 : 2;
+    f32x16 part[kLag + 1];
     f32x4 cscale[4];
     auto fold = [&](int blk, const f32x16& product) {
       const int pi = blk % TM, pj = blk / TM;
@@ -336,13 +356,14 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
       }
       f32x16 product = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j & 1][0], afrag[i][0], zero, 0, 0, 0, 0, 0, 0);
       product = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j & 1][1], afrag[i][1], product, 0, 0, 0, 0, 0, 0);
-      part[blk % 3] = product;
+      part[blk % (kLag + 1)] = product;
       __builtin_amdgcn_sched_barrier(0);
-      if (blk >= 2) fold(blk - 2, part[(blk - 2) % 3]);
+      if (more) issue_k_tile_part(kt + 1, stage ^ 1, blk);
+      if (blk >= kLag) fold(blk - kLag, part[(blk - kLag) % (kLag + 1)]);
       __builtin_amdgcn_sched_barrier(0);
     }
-    fold(kBlocks - 2, part[(kBlocks - 2) % 3]);
-    fold(kBlocks - 1, part[(kBlocks - 1) % 3]);
+#pragma unroll
+    for (int blk = kBlocks - kLag; blk < kBlocks; ++blk) fold(blk, part[blk % (kLag + 1)]);
 #ifdef FSH_TRACE
     asm volatile("" : "+v"(acc[TM - 1][TN - 1]));
     lap(t_compute);
