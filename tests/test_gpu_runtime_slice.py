@@ -163,3 +163,41 @@ def test_unshard_buffers_are_released_through_both_streams(device):
     handoff.release_after_current_stream()  # idempotent
     assert not kept
     torch.cuda.synchronize()
+
+
+def test_two_dense_buckets_share_the_streams(device):
+    """Two BucketedBlockShard buckets (one per layer) under hooks on one
+    context that allows a single reduction in flight: the second bucket's
+    reduction retires the first.  Forward, input gradient and shard gradients
+    equal the unsharded model's, bit for bit (bf16 weights are gathered as they
+    are, gradients reduced in fp32 over one rank)."""
+    from flex_shard_amd import BucketedBlockShard
+
+    gen = torch.Generator().manual_seed(3)
+    model = _mlp(device, gen)
+    plain = _mlp(device, torch.Generator().manual_seed(3))
+    context = BucketCommContext.create(device, max_pending_reduce_grads=1)
+    mesh = FakeMesh(1, 0, LocalReduceGroup(1, 0))
+    runtimes = []
+    for index, layer in enumerate(model):
+        placement = BucketedBlockShard(dims=(0,), blocks_per_rank=(1,))
+        runtime = BucketRuntime.shard_module_params(model, [f"{index}.weight"], placement, mesh, context)
+        runtime.install_hooks(layer)
+        runtimes.append(runtime)
+    x = torch.randn(32, 256, generator=gen).bfloat16().to(device)
+    grad_out = torch.randn(32, 256, generator=gen).bfloat16().to(device)
+    for step in range(2):
+        x_run, x_ref = x.clone().requires_grad_(), x.clone().requires_grad_()
+        out = model(x_run)
+        assert all(not r.is_unsharded for r in runtimes)
+        out.backward(grad_out)
+        context.wait_and_clear_reduce_grad_states()
+        ref = plain(x_ref)
+        ref.backward(grad_out)
+        assert torch.equal(out.detach(), ref.detach()) and torch.equal(x_run.grad, x_ref.grad)
+        for runtime, layer in zip(runtimes, plain):
+            (shard,) = runtime.sharded_params
+            assert torch.equal(shard.grad.view(layer.weight.shape), layer.weight.grad)
+            shard.grad = None
+            layer.weight.grad = None
+    torch.cuda.synchronize()
