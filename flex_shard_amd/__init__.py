@@ -14,6 +14,8 @@ from .custom_placements import (
     BucketedOwnedSegmentSpec,
     Fp8BucketedBlockShard,
     LocalReduceGroup,
+    MixedBucketPlacement,
+    Shard,
     make_bucketed_block_placement_fn,
     make_bucketed_owned_full_param_placement_fn,
     make_fp8_bucketed_block_placement_fn,
@@ -48,12 +50,14 @@ __all__ = [
     "GradientReduction",
     "LocalReduceGroup",
     "LocalStorageLayout",
+    "MixedBucketPlacement",
     "ParamInfo",
     "Placement",
     "PlacementPreparedReduceGrad",
     "PlacementPreparedUnshard",
     "PlacementReduceGradResult",
     "PlacementUnshardResult",
+    "Shard",
     "compose_global_layouts",
     "get_global_layout",
     "make_bucketed_block_placement_fn",

@@ -8,6 +8,7 @@ from .fp8_bucketed_block_shard import (
     Fp8BucketedBlockShard,
     make_fp8_bucketed_block_placement_fn,
 )
+from .mixed_bucket import MixedBucketPlacement
 from .owned import (
     BucketedOwned,
     BucketedOwnedSegmentSpec,
@@ -16,6 +17,7 @@ from .owned import (
     make_bucketed_owned_full_param_placement_fn,
     make_bucketed_owned_full_param_segments,
 )
+from .shard import Shard, make_shard_placement_fn
 from .utils import LocalReduceGroup
 
 __all__ = [
@@ -27,10 +29,13 @@ __all__ = [
     "BucketedOwnedSegmentSpec",
     "Fp8BucketedBlockShard",
     "LocalReduceGroup",
+    "MixedBucketPlacement",
+    "Shard",
     "make_bucketed_block_placement_fn",
     "make_bucketed_owned_expert_block_placement_fn",
     "make_bucketed_owned_expert_block_segments",
     "make_bucketed_owned_full_param_placement_fn",
     "make_bucketed_owned_full_param_segments",
     "make_fp8_bucketed_block_placement_fn",
+    "make_shard_placement_fn",
 ]

@@ -177,7 +177,7 @@ class BucketRuntime:
         cls,
         root: nn.Module,
         fqns: list[str],
-        placement: Placement,
+        placement: "Placement | dict[str, Placement]",
         mesh: Any,
         context: BucketCommContext,
         gradient_reduction: GradientReduction | None = None,
@@ -188,10 +188,14 @@ class BucketRuntime:
         and install them as the modules' parameters.  ``reduce_dtype`` is the
         mixed-precision policy's gradient dtype: full-parameter gradients
         accumulate and are reduced in it."""
-        from ..testing import local_rows, make_param_infos
+        from ..testing import local_rows, make_mixed_param_infos
 
         named = [(fqn, root.get_parameter(fqn)) for fqn in fqns]
-        infos = make_param_infos(named, placement, mesh)
+        if isinstance(placement, dict):  # member placements of one bucket-scoped placement, by fqn
+            param_placements = {fqn: (placement[fqn],) for fqn in fqns}
+        else:
+            param_placements = {fqn: (placement,) for fqn in fqns}
+        infos = make_mixed_param_infos(named, param_placements, mesh)
         for info in infos:
             info.reduce_dtype = reduce_dtype
         device = named[0][1].device
@@ -201,7 +205,10 @@ class BucketRuntime:
         for (fqn, param), info in zip(named, infos, strict=True):
             local = storage[info.byte_offset : info.byte_offset + info.local_numel * param.element_size()]
             local = local.view(param.dtype).view(info.local_shape)
-            local.copy_(local_rows(param, info))
+            if info.bucket_layout is not None:
+                local.copy_(local_rows(param, info))
+            else:  # per-parameter placements (Shard) cut their own shard
+                local.copy_(info.placement.extract_local_shard(param.detach(), mesh.get_local_rank(), mesh.size()))
             sharded = nn.Parameter(local, requires_grad=param.requires_grad)
             module_path, _, name = fqn.rpartition(".")
             module = root.get_submodule(module_path) if module_path else root

@@ -61,6 +61,27 @@ def make_param_infos(named_params: list[tuple[str, nn.Parameter]], placement: Pl
     return infos
 
 
+def make_mixed_param_infos(
+    named_params: list[tuple[str, nn.Parameter]], param_placements: dict[str, tuple[Placement, ...]], mesh
+) -> list[ParamInfo]:
+    """ParamInfos of a bucket whose parameters carry different member
+    placements of one bucket-scoped placement (a mixed bucket): the first
+    parameter's placement lays out the bucket."""
+    layout = param_placements[named_params[0][0]][0].bucket_storage_layout(named_params, param_placements, mesh)
+    infos = []
+    for fqn, param in named_params:
+        p = layout.param_layouts[fqn]
+        infos.append(
+            ParamInfo(
+                fqn=fqn, global_shape=param.shape, global_stride=tuple(param.stride()), dtype=param.dtype,
+                requires_grad=param.requires_grad, placements=param_placements[fqn], local_shape=p.local_shape,
+                local_numel=p.local_numel, byte_offset=p.byte_offset, storage_nbytes=p.storage_nbytes,
+                global_numel=param.numel(), bucket_layout=p.bucket_layout,
+            )
+        )
+    return infos
+
+
 def local_rows(param: torch.Tensor, info: ParamInfo) -> torch.Tensor:
     """The rank's shard of ``param``: a row range of its flattened matrix."""
     if info.local_numel == 0:

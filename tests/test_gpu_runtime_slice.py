@@ -201,3 +201,57 @@ def test_two_dense_buckets_share_the_streams(device):
             shard.grad = None
             layer.weight.grad = None
     torch.cuda.synchronize()
+
+
+def test_mixed_bucket_under_hooks(device):
+    """Biases as Shard(0) members next to the FP8 weights in one mixed bucket
+    of a one-rank mesh, driven by the forward/backward hooks: outputs and all
+    gradients equal the same autograd graph on directly built FP8 weights."""
+    from flex_shard_amd import MixedBucketPlacement
+
+    gen = torch.Generator().manual_seed(5)
+    model = nn.Sequential(nn.Linear(256, 384), nn.Linear(384, 256))
+    with torch.no_grad():
+        for p in model.parameters():
+            p.copy_(torch.randn(p.shape, generator=gen) * 0.05)
+    model = model.to(device=device, dtype=torch.bfloat16)
+    full = {fqn: p.detach().clone() for fqn, p in model.named_parameters()}
+    convert_to_flex_shard_float8_blockwise_linear(model)
+    mixed = MixedBucketPlacement({})
+    member = mixed.blockwise_quant_bucketed_block_shard(
+        Fp8BucketedBlockShard(world_size=1, weight_factory=make_blockwise_fp8_weight)
+    )
+    fqns = ["0.weight", "0.bias", "1.weight", "1.bias"]
+    placements = {fqn: (member if fqn.endswith("weight") else mixed.shard0) for fqn in fqns}
+    context = BucketCommContext.create(device)
+    runtime = BucketRuntime.shard_module_params(
+        model, fqns, placements, FakeMesh(1, 0, LocalReduceGroup(1, 0)), context
+    )
+    runtime.install_hooks(model)
+    x = torch.randn(64, 256, generator=gen).bfloat16().to(device)
+    grad_out = (torch.randn(64, 256, generator=gen) * 0.01).bfloat16().to(device)
+    for step in range(2):
+        x_run = x.clone().requires_grad_()
+        out = model(x_run)
+        assert all(b.untyped_storage().size() == 0 for b in runtime.persistent_buffers)
+        out.backward(grad_out)
+        context.wait_and_clear_reduce_grad_states()
+        # the same graph on weights quantized directly
+        leaves = {}
+        for fqn, value in full.items():
+            if fqn.endswith("weight"):
+                q, s = _quantize_dense_weight_to_blockwise_fp8(value, 128, torch.float8_e4m3fn)
+                leaves[fqn] = BlockwiseFp8Weight(q, s, 128, requires_grad=True)
+            else:
+                leaves[fqn] = value.clone().requires_grad_()
+        x_ref = x.clone().requires_grad_()
+        hidden = prequantized_linear(x_ref, leaves["0.weight"], leaves["0.bias"])
+        ref = prequantized_linear(hidden, leaves["1.weight"], leaves["1.bias"])
+        ref.backward(grad_out)
+        assert torch.equal(out.detach(), ref.detach()) and torch.equal(x_run.grad, x_ref.grad)
+        for bucket_param in runtime.bucket_params:
+            shard, want = bucket_param.sharded_param, leaves[bucket_param.info.fqn].grad
+            assert shard.grad.dtype == torch.bfloat16
+            assert torch.equal(shard.grad.view(want.shape), want.to(torch.bfloat16)), bucket_param.info.fqn
+            shard.grad = None
+    torch.cuda.synchronize()
