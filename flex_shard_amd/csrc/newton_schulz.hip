@@ -946,6 +946,7 @@ struct NsState {
   uint16_t* G;
   uint16_t* P;
   int cur;
+  bool tall;  // the caller's matrix is X^T
 };
 
 int ns_begin(const fsh_ns_problem& q, int32_t steps, float eps, hipStream_t stream, NsState* st) {
@@ -981,6 +982,7 @@ int ns_begin(const fsh_ns_problem& q, int32_t steps, float eps, hipStream_t stre
   st->XT[0] = tall ? x : w0;
   st->XT[1] = w1;
   st->cur = steps & 1;
+  st->tall = tall;
 
   hipLaunchKernelGGL(sumsq_partial_kernel, dim3(kNormBlocksPerMatrix, static_cast<uint32_t>(batch)),
                      dim3(kNormThreads), 0, stream, x, rows * cols, partial);
@@ -1001,8 +1003,10 @@ int ns_begin(const fsh_ns_problem& q, int32_t steps, float eps, hipStream_t stre
 // b G + c G G (symmetric because G is), 2: X' = P X = a X + (b G + c G G) X,
 // also written transposed into the other X^T buffer.  Carrying `a` on P's
 // diagonal (added in fp32 before P is rounded) spares the last product a
-// read of X from HBM per output tile.
-fsh_gemm_desc ns_product(const NsState& st, int which, float a, float b, float c) {
+// read of X from HBM per output tile.  The last step of the iteration writes
+// only the orientation the caller holds: X' for a wide input, and for a tall
+// one X'^T = X^T P (P is symmetric) computed directly.
+fsh_gemm_desc ns_product(const NsState& st, int which, float a, float b, float c, bool last_step) {
   const int64_t s = st.s, l = st.l, sl = s * l, ss = s * s;
   fsh_gemm_desc g;
   memset(&g, 0, sizeof(g));
@@ -1020,8 +1024,13 @@ fsh_gemm_desc ns_product(const NsState& st, int which, float a, float b, float c
     g.alpha = c; g.beta = b;
     g.diag_add = a;
     g.symmetric = 1;
+  } else if (last_step && st.tall) {
+    g.a_dev = st.XT[st.cur]; g.b_dev = st.P; g.c_dev = st.XT[st.cur ^ 1];
+    g.m = l; g.n = s; g.k = s; g.lda = s; g.ldb = s; g.ldc = s;
+    g.stride_a = sl; g.stride_b = ss; g.stride_c = sl;
+    g.alpha = 1.0f; g.beta = 0.0f;
   } else {
-    g.a_dev = st.P; g.b_dev = st.XT[st.cur]; g.c_dev = st.X; g.ct_dev = st.XT[st.cur ^ 1];
+    g.a_dev = st.P; g.b_dev = st.XT[st.cur]; g.c_dev = st.X; g.ct_dev = last_step ? nullptr : st.XT[st.cur ^ 1];
     g.m = s; g.n = l; g.k = s; g.lda = s; g.ldb = s; g.ldc = l; g.ldct = s;
     g.stride_a = ss; g.stride_b = sl; g.stride_c = sl; g.stride_ct = sl;
     g.alpha = 1.0f; g.beta = 0.0f;
@@ -1048,7 +1057,7 @@ FSH_API int fsh_newton_schulz_multi(const fsh_ns_problem* problems, int32_t coun
     // The same product of every problem goes out together: problems are
     // independent of each other, the three products of one are not.
     for (int which = 0; which < 3; ++which) {
-      for (int i = 0; i < count; ++i) descs[i] = ns_product(st[i], which, a, b, c);
+      for (int i = 0; i < count; ++i) descs[i] = ns_product(st[i], which, a, b, c, step + 1 == steps);
       if (int rc = launch_gemms(descs, count, stream)) return rc;
     }
     for (int i = 0; i < count; ++i) st[i].cur ^= 1;
