@@ -496,12 +496,11 @@ int launch_fp8_gemm(Fp8GemmParams& p, bool column_scales, const char* who, void*
   s.tiles_per_matrix = static_cast<int32_t>(tiles);
   s.work_items = tiles;
   s.items_per_xcd = ceil_div(tiles, static_cast<int64_t>(kXcds));
-  static bool reserved = false;
-  if (!reserved) {
-    if (int rc = reserve_lds(&fp8_gemm_blockwise_kernel<false>, Fp8Gemm::kLdsBytes)) return rc;
-    if (int rc = reserve_lds(&fp8_gemm_blockwise_kernel<true>, Fp8Gemm::kLdsBytes)) return rc;
-    reserved = true;
-  }
+  static LdsReservation reserved_block_scales, reserved_column_scales;
+  if (int rc = column_scales
+                   ? reserve_lds_once(reserved_column_scales, &fp8_gemm_blockwise_kernel<true>, Fp8Gemm::kLdsBytes)
+                   : reserve_lds_once(reserved_block_scales, &fp8_gemm_blockwise_kernel<false>, Fp8Gemm::kLdsBytes))
+    return rc;
   const dim3 grid(static_cast<uint32_t>(s.items_per_xcd * kXcds)), block(Fp8Gemm::kThreads);
   if (column_scales)
     hipLaunchKernelGGL(fp8_gemm_blockwise_kernel<true>, grid, block, Fp8Gemm::kLdsBytes, static_cast<hipStream_t>(stream), p);

@@ -4,6 +4,7 @@
 #pragma once
 #include "common.hpp"
 
+#include <atomic>
 #include <type_traits>
 
 namespace fsh {
@@ -485,6 +486,24 @@ int reserve_lds(Kernel kernel, int bytes) {
   hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
   if (err != hipSuccess) return fail(FSH_EHIP, "gemm: cannot reserve %d bytes of LDS: %s", bytes, hipGetErrorString(err));
+  return FSH_OK;
+}
+
+
+// The attribute is per device and function, and sticky: it is set once per
+// device and kernel, whichever host thread gets there first (setting it
+// twice is harmless).
+struct LdsReservation {
+  std::atomic<uint64_t> devices{0};
+};
+template <typename Kernel>
+int reserve_lds_once(LdsReservation& done, Kernel kernel, int bytes) {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) device = 0;
+  const uint64_t bit = (device >= 0 && device < 64) ? (1ull << device) : 0;
+  if (bit && (done.devices.load(std::memory_order_acquire) & bit)) return FSH_OK;
+  if (int rc = reserve_lds(kernel, bytes)) return rc;
+  if (bit) done.devices.fetch_or(bit, std::memory_order_release);
   return FSH_OK;
 }
 

@@ -701,12 +701,9 @@ int64_t compute_units() {
 }
 
 template <typename Kernel>
-int launch_single(Kernel kernel, bool* reserved, int lds_bytes, int threads, const PlannedGemm& plan,
+int launch_single(Kernel kernel, LdsReservation* reserved, int lds_bytes, int threads, const PlannedGemm& plan,
                   hipStream_t stream, const char* name) {
-  if (!*reserved) {  // the attribute is per device function and sticky
-    if (int rc = reserve_lds(kernel, lds_bytes)) return rc;
-    *reserved = true;
-  }
+  if (int rc = reserve_lds_once(*reserved, kernel, lds_bytes)) return rc;
   hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(plan.workgroups)), dim3(threads), lds_bytes, stream, plan.p);
   return check_launch(name);
 }
@@ -717,8 +714,7 @@ int launch_single(Kernel kernel, bool* reserved, int lds_bytes, int threads, con
 // round of another instead of each launch paying its own tail.  The problems
 // of one call must not depend on each other.
 int launch_planned(PlannedGemm* plans, int count, hipStream_t stream) {
-  static bool reserved_dma = false, reserved_persistent = false, reserved_small = false, reserved_edge_big = false,
-              reserved_edge_small = false;
+  static LdsReservation reserved_dma, reserved_persistent, reserved_small, reserved_edge_big, reserved_edge_small;
   constexpr int kDmaLds = kDmaGemmLdsBytes;
   int i = 0;
   while (i < count) {
@@ -769,17 +765,11 @@ int launch_planned(PlannedGemm* plans, int count, hipStream_t stream) {
     for (int k = 1; k < n; ++k) equal_k = equal_k && plans[order[k]].p.K == plans[order[0]].p.K;
     const int64_t units = compute_units();
     if (equal_k && units >= kXcds && units % kXcds == 0 && total > units) {
-      if (!reserved_persistent) {
-        if (int rc = reserve_lds(&gemm_nt_dma_kernel<true>, kDmaLds)) return rc;
-        reserved_persistent = true;
-      }
+      if (int rc = reserve_lds_once(reserved_persistent, &gemm_nt_dma_kernel<true>, kDmaLds)) return rc;
       hipLaunchKernelGGL(gemm_nt_dma_kernel<true>, dim3(static_cast<uint32_t>(units)), dim3(DmaGemm::kThreads),
                          kDmaLds, stream, launch);
     } else {
-      if (!reserved_dma) {
-        if (int rc = reserve_lds(&gemm_nt_dma_kernel<false>, kDmaLds)) return rc;
-        reserved_dma = true;
-      }
+      if (int rc = reserve_lds_once(reserved_dma, &gemm_nt_dma_kernel<false>, kDmaLds)) return rc;
       hipLaunchKernelGGL(gemm_nt_dma_kernel<false>, dim3(static_cast<uint32_t>(total)), dim3(DmaGemm::kThreads),
                          kDmaLds, stream, launch);
     }
