@@ -170,6 +170,7 @@ class BucketRuntime:
         self._hook_handles: list[Any] = []
         self._grads_seen = 0
         self._reduce_when_grads_arrive = False
+        self._pending_unshard: UnshardHandle | None = None
 
     # ------------------------------------------------------------ construction
     @classmethod
@@ -275,10 +276,30 @@ class BucketRuntime:
                     unsharded.requires_grad_(bp.sharded_param.requires_grad)
         self.is_unsharded = True
 
+    def prefetch(self) -> None:
+        """Begin this bucket's unshard on the unshard stream ahead of its use
+        (the quantize + pack and the exchange then run under the consumer
+        stream's work); the next ``unshard`` finishes it instead of beginning
+        one (reference: ``BucketCommContext.prefetch`` / ``take_pending_unshard``,
+        bucket_runtime.py:300-396)."""
+        if not self.is_unsharded and self._pending_unshard is None:
+            self._pending_unshard = self.begin_unshard()
+
+    def release_prefetch(self) -> None:
+        """Drop a prefetched unshard that will not be used."""
+        if self._pending_unshard is not None:
+            self._pending_unshard.release_buffers()
+            self._pending_unshard = None
+            if self.unsharded_params is not None:
+                self.free_persistent_storage()
+
     def unshard(self, *, on_current_stream: bool = False) -> None:
         """Make the unsharded params hold data and swap them into the modules."""
         if not self.is_unsharded:
-            self.finish_unshard(self.begin_unshard(on_current_stream=on_current_stream))
+            result, self._pending_unshard = self._pending_unshard, None
+            if result is None:
+                result = self.begin_unshard(on_current_stream=on_current_stream)
+            self.finish_unshard(result)
         self._swap_in_params(self.unsharded_params)
 
     def _create_unsharded_params(self, full_params: list[torch.Tensor], persistent_buffers: list[torch.Tensor]) -> None:

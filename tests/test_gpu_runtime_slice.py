@@ -255,3 +255,52 @@ def test_mixed_bucket_under_hooks(device):
             assert torch.equal(shard.grad.view(want.shape), want.to(torch.bfloat16)), bucket_param.info.fqn
             shard.grad = None
     torch.cuda.synchronize()
+
+
+def test_prefetched_unshard_is_taken_by_the_next_unshard(device):
+    """The second layer's bucket is prefetched before the first layer runs (its
+    quantize + pack goes to the unshard stream under the first layer's GEMMs);
+    results equal the run without prefetch, and a prefetch that is not used
+    can be released."""
+    gen = torch.Generator().manual_seed(6)
+    model = _mlp(device, gen)
+    convert_to_flex_shard_float8_blockwise_linear(model)
+    context = BucketCommContext.create(device)
+    mesh = FakeMesh(1, 0, LocalReduceGroup(1, 0))
+    runtimes = []
+    for index, layer in enumerate(model):
+        placement = Fp8BucketedBlockShard(world_size=1, weight_factory=make_blockwise_fp8_weight)
+        runtime = BucketRuntime.shard_module_params(model, [f"{index}.weight"], placement, mesh, context)
+        runtime.install_hooks(layer)
+        runtimes.append(runtime)
+    x = torch.randn(64, 256, generator=gen).bfloat16().to(device)
+    grad_out = (torch.randn(64, 256, generator=gen) * 0.01).bfloat16().to(device)
+
+    def run(prefetch: bool):
+        for runtime in runtimes:
+            for shard in runtime.sharded_params:
+                shard.grad = None
+        x_run = x.clone().requires_grad_()
+        if prefetch:
+            runtimes[1].prefetch()
+            assert runtimes[1]._pending_unshard is not None
+        out = model(x_run)
+        assert runtimes[1]._pending_unshard is None
+        if prefetch:  # backward runs layer 1 first, then layer 0
+            runtimes[0].prefetch()
+        out.backward(grad_out)
+        context.wait_and_clear_reduce_grad_states()
+        return out.detach(), x_run.grad, [r.sharded_params[0].grad.clone() for r in runtimes]
+
+    plain = run(False)  # also the first unshard, which creates the persistent buffers
+    for _ in range(2):
+        fetched = run(True)
+        assert torch.equal(plain[0], fetched[0]) and torch.equal(plain[1], fetched[1])
+        assert all(torch.equal(a, b) for a, b in zip(plain[2], fetched[2]))
+    runtimes[0].prefetch()
+    runtimes[0].release_prefetch()
+    assert runtimes[0]._pending_unshard is None
+    assert all(b.untyped_storage().size() == 0 for b in runtimes[0].persistent_buffers)
+    again = run(False)
+    assert torch.equal(plain[0], again[0])
+    torch.cuda.synchronize()
