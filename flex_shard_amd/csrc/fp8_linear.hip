@@ -98,29 +98,32 @@ __global__ __launch_bounds__(kActThreads) void act_quant_1x128_kernel(const ActQ
 }
 
 // ----------------------------------------------------------------- FP8 GEMM
-// 256 x 256 output tile per workgroup, four waves of 128 x 128 (four by four
-// 32x32 blocks): 262 flop per operand byte, which is what keeps the request
-// rate to L2 within reach at FP8 speed (a 128 x 256 tile needs 50 % more
-// operand bytes per flop).  Operand tiles are 128 bytes per row and k-tile and
-// travel global -> LDS directly, 16-byte chunk c of row r in slot c ^ ((r >> 1) & 7),
-// into one of two 64 KB stages.  A lane feeds the matrix core bytes
-// [32 h, 32 h + 32) of each half of its row (h = lane / 32), i.e. chunks 2h
-// and 2h+1 of a 64-byte half.
+// 256 x 256 output tile per workgroup (262 flop per operand byte, which is
+// what keeps the request rate to L2 within reach at FP8 speed), eight waves of
+// 64 x 128 (two by four 32x32 blocks).  A wave's 128 accumulators stay in
+// architectural VGPRs, where the vector ALU folds into them, and two waves
+// share a SIMD, so one wave's folds run under the other's MFMAs.  Operand
+// tiles are 128 bytes per row and k-tile and travel global -> LDS directly,
+// 16-byte chunk c of row r in slot c ^ ((r >> 1) & 7), into one of two 64 KB
+// stages.  A lane feeds the matrix core bytes [32 h, 32 h + 32) of each half
+// of its row (h = lane / 32), i.e. chunks 2h and 2h+1 of a 64-byte half.
 struct Fp8Gemm {
-  static constexpr int BM = 256, BN = 256, BK = 128, WM = 2, WN = 2, TM = 4, TN = 4;
-  static constexpr int kThreads = 256, kWaveM = 128, kWaveN = 128;
+  static constexpr int BM = 256, BN = 256, BK = 128, WM = 4, WN = 2, TM = 2, TN = 4;
+  static constexpr int kWaves = WM * WN, kThreads = 64 * kWaves, kWaveM = BM / WM, kWaveN = BN / WN;
   static constexpr int kRowBytes = 128;
   static constexpr int kABytes = BM * kRowBytes;               // 32 KB
   static constexpr int kStageBytes = (BM + BN) * kRowBytes;    // 64 KB
-  static constexpr int kLoadsA = BM / 8 / 4, kLoadsB = BN / 8 / 4;  // per wave: 8 and 8
+  static constexpr int kFillRows = 8 * kWaves;                 // tile rows per wave-level load of all waves
+  static constexpr int kLoadsA = BM / kFillRows, kLoadsB = BN / kFillRows;  // per wave: 4 and 4
   static constexpr int kPitch = kWaveN * 2 + 8;                // epilogue staging, bytes
   static constexpr int kRegion = kWaveM * kPitch;              // per wave
   static constexpr int kStages = 2;
-  static constexpr int kScaleStageBytes = 4 * kWaveM * 4;      // per stage: [wave][128] row scales
+  static constexpr int kScaleStageBytes = kWaves * kWaveM * 4;  // per stage: [wave][64] row scales
   static constexpr int kScaleOffset = kStages * kStageBytes;
   static constexpr int kWeightScaleOffset = kScaleOffset + kStages * kScaleStageBytes;  // [wave][256] block scales
   static constexpr int kMaxKTilesInLds = 256;
-  static constexpr int kLdsBytes = max_int(kWeightScaleOffset + 4 * kMaxKTilesInLds * 4, 4 * kRegion);
+  static constexpr int kLdsBytes = max_int(kWeightScaleOffset + kWaves * kMaxKTilesInLds * 4, kWaves * kRegion);
+  static_assert(kWaveM == 64, "one 4-byte scale request per wave covers its rows");
 };
 
 struct Fp8GemmParams {
@@ -158,7 +161,7 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
   const int64_t m0 = static_cast<int64_t>(tm) * Cfg::BM, n0 = static_cast<int64_t>(tn) * Cfg::BN;
   const int64_t ktiles = p.k / Cfg::BK;
 
-  // Load side: wave-level load q of a wave fills tile rows [32 q + 8 wave, +8);
+  // Load side: wave-level load q of a wave fills tile rows [64 q + 8 wave, +8);
   // lane l fills slot l & 7 of row l >> 3 there.  Rows past the matrix are
   // read from its last row (their products are never stored).
   const int fill_row = lane >> 3;
@@ -166,13 +169,13 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
   uint32_t a_voff[Cfg::kLoadsA], b_voff[Cfg::kLoadsB];
 #pragma unroll
   for (int q = 0; q < Cfg::kLoadsA; ++q) {
-    int64_t row = m0 + 32 * q + 8 * wave + fill_row;
+    int64_t row = m0 + Cfg::kFillRows * q + 8 * wave + fill_row;
     row = row < p.m ? row : p.m - 1;
     a_voff[q] = static_cast<uint32_t>((row - m0) * p.ldxq + fill_chunk * 16);
   }
 #pragma unroll
   for (int q = 0; q < Cfg::kLoadsB; ++q) {
-    int64_t row = n0 + 32 * q + 8 * wave + fill_row;
+    int64_t row = n0 + Cfg::kFillRows * q + 8 * wave + fill_row;
     row = row < p.n ? row : p.n - 1;
     b_voff[q] = static_cast<uint32_t>((row - n0) * p.ldwq + fill_chunk * 16);
   }
@@ -185,10 +188,11 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
     const uint8_t* a_src = Ab + kt * Cfg::kRowBytes;
     const uint8_t* b_src = Bb + kt * Cfg::kRowBytes;
 #pragma unroll
-    for (int q = 0; q < Cfg::kLoadsA; ++q) dma_load_16(a_voff[q], a_src, stage_off + fill_lds + q * 4096);
+    for (int q = 0; q < Cfg::kLoadsA; ++q)
+      dma_load_16(a_voff[q], a_src, stage_off + fill_lds + q * Cfg::kFillRows * Cfg::kRowBytes);
 #pragma unroll
     for (int q = 0; q < Cfg::kLoadsB; ++q)
-      dma_load_16(b_voff[q], b_src, stage_off + Cfg::kABytes + fill_lds + q * 4096);
+      dma_load_16(b_voff[q], b_src, stage_off + Cfg::kABytes + fill_lds + q * Cfg::kFillRows * Cfg::kRowBytes);
   };
 
   // Fragment side: row = lane & 31 of a 32-row block; chunks 4 kh + 2 h and
@@ -228,42 +232,38 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
   // compiler-visible load here would make the compiler wait for everything in
   // flight, the prefetched tile included.
   const uint32_t scale_lds0 = lds_base + static_cast<uint32_t>(Cfg::kScaleOffset + wave * Cfg::kWaveM * 4);
-  uint32_t scale_voff[2];
-#pragma unroll
-  for (int half = 0; half < 2; ++half) {
-    const int64_t row = m0 + wm * Cfg::kWaveM + half * 64 + lane;
-    scale_voff[half] = static_cast<uint32_t>((row < p.m ? row : p.m - 1) * 4);
-  }
+  const int64_t scale_row = m0 + wm * Cfg::kWaveM + lane;
+  const uint32_t scale_voff = static_cast<uint32_t>((scale_row < p.m ? scale_row : p.m - 1) * 4);
   // Per-column scales of the workgroup's 256 columns take the same road, 64
-  // columns per wave, into [stage][256] floats of the block-scale area.
+  // columns per wave (the first four waves), into [stage][256] floats of the
+  // block-scale area.
   const uint32_t cscale_lds0 = lds_base + static_cast<uint32_t>(Cfg::kWeightScaleOffset + wave * 256);
   const int64_t cscale_col0 = n0 + wave * 64 + lane;
   const uint32_t cscale_voff = static_cast<uint32_t>((cscale_col0 < p.n ? cscale_col0 : p.n - 1) * 4);
   auto issue_scale_loads = [&](int64_t kt, int stage) {
     const uint8_t* xs_row = reinterpret_cast<const uint8_t*>(p.xs + kt * p.m);
-    dma_touch_4(scale_voff[0], xs_row, scale_lds0 + stage * Cfg::kScaleStageBytes);
-    dma_touch_4(scale_voff[1], xs_row, scale_lds0 + stage * Cfg::kScaleStageBytes + 256);
-    if (kColumnScales)
+    dma_touch_4(scale_voff, xs_row, scale_lds0 + stage * Cfg::kScaleStageBytes);
+    if (kColumnScales && wave < 4)
       dma_touch_4(cscale_voff, reinterpret_cast<const uint8_t*>(p.cs + kt * p.n), cscale_lds0 + stage * 1024);
   };
   auto issue_k_tile = [&](int64_t kt, int stage) {
     issue_tile_load(kt, stage * Cfg::kStageBytes);
     issue_scale_loads(kt, stage);
   };
-  // One sixteenth of the next k-tile's requests; issued behind each block's
-  // MFMAs.  Sixteen 1 KB requests in a row keep the wave's instruction issue
-  // waiting on the memory pipeline (0.67 us per k-tile by measurement) while
-  // the matrix core runs dry.
+  // One eighth of the wave's requests for the next k-tile; issued behind each
+  // block's MFMAs rather than all at once, which would hold up the wave's
+  // instruction issue while the matrix core runs dry.
   auto issue_k_tile_part = [&](int64_t kt, int stage, int part) {
     const int stage_off = stage * Cfg::kStageBytes;
     const int q = part >> 1;
     if (part & 1)
-      dma_load_16(b_voff[q], Bb + kt * Cfg::kRowBytes, stage_off + Cfg::kABytes + fill_lds + q * 4096);
+      dma_load_16(b_voff[q], Bb + kt * Cfg::kRowBytes,
+                  stage_off + Cfg::kABytes + fill_lds + q * Cfg::kFillRows * Cfg::kRowBytes);
     else
-      dma_load_16(a_voff[q], Ab + kt * Cfg::kRowBytes, stage_off + fill_lds + q * 4096);
+      dma_load_16(a_voff[q], Ab + kt * Cfg::kRowBytes, stage_off + fill_lds + q * Cfg::kFillRows * Cfg::kRowBytes);
     if (part == 0) issue_scale_loads(kt, stage);
   };
-  static_assert(Cfg::kLoadsA == 8 && Cfg::kLoadsB == 8 && Cfg::TM * Cfg::TN == 16, "one request per block");
+  static_assert(Cfg::kLoadsA + Cfg::kLoadsB == Cfg::TM * Cfg::TN, "one request per block");
   // The block scales of the wave's 128 columns, one per k-tile, are copied
   // to LDS once (a load from global memory inside the loop would again wait
   // for the prefetched tile).
@@ -305,12 +305,14 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
     // A row blocks under the MFMAs of the first column block (they stay for
     // the whole k-tile), each further B column block while the previous one is
     // multiplied.
-    v8i32 afrag[TM][2], bfrag[2][2];
+    // The per-column variant has registers for one set of B fragments only.
+    constexpr int kBSets = kColumnScales ? 1 : 2;
+    v8i32 afrag[TM][2], bfrag[kBSets][2];
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh) bfrag[0][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32), kh);
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh) afrag[0][kh] = read_frag(stage_off, 0, wm * (Cfg::kWaveM / 32), kh);
-    // The sixteen 32x32 blocks, column block by column block: two MFMAs, back
+    // The wave's eight 32x32 blocks, column block by column block: two MFMAs, back
     // to back, give a block's partial product for this scale block.  It is
     // folded into the result (16 fused multiply-adds, or multiply + fused
     // multiply-add with per-column scales) two blocks later, behind that
@@ -319,23 +321,24 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
     // time units per block for the arrangement used here).
     const uint8_t* cscale_lds = lds_bytes + Cfg::kWeightScaleOffset + stage * 1024 + (wn * Cfg::kWaveN + 4 * h) * 4;
     constexpr int kBlocks = TM * TN;
-    // Blocks between a product and its fold; the per-column variant has no
-    // registers left for a third product.
-    constexpr int kLag = kColumnScales ? 1 : 2;
+    // Blocks between a product and its fold.  One: the other wave of the SIMD
+    // keeps the matrix core busy while this one waits for its own product,
+    // and the registers of a third product are needed elsewhere.
+    constexpr int kLag = 1;
     f32x16 part[kLag + 1];
-    f32x4 cscale[4];
     auto fold = [&](int blk, const f32x16& product) {
       const int pi = blk % TM, pj = blk / TM;
-      if (kColumnScales && pi == 0) {
+      if (kColumnScales) {
 #pragma unroll
-        for (int b = 0; b < 4; ++b) cscale[b] = *reinterpret_cast<const f32x4*>(cscale_lds + (pj * 32 + 8 * b) * 4);
-      }
+        for (int b = 0; b < 4; ++b) {  // four column scales at a time: 16 would not fit next to the accumulators
+          const f32x4 cs = *reinterpret_cast<const f32x4*>(cscale_lds + (pj * 32 + 8 * b) * 4);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        if (kColumnScales)
-          acc[pi][pj][r] = __builtin_fmaf(product[r] * s[pi], cscale[r / 4][r % 4], acc[pi][pj][r]);
-        else
-          acc[pi][pj][r] = __builtin_fmaf(product[r], s[pi], acc[pi][pj][r]);
+          for (int e = 0; e < 4; ++e)
+            acc[pi][pj][4 * b + e] = __builtin_fmaf(product[4 * b + e] * s[pi], cs[e], acc[pi][pj][4 * b + e]);
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[pi][pj][r] = __builtin_fmaf(product[r], s[pi], acc[pi][pj][r]);
       }
       // An empty statement that "uses" the folded block keeps its arithmetic
       // on this side of the next scheduling barrier.
@@ -349,15 +352,22 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
 #pragma unroll
         for (int kh = 0; kh < 2; ++kh) afrag[i + 1][kh] = read_frag(stage_off, 0, wm * (Cfg::kWaveM / 32) + i + 1, kh);
       }
-      if (i == 1 && j + 1 < TN) {  // next column block's B fragments
+      if (kBSets == 2 && i == TM - 1 && j + 1 < TN) {  // next column block's B fragments, one block ahead
 #pragma unroll
         for (int kh = 0; kh < 2; ++kh)
-          bfrag[(j + 1) & 1][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32) + j + 1, kh);
+          bfrag[(j + 1) % kBSets][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32) + j + 1, kh);
       }
-      f32x16 product = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j & 1][0], afrag[i][0], zero, 0, 0, 0, 0, 0, 0);
-      product = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j & 1][1], afrag[i][1], product, 0, 0, 0, 0, 0, 0);
+      f32x16 product =
+          __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j % kBSets][0], afrag[i][0], zero, 0, 0, 0, 0, 0, 0);
+      product =
+          __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j % kBSets][1], afrag[i][1], product, 0, 0, 0, 0, 0, 0);
       part[blk % (kLag + 1)] = product;
       __builtin_amdgcn_sched_barrier(0);
+      if (kBSets == 1 && i == TM - 1 && j + 1 < TN) {  // behind the last MFMAs that read the current set
+#pragma unroll
+        for (int kh = 0; kh < 2; ++kh)
+          bfrag[0][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32) + j + 1, kh);
+      }
       if (more) issue_k_tile_part(kt + 1, stage ^ 1, blk);
       if (blk >= kLag) fold(blk - kLag, part[(blk - kLag) % (kLag + 1)]);
       __builtin_amdgcn_sched_barrier(0);
@@ -380,7 +390,7 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
   }
 #ifdef FSH_TRACE
   if (p.schedule.trace && lane == 0) {
-    uint64_t* out = p.schedule.trace + (static_cast<int64_t>(blockIdx.x) * 4 + wave) * 8;
+    uint64_t* out = p.schedule.trace + (static_cast<int64_t>(blockIdx.x) * Cfg::kWaves + wave) * 8;
     out[0] = t_begin; out[1] = t_compute; out[2] = t_wait; out[3] = t_barrier; out[4] = t_mark;
   }
 #endif
