@@ -397,6 +397,9 @@ def main() -> None:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB -> 256 MiB segment copy, the known-size kernel that the "
                     "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
+    ap.add_argument("--only", choices=("muon", "fp8_linear"),
+                    help="profiling aid: run only this secondary section (for counter runs, which slow "
+                    "every kernel down) and print its figures instead of the benchmark line")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit(
@@ -411,6 +414,13 @@ def main() -> None:
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
+    if args.only == "muon":
+        print(json.dumps({"muon_newton_schulz": bench_muon(device)}))
+        return
+    if args.only == "fp8_linear":
+        print(json.dumps({"fp8_linear_forward_8192_tokens": bench_fp8_linear(device),
+                          "fp8_linear_backward_8192_tokens": bench_fp8_linear_backward(device)}))
+        return
     if args.calibrate_copy:
         calibrate_copy(device)
     q = bench_quant_pack(device, args.steps, args.warmup, args.layers)
