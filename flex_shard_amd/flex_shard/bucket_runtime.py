@@ -25,7 +25,7 @@ import torch.nn as nn
 from torch.utils._python_dispatch import is_traceable_wrapper_subclass
 
 from ..bucket_storage import ParamInfo
-from ..placement_contract import GradientReduction, Placement
+from ..placement_contract import GradientReduction, Placement, get_global_layout
 from .bucket_comm import (
     ReduceGradHandle,
     UnshardHandle,
@@ -197,8 +197,9 @@ class BucketRuntime:
         else:
             param_placements = {fqn: (placement,) for fqn in fqns}
         infos = make_mixed_param_infos(named, param_placements, mesh)
-        for info in infos:
+        for (_, param), info in zip(named, infos, strict=True):
             info.reduce_dtype = reduce_dtype
+            info.outer_layout = get_global_layout(param)  # the parameter was already a shard of an outer sharding
         device = named[0][1].device
         nbytes = max((i.byte_offset + i.local_numel * i.dtype.itemsize for i in infos), default=0)
         storage = torch.zeros(max(nbytes, 1), dtype=torch.uint8, device=device)

@@ -304,3 +304,57 @@ def test_prefetched_unshard_is_taken_by_the_next_unshard(device):
     again = run(False)
     assert torch.equal(plain[0], again[0])
     torch.cuda.synchronize()
+
+
+def test_checkpoint_layouts_of_sharded_buckets(device):
+    """Two ranks shard the same model; their state dicts, saved box by box
+    through the declared layouts, rebuild the full weights, and a one-rank
+    runtime loads them back.  Adam's states carry the same layouts."""
+    from flex_shard_amd import get_global_layout
+    from flex_shard_amd.flex_shard import (
+        copy_full_into_shard,
+        copy_shard_into_full,
+        register_optimizer_checkpoint_hook,
+        set_state_dict_global_layouts,
+    )
+
+    gen = torch.Generator().manual_seed(5)
+    reference = _mlp(device, gen)
+    full = {name: p.detach().clone() for name, p in reference.named_parameters()}
+    saved = {name: torch.full_like(p, float("nan")) for name, p in full.items()}
+    context = BucketCommContext.create(device)
+    for rank in range(2):
+        model = _mlp(device, torch.Generator().manual_seed(5))
+        placement = Fp8BucketedBlockShard(world_size=2, weight_factory=make_blockwise_fp8_weight)
+        runtime = BucketRuntime.shard_module_params(
+            model, ["0.weight", "1.weight"], placement, FakeMesh(2, rank, LocalReduceGroup(2, rank)), context
+        )
+        state_dict = model.state_dict()
+        set_state_dict_global_layouts([runtime], state_dict)
+        for name, tensor in state_dict.items():
+            layout = get_global_layout(tensor)
+            assert layout.global_shape == tuple(full[name].shape)
+            assert sum(s[0] for s in layout.local_sizes) == tensor.shape[0]  # whole 128-row blocks of this rank
+            copy_shard_into_full(saved[name], tensor, layout)
+        optimizer = torch.optim.AdamW(model.parameters(), lr=1e-3)
+        register_optimizer_checkpoint_hook(optimizer, [runtime])
+        for p in model.parameters():
+            p.grad = torch.ones_like(p)
+        optimizer.step()
+        states = optimizer.state_dict()["state"]
+        for param_id, name in enumerate(("0.weight", "1.weight")):
+            assert get_global_layout(states[param_id]["exp_avg"]) == get_global_layout(state_dict[name])
+            assert get_global_layout(states[param_id]["step"]) is None
+    assert all(torch.equal(saved[name], full[name]) for name in full)
+
+    model = _mlp(device, torch.Generator().manual_seed(6))  # different weights, overwritten by the load
+    placement = Fp8BucketedBlockShard(world_size=1, weight_factory=make_blockwise_fp8_weight)
+    runtime = BucketRuntime.shard_module_params(
+        model, ["0.weight", "1.weight"], placement, FakeMesh(1, 0, LocalReduceGroup(1, 0)), context
+    )
+    state_dict = model.state_dict()
+    set_state_dict_global_layouts([runtime], state_dict)
+    for name, tensor in state_dict.items():
+        copy_full_into_shard(tensor, saved[name], get_global_layout(tensor))
+    assert all(torch.equal(p.view(full[name].shape), full[name]) for name, p in model.named_parameters())
+    torch.cuda.synchronize()
