@@ -199,28 +199,38 @@ def bench_unpack(device, placement, infos, reps=10):
     from flex_shard_amd.testing import LLAMA3_8B_LAYER, FakeMesh, make_param_infos
 
     md = placement._quant_metadata_from_infos(infos)
-    rows = torch.randint(0, 120, (8, md.packed_send_nbytes_per_rank), dtype=torch.uint8, device=device)
-    for r in range(8):
-        s0 = md.rank_scale_byte_offsets[r]
-        rows[r, s0 : s0 + 4 * md.rank_scale_numels[r]].view(torch.float32).fill_(1e-4)
-    prepared = placement._prepare_local_unshard_payload
+    # Three gathered buffers (0.66 GB): rotating over them, every launch reads
+    # its rows from HBM; repeating one, from the last-level cache, where a
+    # gather that has just written them would leave them.
+    gathered = []
+    for _ in range(3):
+        rows = torch.randint(0, 120, (8, md.packed_send_nbytes_per_rank), dtype=torch.uint8, device=device)
+        for r in range(8):
+            s0 = md.rank_scale_byte_offsets[r]
+            rows[r, s0 : s0 + 4 * md.rank_scale_numels[r]].view(torch.float32).fill_(1e-4)
+        gathered.append(rows)
     from flex_shard_amd.placement_contract import PlacementPreparedUnshard
 
     state = placement._QuantUnshardState(infos=infos, pg=None, debug_fqn=None, metadata=md)
-    local = rows[0]
-    prep = PlacementPreparedUnshard(placement=placement, buffers=[local, rows.view(-1)], placement_state=state)
+    rows = gathered[0]
+    prep = PlacementPreparedUnshard(placement=placement, buffers=[rows[0], rows.view(-1)], placement_state=state)
     total = sum(i.global_numel for i in infos)
     out = torch.empty(total, dtype=torch.bfloat16, device=device)
     prep.persistent = True
     result, _ = placement.finish_prepared_unshard_with_dequant(prep, rows, dequant_out=out)
     prep.persistent_buffers = result.persistent_buffers
-    _, fused_ms = _event_ms(lambda i: placement.finish_prepared_unshard_with_dequant(prep, rows, dequant_out=out), reps, 2)
-    _, compact_ms = _event_ms(lambda i: placement._finish_unshard_from_rank_rows(prep, rows), reps, 2)
+    reps = 3 * ((reps + 2) // 3)
+    _, fused_ms = _event_ms(
+        lambda i: placement.finish_prepared_unshard_with_dequant(prep, gathered[i % 3], dequant_out=out), reps, 3)
+    _, fused_hot_ms = _event_ms(lambda i: placement.finish_prepared_unshard_with_dequant(prep, rows, dequant_out=out), reps, 3)
+    _, compact_ms = _event_ms(lambda i: placement._finish_unshard_from_rank_rows(prep, gathered[i % 3]), reps, 3)
     scales = sum(md.rank_scale_numels)
     return {
         "elems": total,
         "fused_unpack_dequant_ms": fused_ms / reps,
         "fused_GBps": (4 * total + 8 * scales) / (fused_ms / reps) / 1e6,
+        "fused_unpack_dequant_ms_rows_in_cache": fused_hot_ms / reps,
+        "fused_GBps_rows_in_cache": (4 * total + 8 * scales) / (fused_hot_ms / reps) / 1e6,
         "compact_only_ms": compact_ms / reps,
         "compact_GBps": (2 * total + 8 * scales) / (compact_ms / reps) / 1e6,
     }

@@ -104,7 +104,11 @@ __global__ __launch_bounds__(kThreads) void unpack_dequant_kernel(
     for (int k = 0; k < 8; ++k) {
       const int64_t row = tr * 128 + r0 + 16 * k;
       idxs[k] = (row < ch.rows ? row : ch.rows - 1) * ch.in_dim + col;
-      vin[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(src + idxs[k]));
+      // A plain load: with the nontemporal hint this kernel, three quarters of
+      // whose traffic are stores, measured 13 % slower on rows from HBM and
+      // 25 % slower on rows still in the last-level cache (where a gather
+      // has just written them).
+      vin[k] = *reinterpret_cast<const u32x2*>(src + idxs[k]);
     }
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
