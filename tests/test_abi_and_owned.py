@@ -173,3 +173,16 @@ def test_block_shard_layout_math():
     with pytest.raises(ValueError, match="world size"):
         shard.compute_local_shape(torch.Size((6, 4)), 0, 3)
     assert repr(BlockShard((1, 0), dim=1)) == "BlockShard(blocks_per_rank=(1, 0), dim=1)"
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """One rank's share on one GPU is all the benchmark measures: asking for
+    more exits with a message before anything touches a device."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    run = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert run.returncode != 0
+    assert "--gpus must be 1" in (run.stdout + run.stderr)
