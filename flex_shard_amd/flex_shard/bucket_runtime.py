@@ -24,8 +24,8 @@ import torch
 import torch.nn as nn
 from torch.utils._python_dispatch import is_traceable_wrapper_subclass
 
-from ..bucket_storage import ParamInfo
-from ..placement_contract import GradientReduction, Placement, get_global_layout
+from ..bucket_storage import ParamInfo, create_param_infos
+from ..placement_contract import GradientReduction, Placement
 from .bucket_comm import (
     ReduceGradHandle,
     UnshardHandle,
@@ -189,28 +189,21 @@ class BucketRuntime:
         and install them as the modules' parameters.  ``reduce_dtype`` is the
         mixed-precision policy's gradient dtype: full-parameter gradients
         accumulate and are reduced in it."""
-        from ..testing import local_rows, make_mixed_param_infos
-
         named = [(fqn, root.get_parameter(fqn)) for fqn in fqns]
         if isinstance(placement, dict):  # member placements of one bucket-scoped placement, by fqn
             param_placements = {fqn: (placement[fqn],) for fqn in fqns}
         else:
             param_placements = {fqn: (placement,) for fqn in fqns}
-        infos = make_mixed_param_infos(named, param_placements, mesh)
-        for (_, param), info in zip(named, infos, strict=True):
+        infos, total_bytes = create_param_infos(named, param_placements, mesh)
+        for info in infos:
             info.reduce_dtype = reduce_dtype
-            info.outer_layout = get_global_layout(param)  # the parameter was already a shard of an outer sharding
-        device = named[0][1].device
-        nbytes = max((i.byte_offset + i.local_numel * i.dtype.itemsize for i in infos), default=0)
-        storage = torch.zeros(max(nbytes, 1), dtype=torch.uint8, device=device)
+        rank, world_size = mesh.get_local_rank(), mesh.size()
+        storage = torch.zeros(max(total_bytes, 1), dtype=torch.uint8, device=named[0][1].device)
         bucket_params = []
         for (fqn, param), info in zip(named, infos, strict=True):
-            local = storage[info.byte_offset : info.byte_offset + info.local_numel * param.element_size()]
-            local = local.view(param.dtype).view(info.local_shape)
-            if info.bucket_layout is not None:
-                local.copy_(local_rows(param, info))
-            else:  # per-parameter placements (Shard) cut their own shard
-                local.copy_(info.placement.extract_local_shard(param.detach(), mesh.get_local_rank(), mesh.size()))
+            # the placement writes this rank's part of the parameter into the storage and views it
+            info.placement.copy_param_to_storage(storage, info, param, rank, world_size)
+            local = info.placement.make_local_storage_view(storage, info)
             sharded = nn.Parameter(local, requires_grad=param.requires_grad)
             module_path, _, name = fqn.rpartition(".")
             module = root.get_submodule(module_path) if module_path else root

@@ -16,7 +16,7 @@ from collections.abc import Sequence
 import torch
 import torch.nn as nn
 
-from .bucket_storage import ParamInfo
+from .bucket_storage import ParamInfo, create_param_infos
 from .placement_contract import Placement
 
 
@@ -38,27 +38,7 @@ class FakeMesh:
 
 def make_param_infos(named_params: list[tuple[str, nn.Parameter]], placement: Placement, mesh) -> list[ParamInfo]:
     """ParamInfos of parameters sharing one placement's bucket storage layout."""
-    layout = placement.bucket_storage_layout(named_params, {fqn: (placement,) for fqn, _ in named_params}, mesh)
-    infos = []
-    for fqn, param in named_params:
-        p = layout.param_layouts[fqn]
-        infos.append(
-            ParamInfo(
-                fqn=fqn,
-                global_shape=param.shape,
-                global_stride=tuple(param.stride()),
-                dtype=param.dtype,
-                requires_grad=param.requires_grad,
-                placements=(placement,),
-                local_shape=p.local_shape,
-                local_numel=p.local_numel,
-                byte_offset=p.byte_offset,
-                storage_nbytes=p.storage_nbytes,
-                global_numel=param.numel(),
-                bucket_layout=p.bucket_layout,
-            )
-        )
-    return infos
+    return create_param_infos(named_params, {fqn: (placement,) for fqn, _ in named_params}, mesh)[0]
 
 
 def make_mixed_param_infos(
@@ -67,19 +47,7 @@ def make_mixed_param_infos(
     """ParamInfos of a bucket whose parameters carry different member
     placements of one bucket-scoped placement (a mixed bucket): the first
     parameter's placement lays out the bucket."""
-    layout = param_placements[named_params[0][0]][0].bucket_storage_layout(named_params, param_placements, mesh)
-    infos = []
-    for fqn, param in named_params:
-        p = layout.param_layouts[fqn]
-        infos.append(
-            ParamInfo(
-                fqn=fqn, global_shape=param.shape, global_stride=tuple(param.stride()), dtype=param.dtype,
-                requires_grad=param.requires_grad, placements=param_placements[fqn], local_shape=p.local_shape,
-                local_numel=p.local_numel, byte_offset=p.byte_offset, storage_nbytes=p.storage_nbytes,
-                global_numel=param.numel(), bucket_layout=p.bucket_layout,
-            )
-        )
-    return infos
+    return create_param_infos(named_params, param_placements, mesh)[0]
 
 
 def local_rows(param: torch.Tensor, info: ParamInfo) -> torch.Tensor:

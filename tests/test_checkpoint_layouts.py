@@ -29,7 +29,6 @@ from flex_shard_amd.flex_shard import (
     register_optimizer_checkpoint_hook,
     set_state_dict_global_layouts,
 )
-from flex_shard_amd.bucket_storage import ParamInfo
 from flex_shard_amd.testing import FakeMesh, make_param_infos
 
 
@@ -38,18 +37,9 @@ def _factory(fp8_data, recip_scale, block_size, *, orig_dtype, requires_grad):
 
 
 def _infos(named, placement, rank, world_size):
-    mesh = FakeMesh(world_size, rank)
-    if placement.bucket_storage_layout(named, {fqn: (placement,) for fqn, _ in named}, mesh) is not None:
-        return make_param_infos(named, placement, mesh)
-    infos = []  # a per-parameter placement: every parameter is laid out on its own
-    for fqn, param in named:
-        local_shape = placement.compute_local_shape(param.shape, rank, world_size)
-        infos.append(ParamInfo(
-            fqn=fqn, global_shape=param.shape, global_stride=tuple(param.stride()), dtype=param.dtype,
-            requires_grad=param.requires_grad, placements=(placement,), local_shape=local_shape,
-            local_numel=local_shape.numel(), global_numel=param.numel(),
-        ))
-    return infos
+    """Bucket placements lay the bucket out; per-parameter ones (BlockShard)
+    get one parameter after the other."""
+    return make_param_infos(named, placement, FakeMesh(world_size, rank))
 
 
 def _layouts(named, placement, rank, world_size):
