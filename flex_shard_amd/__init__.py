@@ -6,7 +6,7 @@ as the drop-in surface; all device work is hand-written HIP for gfx950 behind
 the C ABI of ``libflexshard_hip.so`` (``include/flexshard_hip.h``).
 """
 
-from .bucket_storage import BucketLayout, BucketParamLayout, ParamInfo
+from .bucket_storage import BucketLayout, BucketParamLayout, ParamInfo, create_param_infos
 from .custom_placements import (
     BlockShard,
     BucketedBlockShard,
@@ -59,6 +59,7 @@ __all__ = [
     "PlacementUnshardResult",
     "Shard",
     "compose_global_layouts",
+    "create_param_infos",
     "get_global_layout",
     "make_bucketed_block_placement_fn",
     "make_bucketed_owned_full_param_placement_fn",
