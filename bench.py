@@ -236,6 +236,35 @@ def bench_unpack(device, placement, infos, reps=10):
     }
 
 
+def bench_gradient_copy_in(device, reps=5):
+    """One-pass copy-in of a Llama-3-8B layer's separate full-parameter
+    gradients into the [8, rank range] reduce-scatter input (one
+    `pack_segments_kernel` launch, zero gaps included): fp32 gradients as
+    they accumulate under an fp32 reduce dtype, and bf16 gradients cast to
+    fp32 on the way."""
+    import torch.nn as nn
+
+    from flex_shard_amd import BucketedBlockShard, LocalReduceGroup
+    from flex_shard_amd.testing import LLAMA3_8B_LAYER, FakeMesh, make_param_infos
+
+    world = 8
+    placement = BucketedBlockShard(dims=(0,), blocks_per_rank=(1,) * world)
+    named = [(n, nn.Parameter(torch.empty(s, device="meta", dtype=torch.bfloat16))) for n, s in LLAMA3_8B_LAYER]
+    mesh = FakeMesh(world, 0, LocalReduceGroup(world, 0))
+    infos = make_param_infos(named, placement, mesh)
+    for info in infos:
+        info.reduce_dtype = torch.float32
+    total = sum(i.global_numel for i in infos)
+    out = {}
+    for key, dtype in (("copy_in_fp32", torch.float32), ("copy_in_bf16_to_fp32", torch.bfloat16)):
+        grads = [torch.randn(i.global_shape, device=device, dtype=dtype) for i in infos]
+        _, ms = _event_ms(lambda i: placement.prepare_reduce_grad(grads, infos, mesh, None), reps, 2)
+        out[key + "_ms"] = ms / reps
+        out[key + "_GBps"] = total * (dtype.itemsize + 4) / (ms / reps) / 1e6
+        del grads
+    return out
+
+
 def bench_gradients(device, reps=5):
     """Config 4: 4 bf16 microbatches accumulated in fp32 over the 218 365 952
     element bucket (placement layout), then the 8-way fixed-order reduction of
@@ -254,7 +283,10 @@ def bench_gradients(device, reps=5):
     _, red_ms = _event_ms(lambda i: hip_ops.reduce_rows(out, contrib, 0), reps * 4, 2)
     acc_per = acc_ms / (4 * reps)
     red_per = red_ms / (reps * 4)
+    del acc, contrib, out
+    copy_in = bench_gradient_copy_in(device, reps)
     return {
+        **copy_in,
         "accumulate_ms_per_microbatch": acc_per,
         "accumulate_GBps": 10 * total / acc_per / 1e6,  # 2 B grad + 4 B read + 4 B write (6 B on the first)
         "reduce_ms": red_per,

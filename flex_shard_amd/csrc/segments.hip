@@ -56,6 +56,31 @@ __device__ __forceinline__ uint16_t cast_elem<float, uint16_t>(float v) {
   return static_cast<uint16_t>(f32_to_bf16_bits(v));
 }
 
+// Eight consecutive elements, both pointers 16-byte aligned.
+__device__ __forceinline__ void cast_group_of_8(const uint16_t* src, float* dst) {
+  const u32x4 v = load_stream_u32x4(src);
+  const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+  f32x4 lo, hi;
+  lo.x = u32_as_f32(d[0] << 16); lo.y = u32_as_f32(d[0] & 0xFFFF0000u);
+  lo.z = u32_as_f32(d[1] << 16); lo.w = u32_as_f32(d[1] & 0xFFFF0000u);
+  hi.x = u32_as_f32(d[2] << 16); hi.y = u32_as_f32(d[2] & 0xFFFF0000u);
+  hi.z = u32_as_f32(d[3] << 16); hi.w = u32_as_f32(d[3] & 0xFFFF0000u);
+  reinterpret_cast<f32x4*>(dst)[0] = lo;
+  reinterpret_cast<f32x4*>(dst)[1] = hi;
+}
+__device__ __forceinline__ void cast_group_of_8(const float* src, uint16_t* dst) {
+  const f32x4 a = load_stream_f32x4(src), b = load_stream_f32x4(src + 4);
+  u32x4 o;
+  o.x = f32_to_bf16_bits(a.x) | (f32_to_bf16_bits(a.y) << 16);
+  o.y = f32_to_bf16_bits(a.z) | (f32_to_bf16_bits(a.w) << 16);
+  o.z = f32_to_bf16_bits(b.x) | (f32_to_bf16_bits(b.y) << 16);
+  o.w = f32_to_bf16_bits(b.z) | (f32_to_bf16_bits(b.w) << 16);
+  *reinterpret_cast<u32x4*>(dst) = o;
+}
+// Same-type pairs never reach the casting branch; these keep it compilable.
+__device__ __forceinline__ void cast_group_of_8(const float*, float*) {}
+__device__ __forceinline__ void cast_group_of_8(const uint16_t*, uint16_t*) {}
+
 // Multi-input gather with cast.  A negative tensor index marks a zero-fill
 // segment.  Same-dtype segments move as bytes with the widest legal vector;
 // casting segments convert element by element (coalesced across the wave).
@@ -81,7 +106,16 @@ __global__ __launch_bounds__(kThreads) void pack_segments_kernel(
     copy_bytes(reinterpret_cast<const uint8_t*>(src), reinterpret_cast<uint8_t*>(dst),
                len * static_cast<int64_t>(sizeof(DST)), threadIdx.x, kThreads);
   } else {
-    for (int64_t i = threadIdx.x; i < len; i += kThreads) dst[i] = cast_elem<SRC, DST>(src[i]);
+    // Eight elements per thread and step when both sides start on a 16-byte
+    // boundary (16 bytes of bf16 against 32 of fp32); the rest, and slices
+    // that do not, go element by element.
+    int64_t done = 0;
+    if (((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0) {
+      const int64_t groups = len / 8;
+      for (int64_t g = threadIdx.x; g < groups; g += kThreads) cast_group_of_8(src + 8 * g, dst + 8 * g);
+      done = groups * 8;
+    }
+    for (int64_t i = done + threadIdx.x; i < len; i += kThreads) dst[i] = cast_elem<SRC, DST>(src[i]);
   }
 }
 

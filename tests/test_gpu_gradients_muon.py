@@ -114,6 +114,36 @@ def test_copy_in_casts_to_the_reduce_dtype_in_the_same_launch(device):
     assert torch.equal(prepared.buffers[0].view(want.shape).cpu(), want)
 
 
+@pytest.mark.parametrize("src_dtype,dst_dtype", [(torch.bfloat16, torch.float32), (torch.float32, torch.bfloat16)])
+def test_casting_pack_for_any_length_and_alignment(device, src_dtype, dst_dtype):
+    """Casting segments move eight elements per thread where both sides are
+    16-byte aligned and element by element elsewhere: lengths around the
+    group and slice sizes, at source and destination offsets of every
+    alignment, plus a zero-fill segment, against torch's cast."""
+    gen = torch.Generator().manual_seed(11)
+    lengths = [1, 7, 8, 9, 63, 4096, 4101, 8192 + 13, 20000]
+    src_offs = [0, 1, 3, 8, 5, 0, 2, 8, 16]
+    inputs = [torch.randn(n + o + 3, generator=gen).to(src_dtype).to(device) for n, o in zip(lengths, src_offs)]
+    dst_offs, cursor = [], 0
+    for k, n in enumerate(lengths):
+        cursor += (0, 1, 4, 0, 5, 0, 3, 8, 0)[k]  # gaps that put the destinations at odd alignments
+        dst_offs.append(cursor)
+        cursor += n
+    zero_at, zero_len = cursor + 2, 37
+    total = zero_at + zero_len + 5
+    out = torch.full((total,), 7.0, dtype=dst_dtype, device=device)
+    table = lambda values: torch.tensor(values, dtype=torch.int64, device=device)
+    hip_ops.pack_segments(
+        table([t.data_ptr() for t in inputs]), table(list(range(len(lengths))) + [-1]), table(src_offs + [0]),
+        table(lengths + [zero_len]), table(dst_offs + [zero_at]), max(lengths), src_dtype, out,
+    )
+    want = torch.full((total,), 7.0, dtype=dst_dtype)
+    for t, n, so, do in zip(inputs, lengths, src_offs, dst_offs):
+        want[do : do + n] = t[so : so + n].cpu().to(dst_dtype)
+    want[zero_at : zero_at + zero_len] = 0
+    assert torch.equal(out.cpu(), want)
+
+
 def test_copy_in_through_a_bucket_while_compiling(device):
     from unittest.mock import patch
 
