@@ -82,6 +82,8 @@ class GemmDesc(Structure):
         ("beta", c_float),
         ("symmetric", c_int32),
         ("diag_add", c_float),
+        ("k_major", c_int32),
+        ("reserved", c_int32),
     ]
 
 

@@ -26,6 +26,7 @@ struct GemmParams {
   float diag_add;         // added to C[i][i] before the rounding
   int32_t tiles_m, tiles_n;
   int32_t symmetric;      // only tiles with tm <= tn are computed; the others are mirrored
+  int32_t k_major;        // A is [K, M] and B is [K, N]: the product is A^T B (large-tile kernel only)
   int32_t tiles_per_matrix;
   int64_t work_items;     // tiles_per_matrix * batch
   int64_t items_per_xcd;  // ceil(work_items / 8); the grid has 8 * items_per_xcd workgroups

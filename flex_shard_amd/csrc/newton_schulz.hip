@@ -392,7 +392,18 @@ constexpr int kDmaGemmLdsBytes =
 // their way into stage 0.  The schedule is static, so the host uses it only
 // when all tiles of the launch are equally long; otherwise each id is its own
 // workgroup and the hardware hands them out as compute units come free.
-template <bool kPersistent>
+//
+// kKMajor: both operands are given k-major, A as [K, M] and B as [K, N] (row
+// strides lda / ldb), i.e. the product is A^T B.  A k-tile of an operand is
+// then 64 rows of 512 bytes.  It lands in LDS as it is (chunk c of k-row r in
+// slot c ^ 4 (r & 3)), and the fragments come out of it through the
+// transposing LDS read of gfx950 (ds_read_b64_tr_b16): within 16 lanes, lane
+// 4 j + q passes the address of four consecutive columns 4 q .. 4 q + 3 of
+// k-row j, and lane t receives column t of k-rows 0 .. 3 -- four consecutive
+// k of one output row, half of an MFMA operand.  The products and their order
+// are those of the k-contiguous form on the transposed operands, so the
+// results are bit-identical.
+template <bool kPersistent, bool kKMajor>
 __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const GemmLaunch launch) {
   using Cfg = DmaGemm;
 #ifdef FSH_TRACE
@@ -426,30 +437,42 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
 
   // Load side.  Wave-level load q (0..7) of this wave fills tile rows
   // [32 q + 8 wave, +8); lane l fills slot l & 7 of row l >> 3 there.
-  const int fill_row = lane >> 3;
-  const int fill_chunk = (lane & 7) ^ (((8 * wave + fill_row) >> 1) & 7);
+  // (k-major: load q fills k-rows [8 q + 2 wave, +2); lane l fills slot
+  // l & 31 of row l >> 5 there.)
+  const int fill_row = kKMajor ? lane >> 5 : lane >> 3;
+  const uint32_t fill_row0 = static_cast<uint32_t>((kKMajor ? 2 : 8) * wave + fill_row);
+  const int fill_chunk = kKMajor ? (lane & 31) ^ (4 * static_cast<int>(fill_row0 & 3))
+                                 : (lane & 7) ^ static_cast<int>((fill_row0 >> 1) & 7);
+  constexpr uint32_t kRowsPerLoadStep = kKMajor ? 8 : 32;
   // M0 takes the LDS byte address relative to the workgroup's allocation.
   typedef __attribute__((address_space(3))) uint8_t* lds_address;
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_address)lds_bytes));
   const uint32_t fill_lds = lds_base + static_cast<uint32_t>(wave * 1024);  // + q * 4096 (+ operand, + stage)
-  const uint32_t fill_row0 = static_cast<uint32_t>(8 * wave + fill_row);
   // Operand tile bases of (problem, batch, tile row / column), k-tile 0.
   auto a_base = [&](int which, int64_t batch, int tm) -> const uint8_t* {
     const GemmParams& q = launch.problem[which];
-    return uniform_ptr(reinterpret_cast<const uint8_t*>(q.A + batch * q.sA + static_cast<int64_t>(tm) * Cfg::BM * q.lda));
+    return uniform_ptr(reinterpret_cast<const uint8_t*>(
+        q.A + batch * q.sA + static_cast<int64_t>(tm) * Cfg::BM * (kKMajor ? 1 : q.lda)));
   };
   auto b_base = [&](int which, int64_t batch, int tn) -> const uint8_t* {
     const GemmParams& q = launch.problem[which];
-    return uniform_ptr(reinterpret_cast<const uint8_t*>(q.B + batch * q.sB + static_cast<int64_t>(tn) * Cfg::BN * q.ldb));
+    return uniform_ptr(reinterpret_cast<const uint8_t*>(
+        q.B + batch * q.sB + static_cast<int64_t>(tn) * Cfg::BN * (kKMajor ? 1 : q.ldb)));
   };
   auto issue_tile_load = [&](const uint8_t* a_src, const uint8_t* b_src, uint32_t a_row_bytes, uint32_t b_row_bytes,
                              int stage_off, int q_first, int q_last) {
 #pragma unroll
     for (int q = q_first; q < q_last; ++q) {
-      dma_load_16((fill_row0 + 32 * q) * a_row_bytes + fill_chunk * 16, a_src, stage_off + fill_lds + q * 4096);
-      dma_load_16((fill_row0 + 32 * q) * b_row_bytes + fill_chunk * 16, b_src,
+      dma_load_16((fill_row0 + kRowsPerLoadStep * q) * a_row_bytes + fill_chunk * 16, a_src,
+                  stage_off + fill_lds + q * 4096);
+      dma_load_16((fill_row0 + kRowsPerLoadStep * q) * b_row_bytes + fill_chunk * 16, b_src,
                   stage_off + Cfg::kOperandBytes + fill_lds + q * 4096);
     }
+  };
+
+  // Operand pointer of k-tile kt: 128 bytes along the rows, or 64 rows down.
+  auto k_tile_ptr = [&](const uint8_t* base, uint32_t row_bytes, int64_t kt) -> const uint8_t* {
+    return kKMajor ? base + kt * (static_cast<int64_t>(Cfg::BK) * row_bytes) : base + kt * Cfg::kRowBytes;
   };
 
   // Fragment side.  Lane l reads row l & 31 of a 32-row block, k chunk
@@ -464,15 +487,42 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
     a_frag[ks] = (frag_base ^ (ks * 32)) + wm * Cfg::kWaveM * Cfg::kRowBytes;
     b_frag[ks] = (frag_base ^ (ks * 32)) + Cfg::kOperandBytes + wn * Cfg::kWaveN * Cfg::kRowBytes;
   }
+  // k-major fragments: lane l = 16 g + t of a wave serves output row
+  // 16 (g & 1) + t of a 32-row block and the k octet g >> 1 of a k step; it
+  // passes the address of columns 4 (t & 3) .. + 3 of k-row (t >> 2) of its
+  // octet's first half, then of its second half (4 rows = 2048 bytes down).
+  // The block index enters the slot through the swizzle: i ^ (k-row & 3).
+  uint32_t a_frag_km[TM], b_frag_km[TN];
+  {
+    const int t = lane & 15, g = lane >> 4;
+    const uint32_t common = static_cast<uint32_t>(((g >> 1) * 8 + (t >> 2)) * 512 + (g & 1) * 32 + (t & 3) * 8);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a_frag_km[i] = common + wm * 256 + ((i ^ (t >> 2)) * 64);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) b_frag_km[j] = Cfg::kOperandBytes + common + wn * 256 + ((j ^ (t >> 2)) * 64);
+  }
   constexpr int scrap_offset = kDmaGemmLdsBytes - Cfg::kScrapBytes;
 
   f32x16 acc[TM][TN];
   bf16x8 af[2][TM], bf[2][TN];
+  auto read_transposed = [&](uint32_t offset) -> bf16x8 {
+    typedef short i16x4 __attribute__((__vector_size__(4 * sizeof(short))));
+    typedef __attribute__((address_space(3))) i16x4* lds_i16x4;
+    const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4)(lds_bytes + offset));
+    const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4)(lds_bytes + offset + 2048));
+    return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
   auto read_a = [&](int set, int stage_off, int ks, int i) {
-    af[set][i] = *reinterpret_cast<const bf16x8*>(lds_bytes + stage_off + a_frag[ks] + i * 32 * Cfg::kRowBytes);
+    if (kKMajor)
+      af[set][i] = read_transposed(stage_off + a_frag_km[i] + ks * 8192);
+    else
+      af[set][i] = *reinterpret_cast<const bf16x8*>(lds_bytes + stage_off + a_frag[ks] + i * 32 * Cfg::kRowBytes);
   };
   auto read_b = [&](int set, int stage_off, int ks, int j) {
-    bf[set][j] = *reinterpret_cast<const bf16x8*>(lds_bytes + stage_off + b_frag[ks] + j * 32 * Cfg::kRowBytes);
+    if (kKMajor)
+      bf[set][j] = read_transposed(stage_off + b_frag_km[j] + ks * 8192);
+    else
+      bf[set][j] = *reinterpret_cast<const bf16x8*>(lds_bytes + stage_off + b_frag[ks] + j * 32 * Cfg::kRowBytes);
   };
   auto read_frags = [&](int set, int stage_off, int ks) {
 #pragma unroll
@@ -519,7 +569,9 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   // B = two requests per wave) into a scrap area, which brings the lines into
   // L2 early.  They are issued after the real requests and may still be in
   // flight when those are waited for (requests complete in order).
-  const uint32_t touch_row = static_cast<uint32_t>(64 * wave + lane);
+  // (k-major: 64 rows of four lines each; thread t asks for line t & 3 of row t >> 2.)
+  const uint32_t touch_row = static_cast<uint32_t>(kKMajor ? (64 * wave + lane) >> 2 : 64 * wave + lane);
+  const uint32_t touch_col = static_cast<uint32_t>(kKMajor ? (lane & 3) * 128 : 0);
   const uint32_t scrap_lds = lds_base + static_cast<uint32_t>(scrap_offset + wave * 256);
   auto k_tile = [&](int64_t kt, int64_t ktiles, auto more_tag) {
     constexpr bool more = decltype(more_tag)::value;
@@ -532,7 +584,7 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
       for (int g = 0; g < TM * TN; ++g) mfma(ks & 1, g / TN, g % TN);
 #pragma unroll
       for (int g = 0; g < TM + TN; ++g) {
-        __builtin_amdgcn_sched_group_barrier(kSchedDsRead, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(kSchedDsRead, kKMajor ? 2 : 1, 0);
         __builtin_amdgcn_sched_group_barrier(kSchedMfma, TM * TN / (TM + TN), 0);
       }
     }
@@ -543,8 +595,8 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
     }
     __syncthreads();
     const bool more2 = more && kt + 2 < ktiles;
-    const uint8_t* a_next = Ab + (kt + 2) * Cfg::kRowBytes;
-    const uint8_t* b_next = Bb + (kt + 2) * Cfg::kRowBytes;
+    const uint8_t* a_next = k_tile_ptr(Ab, a_row_bytes, kt + 2);
+    const uint8_t* b_next = k_tile_ptr(Bb, b_row_bytes, kt + 2);
 #pragma unroll
     for (int g = 0; g < TM * TN; ++g) {
       mfma((KS - 1) & 1, g / TN, g % TN);
@@ -556,8 +608,8 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
       __builtin_amdgcn_sched_barrier(0);
     }
     if (more2 && kt + 1 + Cfg::kTouchAhead < ktiles) {
-      dma_touch_4(touch_row * a_row_bytes, Ab + (kt + 1 + Cfg::kTouchAhead) * Cfg::kRowBytes, scrap_lds);
-      dma_touch_4(touch_row * b_row_bytes, Bb + (kt + 1 + Cfg::kTouchAhead) * Cfg::kRowBytes, scrap_lds);
+      dma_touch_4(touch_row * a_row_bytes + touch_col, k_tile_ptr(Ab, a_row_bytes, kt + 1 + Cfg::kTouchAhead), scrap_lds);
+      dma_touch_4(touch_row * b_row_bytes + touch_col, k_tile_ptr(Bb, b_row_bytes, kt + 1 + Cfg::kTouchAhead), scrap_lds);
     }
   };
 
@@ -576,8 +628,8 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
     __syncthreads();  // also: every wave has left the previous tile's epilogue
     read_frags(0, 0, 0);
     if (ktiles > 1)
-      issue_tile_load(Ab + Cfg::kRowBytes, Bb + Cfg::kRowBytes, a_row_bytes, b_row_bytes, Cfg::kStageBytes, 0,
-                      Cfg::kLoadsPerOperand);
+      issue_tile_load(k_tile_ptr(Ab, a_row_bytes, 1), k_tile_ptr(Bb, b_row_bytes, 1), a_row_bytes, b_row_bytes,
+                      Cfg::kStageBytes, 0, Cfg::kLoadsPerOperand);
     FSH_STAMP(2);
 
     for (int64_t kt = 0; kt + 1 < ktiles; ++kt) k_tile(kt, ktiles, std::true_type{});
@@ -649,6 +701,10 @@ int plan_gemm_cfg(PlannedGemm* plan, int64_t batch) {
     plan->kind = big ? kKernelDma : kKernelInteriorSmall;
   else
     plan->kind = big ? kKernelEdgeBig : kKernelEdgeSmall;
+  if (p.k_major && plan->kind != kKernelDma)
+    return fail(FSH_ENOTSUP,
+                "gemm: k-major operands need whole 256 x 256 x 64 tiles and at least 192 of them (m %lld, n %lld, "
+                "k %lld, batch %lld)", (long long)p.M, (long long)p.N, (long long)p.K, (long long)batch);
   return FSH_OK;
 }
 
@@ -660,13 +716,16 @@ int plan_gemm(const fsh_gemm_desc& d, PlannedGemm* plan) {
   if (d.k % 8 || d.lda % 8 || d.ldb % 8 || d.stride_a % 8 || d.stride_b % 8 || !aligned(d.a_dev, 16) ||
       !aligned(d.b_dev, 16))
     return fail(FSH_ENOTSUP, "gemm: k, lda, ldb and batch strides must be multiples of 8 and A, B 16-byte aligned");
-  if (d.lda < d.k || d.ldb < d.k || d.ldc < d.n || (d.d_dev && d.ldd < d.n) || (d.ct_dev && d.ldct < d.m))
+  // k-contiguous operands have rows of k elements; k-major ones rows of m and of n.
+  if (d.lda < (d.k_major ? d.m : d.k) || d.ldb < (d.k_major ? d.n : d.k) || d.ldc < d.n || (d.d_dev && d.ldd < d.n) ||
+      (d.ct_dev && d.ldct < d.m))
     return fail(FSH_EINVAL, "gemm: leading dimension smaller than the row length");
   if (d.symmetric && (d.m != d.n || d.ct_dev != nullptr))
     return fail(FSH_EINVAL, "gemm: a symmetric product needs m == n and no transposed output");
   GemmParams& p = plan->p;
   memset(&p, 0, sizeof(p));
   p.symmetric = d.symmetric ? 1 : 0;
+  p.k_major = d.k_major ? 1 : 0;
   p.A = static_cast<const uint16_t*>(d.a_dev);
   p.B = static_cast<const uint16_t*>(d.b_dev);
   p.D = static_cast<const uint16_t*>(d.d_dev);
@@ -714,7 +773,8 @@ int launch_single(Kernel kernel, LdsReservation* reserved, int lds_bytes, int th
 // round of another instead of each launch paying its own tail.  The problems
 // of one call must not depend on each other.
 int launch_planned(PlannedGemm* plans, int count, hipStream_t stream) {
-  static LdsReservation reserved_dma, reserved_persistent, reserved_small, reserved_edge_big, reserved_edge_small;
+  static LdsReservation reserved_dma, reserved_persistent, reserved_dma_km, reserved_persistent_km, reserved_small,
+      reserved_edge_big, reserved_edge_small;
   constexpr int kDmaLds = kDmaGemmLdsBytes;
   int i = 0;
   while (i < count) {
@@ -737,7 +797,8 @@ int launch_planned(PlannedGemm* plans, int count, hipStream_t stream) {
     int order[kMaxGemmProblems];
     int n = 0;
     int64_t total = 0;
-    while (i < count && n < kMaxGemmProblems && plans[i].kind == kKernelDma &&
+    const int k_major = plans[i].p.k_major;  // one operand layout per launch
+    while (i < count && n < kMaxGemmProblems && plans[i].kind == kKernelDma && plans[i].p.k_major == k_major &&
            total + plans[i].workgroups <= 0x3FFFFFFFLL) {
       total += plans[i].workgroups;
       order[n++] = i++;
@@ -764,14 +825,20 @@ int launch_planned(PlannedGemm* plans, int count, hipStream_t stream) {
     bool equal_k = true;
     for (int k = 1; k < n; ++k) equal_k = equal_k && plans[order[k]].p.K == plans[order[0]].p.K;
     const int64_t units = compute_units();
-    if (equal_k && units >= kXcds && units % kXcds == 0 && total > units) {
-      if (int rc = reserve_lds_once(reserved_persistent, &gemm_nt_dma_kernel<true>, kDmaLds)) return rc;
-      hipLaunchKernelGGL(gemm_nt_dma_kernel<true>, dim3(static_cast<uint32_t>(units)), dim3(DmaGemm::kThreads),
-                         kDmaLds, stream, launch);
+    const bool resident = equal_k && units >= kXcds && units % kXcds == 0 && total > units;
+    const dim3 grid(static_cast<uint32_t>(resident ? units : total)), block(DmaGemm::kThreads);
+    if (resident && k_major) {
+      if (int rc = reserve_lds_once(reserved_persistent_km, &gemm_nt_dma_kernel<true, true>, kDmaLds)) return rc;
+      hipLaunchKernelGGL((gemm_nt_dma_kernel<true, true>), grid, block, kDmaLds, stream, launch);
+    } else if (resident) {
+      if (int rc = reserve_lds_once(reserved_persistent, &gemm_nt_dma_kernel<true, false>, kDmaLds)) return rc;
+      hipLaunchKernelGGL((gemm_nt_dma_kernel<true, false>), grid, block, kDmaLds, stream, launch);
+    } else if (k_major) {
+      if (int rc = reserve_lds_once(reserved_dma_km, &gemm_nt_dma_kernel<false, true>, kDmaLds)) return rc;
+      hipLaunchKernelGGL((gemm_nt_dma_kernel<false, true>), grid, block, kDmaLds, stream, launch);
     } else {
-      if (int rc = reserve_lds_once(reserved_dma, &gemm_nt_dma_kernel<false>, kDmaLds)) return rc;
-      hipLaunchKernelGGL(gemm_nt_dma_kernel<false>, dim3(static_cast<uint32_t>(total)), dim3(DmaGemm::kThreads),
-                         kDmaLds, stream, launch);
+      if (int rc = reserve_lds_once(reserved_dma, &gemm_nt_dma_kernel<false, false>, kDmaLds)) return rc;
+      hipLaunchKernelGGL((gemm_nt_dma_kernel<false, false>), grid, block, kDmaLds, stream, launch);
     }
     if (int rc = check_launch("gemm_nt_dma_kernel")) return rc;
   }
@@ -826,7 +893,8 @@ __global__ __launch_bounds__(kNormThreads) void sumsq_partial_kernel(const uint1
 
 // Reads matrix b of `in` ([rows, cols]), divides by max(||.||_F, eps) as bf16
 // tensor ops would (norm rounded to bf16, fp32 division, bf16 result), and
-// writes the result to `out_same` ([rows, cols]) and `out_t` ([cols, rows]).
+// writes the result to `out_same` ([rows, cols]) and `out_t` ([cols, rows]);
+// either output may be null.
 // A workgroup owns a 64x64 tile: 16-byte loads and stores of 8 elements along
 // the rows, and for the transposed copy the tile goes through LDS and leaves
 // as 16-byte stores of 8 elements along the columns.  rows and cols are
@@ -846,8 +914,8 @@ __global__ __launch_bounds__(kNormThreads) void normalize_dual_kernel(const uint
   norm = norm < eps_bf16 ? eps_bf16 : norm;
   const int64_t r0 = static_cast<int64_t>(blockIdx.y) * kNormTile, c0 = static_cast<int64_t>(blockIdx.x) * kNormTile;
   const uint16_t* m = in + b * rows * cols;
-  uint16_t* o = out_same + b * rows * cols;
-  uint16_t* ot = out_t + b * rows * cols;
+  uint16_t* o = out_same ? out_same + b * rows * cols : nullptr;
+  uint16_t* ot = out_t ? out_t + b * rows * cols : nullptr;
   const int q = threadIdx.x & 7, line = threadIdx.x >> 3;  // 8 groups of 8 elements per line, 32 lines per pass
 #pragma unroll
   for (int pass = 0; pass < 2; ++pass) {
@@ -862,13 +930,15 @@ __global__ __launch_bounds__(kNormThreads) void normalize_dual_kernel(const uint
         bits[2 * j] = f32_to_bf16_bits(u32_as_f32(d[j] << 16) / norm);
         bits[2 * j + 1] = f32_to_bf16_bits(u32_as_f32(d[j] & 0xFFFF0000u) / norm);
       }
-      store_stream_u32x4(o + r * cols + c, u32x4{bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16),
-                                                   bits[4] | (bits[5] << 16), bits[6] | (bits[7] << 16)});
+      if (o != nullptr)
+        store_stream_u32x4(o + r * cols + c, u32x4{bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16),
+                                                     bits[4] | (bits[5] << 16), bits[6] | (bits[7] << 16)});
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         *reinterpret_cast<uint32_t*>(&tile[lr * kNormPitch + 8 * q + 2 * j]) = bits[2 * j] | (bits[2 * j + 1] << 16);
     }
   }
+  if (ot == nullptr) return;  // the same for the whole workgroup
   __syncthreads();
 #pragma unroll
   for (int pass = 0; pass < 2; ++pass) {
@@ -936,7 +1006,8 @@ struct NsState {
   uint16_t* G;
   uint16_t* P;
   int cur;
-  bool tall;  // the caller's matrix is X^T
+  bool tall;    // the caller's matrix is X^T
+  bool single;  // only X^T is carried from step to step (G = X X^T is then computed from its k-major rows)
 };
 
 int ns_begin(const fsh_ns_problem& q, int32_t steps, float eps, hipStream_t stream, NsState* st) {
@@ -968,9 +1039,15 @@ int ns_begin(const fsh_ns_problem& q, int32_t steps, float eps, hipStream_t stre
   st->G = reinterpret_cast<uint16_t*>(ws + 2 * align256(batch * sl * 2));
   st->P = reinterpret_cast<uint16_t*>(ws + 2 * align256(batch * sl * 2) + align256(batch * ss * 2));
   float* partial = reinterpret_cast<float*>(ws + 2 * align256(batch * sl * 2) + 2 * align256(batch * ss * 2));
+  // With whole 256 x 256 x 64 tiles, and enough of them for the large-tile
+  // kernel, G = X X^T is computed from X^T as it lies (k-major operands), so
+  // X itself is never written: a tall input alternates between the caller's
+  // buffer and one workspace buffer, a wide one between the two workspace
+  // buffers and its last step writes X' = P X into the caller's buffer.
+  st->single = steps > 0 && s % 256 == 0 && l % 64 == 0 && (s / 256) * (s / 256 + 1) / 2 * batch >= 192;
   st->X = tall ? w0 : x;
   st->XT[0] = tall ? x : w0;
-  st->XT[1] = w1;
+  st->XT[1] = (st->single && tall) ? w0 : w1;
   st->cur = steps & 1;
   st->tall = tall;
 
@@ -981,6 +1058,7 @@ int ns_begin(const fsh_ns_problem& q, int32_t steps, float eps, hipStream_t stre
   // and X^T for a tall one.
   uint16_t* same = tall ? st->XT[st->cur] : st->X;
   uint16_t* transposed = tall ? st->X : st->XT[st->cur];
+  if (st->single) (tall ? transposed : same) = nullptr;
   const dim3 grid(static_cast<uint32_t>(ceil_div(cols, (int64_t)kNormTile)),
                   static_cast<uint32_t>(ceil_div(rows, (int64_t)kNormTile)), static_cast<uint32_t>(batch));
   if (grid.y > 65535) return fail(FSH_ENOTSUP, "newton_schulz: more than %d row tiles", 65535 * kNormTile);
@@ -991,7 +1069,9 @@ int ns_begin(const fsh_ns_problem& q, int32_t steps, float eps, hipStream_t stre
 
 // The three products of one iteration; `which` = 0: G = X X^T, 1: P = a I +
 // b G + c G G (symmetric because G is), 2: X' = P X = a X + (b G + c G G) X,
-// also written transposed into the other X^T buffer.  Carrying `a` on P's
+// also written transposed into the other X^T buffer -- or, when only X^T is
+// carried, X'^T = X^T P alone, with G read from the k-major rows of X^T and
+// the last step of a wide input written as X' = P X.  Carrying `a` on P's
 // diagonal (added in fp32 before P is rounded) spares the last product a
 // read of X from HBM per output tile.  The last step of the iteration writes
 // only the orientation the caller holds: X' for a wide input, and for a tall
@@ -1001,7 +1081,14 @@ fsh_gemm_desc ns_product(const NsState& st, int which, float a, float b, float c
   fsh_gemm_desc g;
   memset(&g, 0, sizeof(g));
   g.batch = st.batch;
-  if (which == 0) {
+  if (which == 0 && st.single) {
+    g.a_dev = st.XT[st.cur]; g.b_dev = st.XT[st.cur]; g.c_dev = st.G;
+    g.m = s; g.n = s; g.k = l; g.lda = s; g.ldb = s; g.ldc = s;
+    g.stride_a = sl; g.stride_b = sl; g.stride_c = ss;
+    g.alpha = 1.0f; g.beta = 0.0f;
+    g.symmetric = 1;
+    g.k_major = 1;
+  } else if (which == 0) {
     g.a_dev = st.X; g.b_dev = st.X; g.c_dev = st.G;
     g.m = s; g.n = s; g.k = l; g.lda = l; g.ldb = l; g.ldc = s;
     g.stride_a = sl; g.stride_b = sl; g.stride_c = ss;
@@ -1014,13 +1101,15 @@ fsh_gemm_desc ns_product(const NsState& st, int which, float a, float b, float c
     g.alpha = c; g.beta = b;
     g.diag_add = a;
     g.symmetric = 1;
-  } else if (last_step && st.tall) {
+  } else if (st.single ? (st.tall || !last_step) : (last_step && st.tall)) {
+    // X'^T = X^T P (P is symmetric), the orientation that is carried
     g.a_dev = st.XT[st.cur]; g.b_dev = st.P; g.c_dev = st.XT[st.cur ^ 1];
     g.m = l; g.n = s; g.k = s; g.lda = s; g.ldb = s; g.ldc = s;
     g.stride_a = sl; g.stride_b = ss; g.stride_c = sl;
     g.alpha = 1.0f; g.beta = 0.0f;
   } else {
-    g.a_dev = st.P; g.b_dev = st.XT[st.cur]; g.c_dev = st.X; g.ct_dev = last_step ? nullptr : st.XT[st.cur ^ 1];
+    g.a_dev = st.P; g.b_dev = st.XT[st.cur]; g.c_dev = st.X;
+    g.ct_dev = (last_step || st.single) ? nullptr : st.XT[st.cur ^ 1];
     g.m = s; g.n = l; g.k = s; g.lda = s; g.ldb = s; g.ldc = l; g.ldct = s;
     g.stride_a = ss; g.stride_b = sl; g.stride_c = sl; g.stride_ct = sl;
     g.alpha = 1.0f; g.beta = 0.0f;

@@ -356,16 +356,23 @@ def newton_schulz_multi(
 def _gemm_desc(
     a: torch.Tensor, b: torch.Tensor, d: torch.Tensor | None, alpha: float, beta: float,
     out: torch.Tensor | None, out_t: torch.Tensor | None, symmetric: bool, diag_add: float = 0.0,
+    k_major: bool = False,
 ) -> tuple["_native.GemmDesc", torch.Tensor]:
     _require_gpu(a, b)
     if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16 or not a.is_contiguous() or not b.is_contiguous():
         raise ValueError("a and b must be contiguous bf16")
     a3 = a if a.ndim == 3 else a.unsqueeze(0)
     b3 = b if b.ndim == 3 else b.unsqueeze(0)
-    batch, m, k = a3.shape
-    if b3.shape[0] != batch or b3.shape[2] != k:
-        raise ValueError(f"shape mismatch: a {tuple(a.shape)} vs b {tuple(b.shape)}")
-    n = b3.shape[1]
+    if k_major:  # [batch, k, m] and [batch, k, n]
+        batch, k, m = a3.shape
+        if b3.shape[0] != batch or b3.shape[1] != k:
+            raise ValueError(f"shape mismatch: a {tuple(a.shape)} vs b {tuple(b.shape)}")
+        n = b3.shape[2]
+    else:
+        batch, m, k = a3.shape
+        if b3.shape[0] != batch or b3.shape[2] != k:
+            raise ValueError(f"shape mismatch: a {tuple(a.shape)} vs b {tuple(b.shape)}")
+        n = b3.shape[1]
     if out is None:
         out = torch.empty((batch, m, n) if a.ndim == 3 else (m, n), dtype=torch.bfloat16, device=a.device)
     for name, t, shape in (("d", d, (m, n)), ("out", out, (m, n)), ("out_t", out_t, (n, m))):
@@ -380,26 +387,30 @@ def _gemm_desc(
     desc.c_dev = out.data_ptr()
     desc.ct_dev = out_t.data_ptr() if out_t is not None else None
     desc.m, desc.n, desc.k = m, n, k
-    desc.lda, desc.ldb, desc.ldd, desc.ldc, desc.ldct = k, k, n, n, m
+    desc.lda, desc.ldb = (m, n) if k_major else (k, k)
+    desc.ldd, desc.ldc, desc.ldct = n, n, m
     desc.batch = batch
     desc.stride_a, desc.stride_b = m * k, n * k
     desc.stride_d = desc.stride_c = desc.stride_ct = m * n
     desc.alpha, desc.beta = alpha, beta
     desc.symmetric = 1 if symmetric else 0
     desc.diag_add = diag_add
+    desc.k_major = 1 if k_major else 0
     return desc, out
 
 
 def gemm_nt(
     a: torch.Tensor, b: torch.Tensor, *, d: torch.Tensor | None = None, alpha: float = 1.0, beta: float = 0.0,
     out: torch.Tensor | None = None, out_t: torch.Tensor | None = None, symmetric: bool = False,
-    diag_add: float = 0.0,
+    diag_add: float = 0.0, k_major: bool = False,
 ) -> torch.Tensor:
     """``bf16(alpha * a @ b^T + beta * d + diag_add * I)`` for contiguous bf16
     [batch, m, k] / [batch, n, k] (or 2-D) operands; optionally also the
     transpose.  With ``symmetric`` the caller guarantees a symmetric result
-    (m == n); only the upper triangle of tiles is computed and mirrored."""
-    desc, out = _gemm_desc(a, b, d, alpha, beta, out, out_t, symmetric, diag_add)
+    (m == n); only the upper triangle of tiles is computed and mirrored.  With
+    ``k_major`` the operands are [batch, k, m] / [batch, k, n] and the product
+    is ``a^T @ b`` (large whole-tile problems only)."""
+    desc, out = _gemm_desc(a, b, d, alpha, beta, out, out_t, symmetric, diag_add, k_major)
     status = _native.lib().fsh_gemm_bf16_nt(ctypes.byref(desc), stream_ptr(a.device))
     _native.check(status, "fsh_gemm_bf16_nt")
     return out
@@ -415,7 +426,7 @@ def gemm_nt_group(problems: Sequence[dict]) -> list[torch.Tensor]:
     for i, q in enumerate(problems):
         desc, out = _gemm_desc(
             q["a"], q["b"], q.get("d"), q.get("alpha", 1.0), q.get("beta", 0.0), q.get("out"), q.get("out_t"),
-            q.get("symmetric", False), q.get("diag_add", 0.0),
+            q.get("symmetric", False), q.get("diag_add", 0.0), q.get("k_major", False),
         )
         descs[i] = desc
         outs.append(out)

@@ -225,6 +225,11 @@ typedef struct fsh_gemm_desc {
                         and d symmetric); only the tiles on or above the diagonal are
                         computed and the rest is mirrored.  ct_dev must be null. */
   float diag_add;    /* added to C[b][i][i] in fp32 before the rounding to bf16 (0: plain product) */
+  int32_t k_major;   /* nonzero: A is [k, m] and B is [k, n] (row strides lda / ldb), so the product
+                        is A^T . B; same products in the same order as the k-contiguous form on
+                        the transposed operands.  Needs m, n multiples of 256, k of 64, and at
+                        least 192 tiles of 256 x 256 in all. */
+  int32_t reserved;  /* zero */
 } fsh_gemm_desc;
 int fsh_gemm_bf16_nt(const fsh_gemm_desc* desc, void* stream);
 /* `count` independent products; those that qualify for the large-tile kernel

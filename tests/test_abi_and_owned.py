@@ -44,7 +44,7 @@ def test_library_exports_every_declared_symbol():
 def test_struct_sizes_match_the_header():
     assert ctypes.sizeof(_native.QuantChunk) == 56
     assert ctypes.sizeof(_native.UnpackChunk) == 56
-    assert ctypes.sizeof(_native.GemmDesc) == 5 * 8 + 14 * 8 + 2 * 4 + 2 * 4
+    assert ctypes.sizeof(_native.GemmDesc) == 5 * 8 + 14 * 8 + 2 * 4 + 2 * 4 + 2 * 4
 
 
 def test_host_side_argument_checks_need_no_gpu():
