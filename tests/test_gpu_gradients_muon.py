@@ -362,6 +362,57 @@ def test_newton_schulz_matches_torch_muon_routine(device, shape, golden):
         assert (mine.view(-1, *shape[-2:])[0].float() - small.float()).abs().max().item() <= tol
 
 
+@pytest.mark.parametrize("shape,steps", [((20, 1024, 1280), 5), ((20, 1280, 1024), 5), ((24, 1024, 1024), 4), ((20, 1280, 1024), 1)])
+def test_newton_schulz_with_one_orientation_carried(device, shape, steps, golden):
+    """Batches with whole 256 x 256 x 64 tiles and at least 192 of them carry
+    only X^T between steps (G from its k-major rows; a wide input's last step
+    written as X' = P X): wide, tall and square inputs, odd, even and single
+    step counts, first and last matrix against torch's routine."""
+    from torch.optim._muon import _zeropower_via_newtonschulz as torch_ns
+
+    tol = golden["muon_tolerance"]["atol"]
+    gen = torch.Generator().manual_seed(8)
+    g = torch.randn(shape, generator=gen).bfloat16()
+    keep = g.clone()
+    on_gpu = g.to(device)
+    mine = _zeropower_via_newtonschulz(on_gpu, ns_steps=steps).cpu()
+    assert torch.equal(on_gpu.cpu(), keep)
+    for index in (0, shape[0] - 1):
+        ref = torch_ns(g[index], COEFFS, steps, 1e-7)
+        assert (mine[index].float() - ref.float()).abs().max().item() <= tol
+    # every matrix of the batch went through the same launches: same result for equal inputs
+    twice = torch.stack([g[0], g[0]] * (shape[0] // 2)).contiguous().to(device)
+    out = _zeropower_via_newtonschulz(twice, ns_steps=steps)
+    assert torch.equal(out[0], out[1]) and torch.equal(out[0], out[-1]) and torch.equal(out[0].cpu(), mine[0])
+
+
+@pytest.mark.parametrize("batch,m,n,k,symmetric", [(3, 2048, 2048, 320, False), (6, 2048, 2048, 448, True), (1, 4096, 3584, 64, False)])
+def test_gemm_k_major_equals_the_k_contiguous_form(device, batch, m, n, k, symmetric):
+    """Operands given as [k, m] and [k, n]: the fragments come out of LDS
+    through the transposing read, the products and their order are those of
+    the k-contiguous form on the transposed operands -- bit-identical."""
+    gen = torch.Generator().manual_seed(9)
+    a_km = torch.randn(batch, k, m, generator=gen).bfloat16().to(device)
+    b_km = a_km if symmetric else torch.randn(batch, k, n, generator=gen).bfloat16().to(device)
+    a_nt, b_nt = a_km.transpose(1, 2).contiguous(), b_km.transpose(1, 2).contiguous()
+    want = hip_ops.gemm_nt(a_nt, b_nt, symmetric=symmetric)
+    got = hip_ops.gemm_nt(a_km, b_km, symmetric=symmetric, k_major=True)
+    assert torch.equal(got, want)
+    ref = torch.bmm(a_nt.float(), b_nt.float().transpose(1, 2))
+    assert ((got.float() - ref).abs().max() / ref.abs().max()).item() < 5e-3
+    if symmetric:
+        assert torch.equal(got, got.transpose(1, 2))
+
+
+def test_gemm_k_major_needs_the_large_tile_kernel(device):
+    a = torch.randn(1, 64, 256, device=device).bfloat16()
+    with pytest.raises(RuntimeError, match="k-major operands need whole 256 x 256 x 64 tiles"):
+        hip_ops.gemm_nt(a, a, k_major=True)  # one tile
+    b = torch.randn(3, 64, 2048 + 8, device=device).bfloat16()
+    with pytest.raises(RuntimeError, match="k-major operands need whole 256 x 256 x 64 tiles"):
+        hip_ops.gemm_nt(b, b, k_major=True)  # ragged tiles
+
+
 def test_newton_schulz_leaves_its_input_untouched_and_handles_zero(device):
     g = torch.randn(128, 128, device=device).bfloat16()
     keep = g.clone()
