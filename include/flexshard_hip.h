@@ -205,7 +205,8 @@ int fsh_newton_schulz_multi(const fsh_ns_problem* problems, int32_t count, float
 /* Batched bf16 "NT" GEMM, the building block of (6), exported for tests:
  *   C[b] = bf16(alpha * A[b] . B[b]^T + beta * D[b] + diag_add * I)   fp32 accumulation
  * A is [m, k] with row stride lda, B is [n, k] with row stride ldb (both
- * k-contiguous), D and C are [m, n] with row strides ldd / ldc.  D may be NULL
+ * k-contiguous; see k_major for the other layout), D and C are [m, n] with
+ * row strides ldd / ldc.  D may be NULL
  * (beta ignored) or alias C.  ct_dev, when not NULL, also receives C[b]^T as
  * an [n, m] matrix with row stride ldct.  Batch strides are in elements.
  * k and all leading dimensions must be multiples of 8 and all pointers
