@@ -364,10 +364,11 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_nt_interior_kernel(const G
 // reorders nor counts; everything else in the loop is compiler-visible and is
 // pinned around them with sched_barrier.
 //
-// The chip is power-limited in this kernel (the shader clock settles near
-// 1.2-1.4 GHz under sustained MFMA load), so what counts is data moved per
-// MFMA, not latency hiding: warming L2 with early touches of later k-tiles
-// was measured and bought nothing.
+// The part does not hold its peak clock under this kernel (about 1.65 GHz by
+// the MFMA-busy counters against the delivered rate).  Operand requests
+// complete in order, so a k-tile waits for its slowest line: kTouchAhead
+// k-tiles ahead every line of both operand tiles is asked for once (4 bytes
+// into a scrap area), which brings it into L2 before the real request.
 struct DmaGemm {
   static constexpr int BM = 256, BN = 256, BK = 64, WM = 2, WN = 2, TM = 4, TN = 4;
   static constexpr int kThreads = 256, kWaveM = 128, kWaveN = 128, KS = BK / 16;
