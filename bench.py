@@ -4,16 +4,19 @@
 Headline: fused FP8 tile quantize + pack of one rank's share (rank 0 of 8) of a
 Llama-3-8B layer bucket: q, k, v and the first 512 rows of o = 27 262 976 bf16
 elements in 4 chunks, packed into a 27 531 840-byte payload.  A step is one
-such launch on one layer's shards; steps rotate over `--layers` distinct layer
-buckets so the inputs come from HBM, not from the 256 MB last-level cache.
-`value` is algorithmic bytes moved per second over the whole timed region,
-inputs resident in HBM.
+pass over `--layers` distinct layer buckets, one such launch per layer (what a
+training step does with the layers of a model), so the inputs of every launch
+come from HBM, not from the 256 MB last-level cache.  Before anything is
+timed, every layer bucket is packed twice (launch tables cached, allocator
+blocks in place), whatever `--warmup` says.  `value` is algorithmic bytes moved
+per second over the whole timed region, inputs resident in HBM.
 
 One JSON line is printed.  Besides the contract fields it carries
   roofline      the dominant kernel against the 8 TB/s HBM peak, timed with
                 events on the launch stream over the same timed region
   cpu_baseline  the oracle's eager-torch restatement of the reference path on
-                the host cores, on the same rank-0 share
+                the host cores, on the same rank-0 share (the gradient path
+                and Newton-Schulz have their own CPU legs under `secondary`)
   secondary     unpack+dequant of the 8-rank gathered layout, the fp32
                 gradient path, the 48-matrix Muon / Newton-Schulz step, and the
                 forward and backward products of the prequantized-weight
@@ -37,13 +40,29 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor figure
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
 FP8_MFMA_PEAK_TFLOPS = 5000.0  # MI355X dense fp8, vendor figure
-# HBM bytes per launch of quantize_pack_bf16_kernel on the default workload, from
-# two counter runs (FETCH_SIZE, then WRITE_SIZE) of this script, each scaled by
-# the same counter's reading for the 256 MiB --calibrate-copy kernel:
-# 26 669.0 KiB x 1.9937 read + 26 932.2 KiB x 1.0 written.  Counters cannot be
-# read inside a timed run, so the figure is carried here and only reported
-# for the workload it was measured on.
-PROFILED_TRAFFIC_BYTES = {(27262976, 27531840): 82_024_000}
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "quantize_pack_bf16_kernel_llama3_8b_layer_rank0.md")
+
+
+def profiled_traffic(elems: int, payload_nbytes: int):
+    """HBM bytes per launch of the dominant kernel as the counter runs
+    (FETCH_SIZE, then WRITE_SIZE, each scaled by the same counter's reading for
+    a plain copy of known size) found them.  Counters cannot be read inside a
+    timed run, so the figure is read from the committed summary of those runs,
+    which names the workload and the commit of the kernel it was measured on:
+    a line `traffic_bytes_per_launch: <bytes> elems=<n> payload_nbytes=<n> commit=<sha>`.
+    Returns (bytes, commit) or (None, None) when the summary has no line for
+    this workload."""
+    import re
+
+    try:
+        with open(TRAFFIC_PROFILE) as fh:
+            text = fh.read()
+    except OSError:
+        return None, None
+    for m in re.finditer(r"traffic_bytes_per_launch:\s*(\d+)\s+elems=(\d+)\s+payload_nbytes=(\d+)\s+commit=(\w+)", text):
+        if int(m.group(2)) == elems and int(m.group(3)) == payload_nbytes:
+            return int(m.group(1)), m.group(4)
+    return None, None
 
 
 def _factory(fp8_data, recip_scale, block_size, *, orig_dtype, requires_grad):
@@ -90,7 +109,9 @@ def build_quant_workload(device, layers: int, rank: int = 0, spec=None, std: flo
     return placement, mesh, infos, work
 
 
-def bench_quant_pack(device, steps, warmup, layers, rank: int = 0, spec=None, std: float = 0.02):
+def bench_quant_pack(device, steps, warmup, layers, rank: int = 0, spec=None, std: float = 0.02, extras: bool = False):
+    """One step = one pass over the `layers` layer buckets: one fused
+    quantize+pack launch per bucket through the placement."""
     placement, mesh, infos, work = build_quant_workload(device, layers, rank, spec, std)
     metadata = placement._quant_metadata_from_infos(infos)
     plan = metadata.rank_pack_plans[rank]
@@ -99,25 +120,87 @@ def bench_quant_pack(device, steps, warmup, layers, rank: int = 0, spec=None, st
     algo_bytes = 3 * elems + 4 * scales  # 2 B read + 1 B write per element, 4 B per tile scale
     payloads = [torch.empty(metadata.packed_send_nbytes_per_rank, dtype=torch.uint8, device=device) for _ in work]
 
-    def step(i):
-        _, shards = work[i % len(work)]
-        # The placement's own entry point; the payload buffer is recycled the
-        # way the caching allocator recycles it in a training loop.
-        payloads[i % len(work)] = placement._pack_local_quantized_chunks(shards, infos, rank, metadata)
+    def launch(layer):
+        # The placement's pack step; the payload buffer is recycled the way the
+        # caching allocator recycles it in a training loop.
+        payloads[layer] = placement._pack_local_quantized_chunks(work[layer][1], infos, rank, metadata)
 
+    def step(i):
+        for layer in range(len(work)):
+            launch(layer)
+
+    # Steady state first, independent of --warmup: every bucket's launch table
+    # is built and cached and every payload block has been through the
+    # allocator before the clock starts.
+    for _ in range(2):
+        step(0)
+    torch.cuda.synchronize()
     wall_ms, event_ms = _event_ms(step, steps, warmup)
-    # Hot-cache variant (one layer over and over) for the record.
-    _, hot_ms = _event_ms(lambda i: step(0), steps, 5)
-    return {
+    out = {
         "elems": elems,
         "algo_bytes": algo_bytes,
+        "launches_per_step": len(work),
         "wall_ms": wall_ms,
         "event_ms": event_ms,
-        "hot_event_ms": hot_ms,
         "payload_nbytes": metadata.packed_send_nbytes_per_rank,
         "chunks": len(plan.chunks),
         "work": (placement, infos, work, metadata, payloads),
     }
+    if not extras:
+        return out
+    n = steps * len(work)
+    # Hot-cache variant (one layer over and over) for the record.
+    _, hot_ms = _event_ms(lambda i: launch(0), n, 5)
+    out["hot_us"] = hot_ms / n * 1e3
+
+    # The contract entry: prepare_unshard_bucket = payload-cache bookkeeping,
+    # pack, and the allocation of the W x row gather output.  Host time is the
+    # time the calls take to issue (nothing waits for the GPU inside them).
+    for layer in range(len(work)):
+        placement.prepare_unshard_bucket(work[layer][1], infos, mesh, None)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(n):
+        placement.prepare_unshard_bucket(work[i % len(work)][1], infos, mesh, None)
+    t_issued = time.perf_counter()
+    stop.record()
+    torch.cuda.synchronize()
+    out["contract_us"] = start.elapsed_time(stop) / n * 1e3
+    out["contract_host_us"] = (t_issued - t0) / n * 1e6
+    t0 = time.perf_counter()
+    for i in range(n):
+        launch(i % len(work))
+    out["pack_host_us"] = (time.perf_counter() - t0) / n * 1e6
+    torch.cuda.synchronize()
+
+    # Two buckets in flight on two streams of the same (default) priority, the
+    # way a prefetching runtime issues the next bucket's pack while the current
+    # one drains: launches alternate between the streams.
+    streams = [torch.cuda.Stream(device), torch.cuda.Stream(device)]
+    ready = torch.cuda.Event()
+    ready.record()
+    for st in streams:
+        st.wait_event(ready)
+    for rep in range(2):  # the first repetition warms both streams
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        joined = torch.cuda.Event()
+        with torch.cuda.stream(streams[0]):
+            start.record()
+        fence = torch.cuda.Event()
+        fence.record(streams[0])
+        streams[1].wait_event(fence)
+        for i in range(n):
+            with torch.cuda.stream(streams[i % 2]):
+                launch(i % len(work))
+        joined.record(streams[1])
+        streams[0].wait_event(joined)
+        with torch.cuda.stream(streams[0]):
+            stop.record()
+        torch.cuda.synchronize()
+    out["two_stream_us"] = start.elapsed_time(stop) / n * 1e3
+    return out
 
 
 def bench_other_shares(device):
@@ -128,12 +211,12 @@ def bench_other_shares(device):
 
     out = {}
     for name, kwargs, steps in (
-        ("llama3_8b_rank6", dict(layers=8, rank=6), 200),
-        ("deepseek_v3_experts_rank0", dict(layers=2, rank=0, spec=DEEPSEEK_V3_EXPERTS, std=0.006), 40),
+        ("llama3_8b_rank6", dict(layers=8, rank=6), 25),
+        ("deepseek_v3_experts_rank0", dict(layers=2, rank=0, spec=DEEPSEEK_V3_EXPERTS, std=0.006), 20),
     ):
-        q = bench_quant_pack(device, steps, 10, **kwargs)
+        q = bench_quant_pack(device, steps, 2, **kwargs)
         q.pop("work")
-        us = q["event_ms"] / steps * 1e3
+        us = q["event_ms"] / (steps * q["launches_per_step"]) * 1e3
         out[name] = {"elems": q["elems"], "chunks": q["chunks"], "algorithmic_bytes": q["algo_bytes"],
                      "us_per_launch": us, "GBps": q["algo_bytes"] / us / 1e3,
                      "frac_of_hbm_peak": q["algo_bytes"] / us / 1e3 / HBM_PEAK_GBPS}
@@ -189,6 +272,76 @@ def cpu_baseline_quant(work, infos, metadata, budget_s: float = 20.0):
         times.append(time.perf_counter() - t0)
     times.sort()
     return times[len(times) // 2], len(times), torch.get_num_threads()
+
+
+def cpu_baseline_gradients(reps: int = 5):
+    """Config 4 on the host cores, on a bounded sample: one rank range
+    (27 295 744 elements, an eighth of the layer bucket) through the oracle's
+    eager restatement of the fp32 microbatch accumulation (4 bf16 microbatches)
+    and of the fixed-order 8-way fold."""
+    from oracle import eager
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    seg, world = 27295744, 8
+    gen = torch.Generator().manual_seed(7)
+    micro = [(torch.randn(seg, generator=gen) * 1e-3).bfloat16() for _ in range(4)]
+    eager.accumulate_microbatches(micro)
+    acc_t = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        eager.accumulate_microbatches(micro)
+        acc_t.append(time.perf_counter() - t0)
+    del micro
+    contrib = [torch.randn(seg, generator=gen) * 1e-3 for _ in range(world)]
+    eager.reduce_rank_contributions(contrib, 0, seg)
+    red_t = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        eager.reduce_rank_contributions(contrib, 0, seg)
+        red_t.append(time.perf_counter() - t0)
+    acc_s, red_s = sorted(acc_t)[reps // 2], sorted(red_t)[reps // 2]
+    return {
+        "kind": "port",
+        "cores": torch.get_num_threads(),
+        "sample": f"one rank range of {seg} elements (1/8 of the bucket): 4 bf16 microbatches accumulated in fp32, "
+        f"then the 8-way fixed-order fold of that range; eager torch, median of {reps}",
+        "accumulate_ms_per_microbatch_on_sample": round(acc_s / 4 * 1e3, 3),
+        "accumulate_GBps": round(10 * seg * 4 / acc_s / 1e9, 3),
+        "reduce_ms": round(red_s * 1e3, 3),
+        "reduce_GBps": round(36 * seg / red_s / 1e9, 3),
+    }
+
+
+def cpu_baseline_newton_schulz(flops_full: int, per_shape: int = 2, reps: int = 3):
+    """Config 5 on the host cores, on a bounded sample: `per_shape` matrices
+    of each of the two shapes through torch's own Newton-Schulz
+    (torch.optim._muon._zeropower_via_newtonschulz, the routine the oracle is
+    pinned to), scaled linearly to the 24 + 24 matrices."""
+    from torch.optim._muon import _zeropower_via_newtonschulz as torch_ns
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    gen = torch.Generator().manual_seed(11)
+    coeffs, steps, eps = (3.4445, -4.7750, 2.0315), 5, 1e-7
+    total_s = 0.0
+    for shape in ((7168, 2048), (2048, 2048)):
+        mats = [torch.randn(shape, generator=gen).bfloat16() for _ in range(per_shape)]
+        torch_ns(mats[0], coeffs, steps, eps)
+        times = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            for m in mats:
+                torch_ns(m, coeffs, steps, eps)
+            times.append(time.perf_counter() - t0)
+        total_s += sorted(times)[reps // 2] * (24 / per_shape)
+    return {
+        "kind": "port",
+        "cores": torch.get_num_threads(),
+        "sample": f"{per_shape} matrices of [7168, 2048] and {per_shape} of [2048, 2048] through "
+        f"torch.optim._muon._zeropower_via_newtonschulz in bf16 on the host, median of {reps}, scaled by "
+        f"{24 // per_shape} to the 24 + 24 matrices",
+        "newton_schulz_ms_scaled_to_full_config": round(total_s * 1e3, 1),
+        "TFLOPs": round(flops_full / total_s / 1e12, 4),
+    }
 
 
 def bench_unpack(device, placement, infos, reps=10):
@@ -431,8 +584,8 @@ def calibrate_copy(device, nbytes: int = 256 << 20, reps: int = 4) -> None:
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=400)
-    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--steps", type=int, default=50, help="timed passes over the layer buckets")
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--layers", type=int, default=8, help="distinct layer buckets the steps rotate over")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-secondary", action="store_true")
@@ -465,13 +618,16 @@ def main() -> None:
         return
     if args.calibrate_copy:
         calibrate_copy(device)
-    q = bench_quant_pack(device, args.steps, args.warmup, args.layers)
+    q = bench_quant_pack(device, args.steps, args.warmup, args.layers, extras=True)
     placement, infos, work, metadata, payloads = q.pop("work")
     check_against_oracle(placement, infos, work, metadata, payloads)
+    launches = args.steps * q["launches_per_step"]
+    step_bytes = q["algo_bytes"] * q["launches_per_step"]
     ms_per_step = q["wall_ms"] / args.steps
-    value = q["algo_bytes"] / (ms_per_step * 1e-3) / 1e9
-    kernel_ms = q["event_ms"] / args.steps
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    kernel_ms = q["event_ms"] / launches
     achieved = q["algo_bytes"] / (kernel_ms * 1e-3) / 1e9
+    traffic, traffic_commit = profiled_traffic(q["elems"], q["payload_nbytes"])
 
     result = {
         "metric": "FP8 quantize+pack GB/s (% HBM peak), Llama-3-8B layer bucket; Muon NS TFLOP/s",
@@ -489,7 +645,9 @@ def main() -> None:
         "config": {
             "workload": "Llama-3-8B layer bucket (q,k,v,o,gate,up,down), rank 0 of 8: q, k, v, o[0:512] = "
             f"{q['elems']} bf16 elements in {q['chunks']} chunks -> {q['payload_nbytes']}-byte FP8 payload, "
-            f"128x128 tiles; steps rotate over {args.layers} layer buckets (cold HBM)",
+            f"128x128 tiles; one step = one pass over {args.layers} layer buckets, one launch each (cold HBM); "
+            "every bucket packed twice untimed before the warm-up (launch tables and allocator blocks in place)",
+            "launches_per_step": q["launches_per_step"],
             "device": torch.cuda.get_device_name(0),
             "percent_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 1),
         },
@@ -500,10 +658,27 @@ def main() -> None:
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": PROFILED_TRAFFIC_BYTES.get((q["elems"], q["payload_nbytes"])),
+            "traffic": traffic,
+            "traffic_measured_at_commit": traffic_commit,
             "algorithmic_bytes_per_launch": q["algo_bytes"],
             "avg_launch_us": round(kernel_ms * 1e3, 2),
-            "avg_launch_us_hot_cache": round(q["hot_event_ms"] / args.steps * 1e3, 2),
+            "avg_launch_us_hot_cache": round(q["hot_us"], 2),
+        },
+        # The same launch through the contract method (payload-cache
+        # bookkeeping, pack, allocation of the W x row gather output), the host
+        # time either call takes to issue, and the rate with two buckets in
+        # flight on two default-priority streams.
+        "contract_entry": {
+            "prepare_unshard_bucket_us_per_call": round(q["contract_us"], 2),
+            "prepare_unshard_bucket_GBps": round(q["algo_bytes"] / q["contract_us"] / 1e3, 1),
+            "prepare_unshard_bucket_host_us_per_call": round(q["contract_host_us"], 2),
+            "pack_step_host_us_per_call": round(q["pack_host_us"], 2),
+        },
+        "two_buckets_in_flight": {
+            "streams": 2,
+            "us_per_launch": round(q["two_stream_us"], 2),
+            "GBps": round(q["algo_bytes"] / q["two_stream_us"] / 1e3, 1),
+            "frac_of_hbm_peak": round(q["algo_bytes"] / q["two_stream_us"] / 1e3 / HBM_PEAK_GBPS, 4),
         },
     }
     if not args.skip_cpu:
@@ -532,6 +707,9 @@ def main() -> None:
         torch.cuda.empty_cache()
         muon = bench_muon(device)
         secondary["muon_newton_schulz"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in muon.items()}
+        if not args.skip_cpu:
+            secondary["gradient_path"]["cpu_baseline"] = cpu_baseline_gradients()
+            secondary["muon_newton_schulz"]["cpu_baseline"] = cpu_baseline_newton_schulz(muon["ns_flop"])
         torch.cuda.empty_cache()
         secondary["fp8_linear_forward_8192_tokens"] = {
             name: {k: round(v, 4) for k, v in d.items()} for name, d in bench_fp8_linear(device).items()

@@ -484,9 +484,13 @@ int launch_fp8_gemm(Fp8GemmParams& p, bool column_scales, const char* who, void*
   if (p.m < 0 || p.n < 0 || p.k < 0) return fail(FSH_EINVAL, "%s: negative size", who);
   if (p.m == 0 || p.n == 0) return FSH_OK;
   if (!p.xq || !p.xs || !p.wq || !p.out || (column_scales ? !p.cs : !p.ws)) return fail(FSH_EINVAL, "%s: null pointer", who);
-  if (p.k == 0 || p.k % 128 || p.k / 128 > Fp8Gemm::kMaxKTilesInLds)
-    return fail(FSH_ENOTSUP, "%s: k must be a positive multiple of 128 (pad the operands) and at most %d, got %lld", who,
-                128 * Fp8Gemm::kMaxKTilesInLds, (long long)p.k);
+  if (p.k == 0 || p.k % 128)
+    return fail(FSH_ENOTSUP, "%s: k must be a positive multiple of 128 (pad the operands), got %lld", who, (long long)p.k);
+  // Only the block-scale variant keeps one weight scale per k-tile in LDS; the
+  // column-scale variant contracts over tokens and takes any length.
+  if (!column_scales && p.k / 128 > Fp8Gemm::kMaxKTilesInLds)
+    return fail(FSH_ENOTSUP, "%s: k must be at most %d, got %lld", who, 128 * Fp8Gemm::kMaxKTilesInLds, (long long)p.k);
+  if (p.k >= (1LL << 31)) return fail(FSH_ENOTSUP, "%s: k must be below 2^31, got %lld", who, (long long)p.k);
   if (p.ldxq < p.k || p.ldwq < p.k || p.ldo < p.n)
     return fail(FSH_EINVAL, "%s: a leading dimension is smaller than its row", who);
   if (p.ldxq % 16 || p.ldwq % 16 || !aligned(p.xq, 16) || !aligned(p.wq, 16) || !aligned(p.out, 2))

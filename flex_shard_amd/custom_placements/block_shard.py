@@ -32,7 +32,7 @@ from ..placement_contract import (
     PlacementUnshardResult,
 )
 from ..profiling import record_comm, record_copy_in, record_copy_out, record_range
-from ._copy_kernels import SegmentPackDescriptor
+from ._copy_kernels import SegmentCopyDescriptor, SegmentPackDescriptor, copy_segments, pack_segments_into_flat_buffer
 from .utils import (
     all_gather_rows,
     copy_tensor_to_dtype,
@@ -218,6 +218,8 @@ class BucketedBlockShard(Placement):
         self.dims = dims
         self.blocks_per_rank = blocks_per_rank
         self._reduce_copy_in_plans: dict = {}
+        self._send_row_descriptors: dict = {}
+        self._scatter_descriptors: dict = {}
 
     def __eq__(self, other: object) -> bool:
         if not isinstance(other, BucketedBlockShard):
@@ -439,19 +441,61 @@ class BucketedBlockShard(Placement):
             raise ValueError("BucketedBlockShard requires one unsharded dtype per bucket.")
         with record_copy_in():
             send = self._make_local_bucket_view(tensors, infos)
-            scratch: list[torch.Tensor] = []
-            if send.dtype != dtype:
-                send, scratch = pack_tensors_into_flat_buffer_with_scratch([send], dtype)
-            else:
-                send = copy_tensor_to_dtype(send, dtype)
-            short_by = max(self._bucket_layout(infos[0]).rank_numels) - send.numel()
-            if short_by > 0:
-                send = nn.functional.pad(send, (0, short_by))
+            send, scratch = self._send_row(send, dtype, max(self._bucket_layout(infos[0]).rank_numels))
         return PlacementPreparedUnshard(
             placement=self,
             buffers=[send, *scratch],
             placement_state=BucketedBlockShard._UnshardState(infos=infos, pg=mesh.get_group(), debug_fqn=debug_fqn),
         )
+
+    def _send_row(self, local: torch.Tensor, dtype: torch.dtype, widest: int) -> tuple[torch.Tensor, list[torch.Tensor]]:
+        """The all-gather input of this rank: its flat range in the unsharded
+        dtype, zero-padded to the longest rank range.  A range that already
+        has that dtype and length is sent as it lies (no copy); anything else
+        is one cast-pack launch that writes the cast elements and the zero pad
+        together (the reference casts with a foreach copy and then pads with
+        ``F.pad``, custom_placements/block_shard.py:948-958).  Returns the row
+        and the tensors to keep alive until the launch has run."""
+        short_by = widest - local.numel()
+        if local.dtype == dtype and short_by <= 0:
+            return local, []
+        floats = (torch.float32, torch.bfloat16)
+        if (
+            torch.compiler.is_compiling()
+            or local.device.type != "cuda"
+            or local.dtype not in floats
+            or dtype not in floats
+            or local.numel() == 0
+        ):
+            send, scratch = local, []
+            if send.dtype != dtype:
+                send, scratch = pack_tensors_into_flat_buffer_with_scratch([send], dtype)
+            else:
+                send = copy_tensor_to_dtype(send, dtype)
+            if short_by > 0:
+                send = nn.functional.pad(send, (0, short_by))
+            return send, scratch
+        key = (local.numel(), widest, local.device)
+        descriptor = self._send_row_descriptors.get(key)
+        if descriptor is None:
+            pad = [(-1, 0, short_by, local.numel())] if short_by > 0 else []
+            segments = [(0, 0, local.numel(), 0), *pad]
+            descriptor = SegmentPackDescriptor.create(
+                ninputs=1,
+                tensor_indices=[seg[0] for seg in segments],
+                src_offsets=[seg[1] for seg in segments],
+                numels=[seg[2] for seg in segments],
+                dst_offsets=[seg[3] for seg in segments],
+                device=local.device,
+            )
+            if len(self._send_row_descriptors) >= 16:
+                self._send_row_descriptors.clear()
+            self._send_row_descriptors[key] = descriptor
+        row = torch.empty(max(widest, local.numel()), dtype=dtype, device=local.device)
+        keep = pack_segments_into_flat_buffer([local], (), (), (), (), row, descriptor=descriptor)
+        if keep is None:
+            raise AssertionError("BucketedBlockShard send-row pack was declined for a contiguous float range.")
+        return row, keep
 
     def run_prepared_unshard(self, prepared: PlacementPreparedUnshard, *, async_op: bool = False) -> Any | None:
         state = prepared.placement_state
@@ -477,10 +521,32 @@ class BucketedBlockShard(Placement):
 
     def _scatter_padded_rows_into_bucket(self, bucket: torch.Tensor, rows: torch.Tensor, layout: "BucketLayout") -> None:
         """Copy each rank's valid prefix of its padded gathered row into its
-        range of ``bucket`` (uneven ranges only)."""
-        in_bucket, in_rows = _rank_range_views(bucket, rows, layout.rank_offsets, layout.rank_numels)
+        range of ``bucket`` (uneven ranges only): one segment-copy launch for
+        all ranks (the reference issues a foreach copy over per-rank views,
+        custom_placements/block_shard.py:998-1011)."""
         with record_copy_out():
-            foreach_copy_(in_bucket, in_rows)
+            if torch.compiler.is_compiling() or bucket.device.type != "cuda" or not rows.is_contiguous():
+                in_bucket, in_rows = _rank_range_views(bucket, rows, layout.rank_offsets, layout.rank_numels)
+                foreach_copy_(in_bucket, in_rows)
+                return
+            key = (id(layout), rows.shape[1], bucket.device)
+            cached = self._scatter_descriptors.get(key)
+            if cached is None or cached[0] is not layout:
+                live = [
+                    (rank * rows.shape[1], count, start)
+                    for rank, (start, count) in enumerate(zip(layout.rank_offsets, layout.rank_numels, strict=True))
+                    if count
+                ]
+                descriptor = SegmentCopyDescriptor.create(
+                    src_offsets=[seg[0] for seg in live],
+                    numels=[seg[1] for seg in live],
+                    dst_offsets=[seg[2] for seg in live],
+                    device=bucket.device,
+                )
+                if len(self._scatter_descriptors) >= 16:
+                    self._scatter_descriptors.clear()
+                self._scatter_descriptors[key] = cached = (layout, descriptor)
+            copy_segments(rows, bucket, cached[1])
 
     def finish_prepared_unshard(self, prepared: PlacementPreparedUnshard) -> PlacementUnshardResult:
         state = prepared.placement_state

@@ -512,7 +512,14 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
                     f"Quantized pack plan parameter order changed: expected {chunk.fqn!r} at index "
                     f"{chunk.param_index}, got {info.fqn!r}."
                 )
-            shard = tensors[chunk.param_index].reshape(chunk.local_shape)
+            source = tensors[chunk.param_index]
+            shard = source.reshape(chunk.local_shape)
+            if shard.untyped_storage().data_ptr() != source.untyped_storage().data_ptr():
+                # The shard could not be viewed as [rows, in_dim] (e.g. a strided
+                # slice of a stacked parameter), so reshape made a temporary
+                # copy.  Its address must not outlive this call in a cached
+                # launch table.
+                staged.append(shard)
             if shard.numel() != chunk.qdata_numel:
                 raise AssertionError(
                     f"Quantized local dense shard does not match planned chunk for {chunk.fqn!r}: "

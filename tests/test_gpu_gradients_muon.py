@@ -707,3 +707,77 @@ def test_owned_muon_step_matches_torch_optim_muon(device, golden):
         before = [p.clone() for p in mine]
         opt_mine.step([None] + [torch.zeros_like(p) for p in mine[1:]])
     assert all(torch.equal(a, b) for a, b in zip(mine, before))
+
+
+# ------------------------------------------- config 5 at the benchmarked size
+CONFIG5_SHAPES = [(7168, 2048)] * 24 + [(2048, 2048)] * 24
+
+
+def _direction_error(mine: torch.Tensor, ref: torch.Tensor) -> tuple[float, float]:
+    diff = mine.float() - ref.float()
+    return diff.abs().max().item(), (diff.norm() / ref.float().norm()).item()
+
+
+def test_newton_schulz_multi_config5_batches_match_torch_routine(device, golden):
+    """The two batches the benchmark times, 24 x [7168, 2048] and
+    24 x [2048, 2048], in one newton_schulz_multi call (the launches shared by
+    both shape groups, one orientation carried, k-major operands, resident
+    workgroups): first and last matrix of each shape, element by element,
+    against torch's own Newton-Schulz (the reference's 2-D branch,
+    dist_muon/optimizer.py:2120-2151) at the reference's bar
+    (tests/test_dist_muon_optimizer.py:206-212), plus a relative Frobenius
+    bound so that the comparison has teeth on entries of size 0.02."""
+    from torch.optim._muon import _zeropower_via_newtonschulz as torch_ns
+
+    tol = golden["muon_tolerance"]["atol"]
+    batches = [seeded_normal((24, 7168, 2048), 1.0, 41, device), seeded_normal((24, 2048, 2048), 1.0, 42, device)]
+    inputs = {(b.shape[1], index): b[index].cpu() for b in batches for index in (0, 23)}
+    hip_ops.newton_schulz_multi([(b, None) for b in batches], COEFFS, 5, 1e-7)
+    for b in batches:
+        for index in (0, 23):
+            ref = torch_ns(inputs[(b.shape[1], index)], COEFFS, 5, 1e-7)
+            worst, rel = _direction_error(b[index].cpu(), ref)
+            print(f"config 5 NS {tuple(b.shape[1:])}[{index}]: max abs {worst:.3e}, rel Frobenius {rel:.3e}", flush=True)
+            assert worst <= tol
+            assert rel <= 2e-2
+        # equal inputs in different batch slots give equal bits
+    again = torch.stack([inputs[(7168, 0)]] * 24).to(device)
+    hip_ops.newton_schulz_multi([(again, None), (batches[1].normal_(), None)], COEFFS, 5, 1e-7)
+    assert torch.equal(again[0], again[23]) and torch.equal(again[0], batches[0][0])
+
+
+def test_owned_muon_step_config5_matches_reference_step(device, golden):
+    """One OwnedMuon.step over the 48 matrices of config 5 (gradients N(0, 1),
+    momentum 0.95, Nesterov, 5 steps): orthogonalized direction and updated
+    parameter of the first and last matrix of each shape against the
+    reference step in eager torch on the host (dist_muon/optimizer.py
+    :2049-2151)."""
+    tol = golden["muon_tolerance"]["atol"]
+    params = [seeded_normal(s, 0.02, 2000 + i, device) for i, s in enumerate(CONFIG5_SHAPES)]
+    grads = [seeded_normal(s, 1.0, 3000 + i, device) for i, s in enumerate(CONFIG5_SHAPES)]
+    checked = (0, 23, 24, 47)
+    before = {i: params[i].cpu() for i in checked}
+    opt = OwnedMuon(params)
+    opt.step(grads)
+    for i in checked:
+        shape = CONFIG5_SHAPES[i]
+        slot = opt._groups[shape].index(i)
+        direction = opt._batch[shape][slot].cpu()
+        momentum = torch.zeros(shape, dtype=torch.bfloat16)
+        g = grads[i].cpu()
+        momentum.lerp_(g, 1 - 0.95)
+        update = torch.lerp(g, momentum, 0.95)
+        ref_direction = eager.newton_schulz(update, COEFFS, 5, 1e-7)
+        worst, rel = _direction_error(direction, ref_direction)
+        print(f"config 5 Muon {shape}[{i}]: direction max abs {worst:.3e}, rel Frobenius {rel:.3e}", flush=True)
+        assert worst <= tol
+        assert rel <= 2e-2
+        assert torch.equal(opt.momentum_buffers[i].cpu(), momentum)
+        p_ref = before[i].clone()
+        p_ref.mul_(1 - 1e-3 * 0.1)
+        p_ref.add_(ref_direction, alpha=-eager.adjusted_lr(1e-3, None, shape))
+        assert (params[i].cpu().float() - p_ref.float()).abs().max().item() <= tol
+        assert torch.allclose(params[i].cpu().float(), p_ref.float(), rtol=2.0**-7, atol=2e-5)  # one bf16 ulp
+    assert opt.flops_per_step() == 2 * (
+        _estimate_muon_compute_cost((24, 7168, 2048), 5) + _estimate_muon_compute_cost((24, 2048, 2048), 5)
+    )
