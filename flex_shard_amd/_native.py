@@ -101,6 +101,7 @@ class NsProblem(Structure):
 
 
 MAX_NS_PROBLEMS = 16
+NS_STATIC_SCRATCH_BYTES = 128 << 20
 
 
 # name -> (restype, argtypes); every symbol include/flexshard_hip.h declares.
@@ -127,6 +128,9 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "fsh_newton_schulz": (
         c_int,
         [c_void_p, c_int64, c_int64, c_int64, c_float, c_float, c_float, c_int32, c_float, c_void_p, c_int64, c_void_p],
+    ),
+    "fsh_newton_schulz_noalloc": (
+        c_int, [c_void_p, c_int64, c_int64, c_int64, c_float, c_float, c_float, c_int32, c_float, c_void_p],
     ),
     "fsh_newton_schulz_multi": (
         c_int, [POINTER(NsProblem), c_int32, c_float, c_float, c_float, c_int32, c_float, c_void_p],

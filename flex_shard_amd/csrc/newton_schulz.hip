@@ -1159,3 +1159,69 @@ FSH_API int fsh_newton_schulz(void* x_dev, int64_t batch, int64_t rows, int64_t 
   q.workspace_nbytes = workspace_nbytes;
   return fsh_newton_schulz_multi(&q, 1, a, b, c, steps, eps, stream_);
 }
+
+// ------------------------------------------------------------------------
+// Allocation-free variant: the workspace is a static device array.
+//
+// `scratch` is a host-side stand-in for the device array, not a device
+// address: each GPU holds its own copy at its own address, resolved once per
+// device with hipGetSymbolAddress while that device is current.  Everything
+// below uses the resolved pointer, never the array's name.
+namespace fsh {
+namespace {
+
+static __device__ __align__(256) uint8_t scratch[FSH_NS_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// The current device's copy of `scratch`.
+int static_scratch(void** out) {
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess) return fail(FSH_EHIP, "fsh_newton_schulz_noalloc: hipGetDevice: %s", hipGetErrorString(err));
+  if (device < 0 || device >= kMaxDevices)
+    return fail(FSH_ENOTSUP, "fsh_newton_schulz_noalloc: device index %d outside [0, %d)", device, kMaxDevices);
+  void* ptr = g_scratch_ptr[device].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || ptr == nullptr)
+      return fail(FSH_EHIP, "fsh_newton_schulz_noalloc: hipGetSymbolAddress(scratch) on device %d: %s", device,
+                  hipGetErrorString(err));
+    g_scratch_ptr[device].store(ptr, std::memory_order_release);  // every thread resolves the same address
+  }
+  *out = ptr;
+  return FSH_OK;
+}
+
+}  // namespace
+}  // namespace fsh
+
+FSH_API int fsh_newton_schulz_noalloc(void* x_dev, int64_t batch, int64_t rows, int64_t cols, float a, float b,
+                                      float c, int32_t steps, float eps, void* stream_) {
+  using namespace fsh;
+  if (batch <= 0 || rows <= 0 || cols <= 0)
+    return fail(FSH_EINVAL, "fsh_newton_schulz_noalloc: bad sizes (batch %lld, rows %lld, cols %lld)", (long long)batch,
+                (long long)rows, (long long)cols);
+  // Checked in wide arithmetic before the byte count is formed: a huge request must not wrap around.
+  const int64_t s = rows < cols ? rows : cols, l = rows < cols ? cols : rows;
+  if (batch > 65535 || l > (1LL << 24) || s * l > FSH_NS_STATIC_SCRATCH_BYTES / 4 / batch)
+    return fail(FSH_ENOTSUP,
+                "fsh_newton_schulz_noalloc: batch %lld of %lld x %lld exceeds the %lld-byte static scratch; call "
+                "fsh_newton_schulz with a workspace of fsh_newton_schulz_workspace_bytes()",
+                (long long)batch, (long long)rows, (long long)cols, (long long)FSH_NS_STATIC_SCRATCH_BYTES);
+  const int64_t need = fsh_newton_schulz_workspace_bytes(batch, rows, cols);
+  if (need > FSH_NS_STATIC_SCRATCH_BYTES)
+    return fail(FSH_ENOTSUP,
+                "fsh_newton_schulz_noalloc: batch %lld of %lld x %lld needs %lld bytes of scratch, the static scratch "
+                "holds %lld; call fsh_newton_schulz with a workspace of that size",
+                (long long)batch, (long long)rows, (long long)cols, (long long)need,
+                (long long)FSH_NS_STATIC_SCRATCH_BYTES);
+  void* ptr = nullptr;
+  if (int rc = static_scratch(&ptr)) return rc;
+  // Every region of the workspace is written before it is read (norm
+  // partials, both iterate buffers, G and P), so nothing has to be cleared
+  // between calls.
+  return fsh_newton_schulz(x_dev, batch, rows, cols, a, b, c, steps, eps, ptr, FSH_NS_STATIC_SCRATCH_BYTES, stream_);
+}
+

@@ -34,7 +34,7 @@ __all__ = [
     "QuantChunkSpec", "QuantPackPlan", "accumulate_grad", "act_quant_128x1_transposed", "act_quant_1x128",
     "copy_segments", "fp8_gemm_1x128_128x1", "fp8_gemm_1x128_128x128", "fp8_gemm_1x128_128x128_dgrad",
     "fp8_transpose", "gemm_nt", "gemm_nt_group", "muon_apply", "muon_prepare", "newton_schulz_multi",
-    "newton_schulz", "newton_schulz_workspace_bytes", "pack_segments", "quantize_pack",
+    "newton_schulz", "newton_schulz_noalloc", "newton_schulz_workspace_bytes", "pack_segments", "quantize_pack",
     "reduce_rows", "stream_ptr", "unpack_dequant", "zero_segments",
 ]
 
@@ -310,6 +310,26 @@ def newton_schulz(
         stream_ptr(x.device),
     )
     _native.check(status, "fsh_newton_schulz")
+    return x
+
+
+def newton_schulz_noalloc(
+    x: torch.Tensor, coefficients: tuple[float, float, float], steps: int, eps: float
+) -> torch.Tensor:
+    """``newton_schulz`` on the library's static device scratch: nothing is
+    allocated, by this wrapper or by the library.  The batch must fit the
+    scratch (``_native.NS_STATIC_SCRATCH_BYTES``); calls on one GPU share it,
+    so calls that overlap on different streams race."""
+    _require_gpu(x)
+    if x.dtype != torch.bfloat16 or not x.is_contiguous() or x.ndim not in (2, 3):
+        raise ValueError("x must be a contiguous bf16 matrix or batch of matrices")
+    batch = 1 if x.ndim == 2 else x.shape[0]
+    rows, cols = x.shape[-2:]
+    a, b, c = coefficients
+    status = _native.lib().fsh_newton_schulz_noalloc(
+        x.data_ptr(), batch, rows, cols, a, b, c, steps, eps, stream_ptr(x.device)
+    )
+    _native.check(status, "fsh_newton_schulz_noalloc")
     return x
 
 

@@ -202,6 +202,23 @@ typedef struct fsh_ns_problem {
 int fsh_newton_schulz_multi(const fsh_ns_problem* problems, int32_t count, float a, float b, float c,
                             int32_t steps, float eps, void* stream);
 
+/* Allocation-free variant of fsh_newton_schulz.  It has no counterpart in the
+ * reference: it is for callers that cannot allocate device memory or bring a
+ * workspace (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc).  The workspace is a static device array of
+ * FSH_NS_STATIC_SCRATCH_BYTES inside the library, held on every GPU the
+ * library runs on until the process ends; its address on the current device
+ * is resolved on the first call on that device (so make that first call
+ * outside any graph capture).  The call allocates and frees nothing.  A batch
+ * whose fsh_newton_schulz_workspace_bytes() exceeds the static scratch is
+ * rejected with FSH_ENOTSUP.  All calls on one GPU share the one array: calls
+ * that overlap on a GPU (different streams, or threads) race and must be
+ * serialized by the caller; calls on one stream are ordered by the stream.
+ * Results are those of fsh_newton_schulz, bit for bit. */
+#define FSH_NS_STATIC_SCRATCH_BYTES (128LL << 20)
+int fsh_newton_schulz_noalloc(void* x_dev, int64_t batch, int64_t rows, int64_t cols, float a, float b,
+                              float c, int32_t steps, float eps, void* stream);
+
 /* Batched bf16 "NT" GEMM, the building block of (6), exported for tests:
  *   C[b] = bf16(alpha * A[b] . B[b]^T + beta * D[b] + diag_add * I)   fp32 accumulation
  * A is [m, k] with row stride lda, B is [n, k] with row stride ldb (both
