@@ -100,6 +100,24 @@ class NsProblem(Structure):
     ]
 
 
+class MuonGroup(Structure):
+    """``fsh_muon_group``."""
+
+    _fields_ = [
+        ("param_ptrs_dev", c_void_p),
+        ("grad_ptrs_dev", c_void_p),
+        ("momentum_ptrs_dev", c_void_p),
+        ("batch_dev", c_void_p),
+        ("batch", c_int64),
+        ("rows", c_int64),
+        ("cols", c_int64),
+        ("workspace_dev", c_void_p),
+        ("workspace_nbytes", c_int64),
+        ("neg_adjusted_lr", c_float),
+        ("direction_scale", c_float),
+    ]
+
+
 MAX_NS_PROBLEMS = 16
 NS_STATIC_SCRATCH_BYTES = 128 << 20
 
@@ -158,6 +176,11 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     ),
     "fsh_muon_prepare": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_float, c_float, c_int32, c_void_p]),
     "fsh_muon_apply": (c_int, [c_void_p, c_void_p, c_int64, c_float, c_float, c_float, c_void_p]),
+    "fsh_muon_step": (
+        c_int,
+        [POINTER(MuonGroup), c_int32, c_float, c_float, c_int32, c_float, c_float, c_float, c_float, c_int32, c_float,
+         c_void_p],
+    ),
 }
 
 _LIB: ctypes.CDLL | None = None

@@ -4,6 +4,7 @@
 // All are HBM-bound streaming kernels: 16-byte accesses, grid-stride loops
 // sized to a few workgroups per compute unit.
 #include "common.hpp"
+#include "muon_elementwise.hpp"
 
 namespace fsh {
 namespace {
@@ -113,33 +114,6 @@ __global__ __launch_bounds__(kThreads) void reduce_rows_kernel(float* __restrict
   }
 }
 
-// torch.lerp(start, end, w) in fp32: w < 0.5 ? start + w*(end-start)
-//                                            : end - (end-start)*(1-w).
-__device__ __forceinline__ float lerp_f32(float start, float end, float w) {
-  const float diff = end - start;
-  return w < 0.5f ? start + w * diff : end - diff * (1.0f - w);
-}
-
-// Eight bf16 values of a 16-byte vector as floats, and back.
-__device__ __forceinline__ void unpack8(const u32x4 v, float* f) {
-  const uint32_t d[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    f[2 * j] = u32_as_f32(d[j] << 16);
-    f[2 * j + 1] = u32_as_f32(d[j] & 0xFFFF0000u);
-  }
-}
-__device__ __forceinline__ u32x4 pack8(const uint32_t* bits) {
-  return u32x4{bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16), bits[4] | (bits[5] << 16),
-               bits[6] | (bits[7] << 16)};
-}
-
-__device__ __forceinline__ void muon_prepare_one(float m, float g, float one_minus_mu, float mu, int nesterov,
-                                                 uint32_t* m_bits, uint32_t* out_bits) {
-  *m_bits = f32_to_bf16_bits(lerp_f32(m, g, one_minus_mu));
-  *out_bits = nesterov ? f32_to_bf16_bits(lerp_f32(g, bf16_bits_to_f32(*m_bits), mu)) : *m_bits;
-}
-
 // m = bf16(lerp(m, g, 1-mu)); out = nesterov ? bf16(lerp(g, m, mu)) : m.
 // 8 elements (16 bytes) per thread and iteration when the three pointers are
 // 16-byte aligned, then a scalar tail; scalar throughout otherwise.
@@ -171,12 +145,6 @@ __global__ __launch_bounds__(kThreads) void muon_prepare_kernel(uint16_t* __rest
     mom[i] = static_cast<uint16_t>(mb);
     out[i] = static_cast<uint16_t>(ob);
   }
-}
-
-__device__ __forceinline__ uint32_t muon_apply_one(float p, float d, float decay, float neg_lr, float dir_scale) {
-  if (dir_scale != 1.0f) d = bf16_bits_to_f32(f32_to_bf16_bits(d * dir_scale));
-  p = bf16_bits_to_f32(f32_to_bf16_bits(p * decay));
-  return f32_to_bf16_bits(p + neg_lr * d);
 }
 
 // p = bf16(p * decay); p = bf16(p + neg_lr * d'), d' = scale == 1 ? d : bf16(d * scale).

@@ -20,6 +20,7 @@
 // buffering with one barrier per k-tile; LDS rows padded by 16 bytes so the
 // 64 lanes of a ds_read_b128 hit distinct banks.
 #include "mfma_tiles.hpp"
+#include "muon_elementwise.hpp"
 
 namespace fsh {
 namespace {
@@ -862,6 +863,27 @@ int launch_gemms(const fsh_gemm_desc* descs, int count, hipStream_t stream) {
 constexpr int kNormThreads = 256;
 constexpr int kNormBlocksPerMatrix = 64;
 
+// s plus the squares of the eight bf16 values of v, added one after the
+// other in element order.
+__device__ __forceinline__ float add_squares8(float s, const u32x4 v) {
+  const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float lo = u32_as_f32(d[j] << 16), hi = u32_as_f32(d[j] & 0xFFFF0000u);
+    s += lo * lo;
+    s += hi * hi;
+  }
+  return s;
+}
+// The workgroup's total in a fixed order: lanes by the wave reduction, then
+// the four waves as (0 + 1) + (2 + 3).  All threads call it.
+__device__ __forceinline__ void store_block_partial(float s, float* lds, float* slot) {
+  s = wave_sum_f32(s);
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) *slot = (lds[0] + lds[1]) + (lds[2] + lds[3]);
+}
+
 // partial[b][j] = sum of squares of slice j of matrix b in fp32.  The order
 // is fixed: a thread walks its 8-element groups front to back, lanes are
 // folded by the wave reduction, waves left to right.  numel is a multiple of
@@ -876,20 +898,122 @@ __global__ __launch_bounds__(kNormThreads) void sumsq_partial_kernel(const uint1
   const int64_t begin = blockIdx.x * per;
   const int64_t end = (begin + per) < groups ? (begin + per) : groups;
   float s = 0.0f;
-  for (int64_t g = begin + threadIdx.x; g < end; g += kNormThreads) {
-    const u32x4 v = load_stream_u32x4(m + g * 8);
-    const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+  for (int64_t g = begin + threadIdx.x; g < end; g += kNormThreads) s = add_squares8(s, load_stream_u32x4(m + g * 8));
+  store_block_partial(s, lds, &partial[b * kNormBlocksPerMatrix + blockIdx.x]);
+}
+
+// The momentum step of Muon for a batch of separately allocated matrices,
+// fused with the sum of squares of its output: for matrix b (blockIdx.y)
+//   m = bf16(lerp(m, g, 1 - mu));  u = nesterov ? bf16(lerp(g, m, mu)) : m
+// with u written to slot b of the contiguous batch buffer, and partial[b][j]
+// = the sum of squares of slice j of u.  Slices, the walk of a thread through
+// its slice and the order of the additions are those of sumsq_partial_kernel
+// on the stored u, so the partials are the same bits and the orthogonalization
+// that follows need not read u again to find its norm.
+struct MuonPrepareBatch {
+  const int64_t* momentum_ptrs;  // device table [batch]
+  const int64_t* grad_ptrs;      // device table [batch]
+  uint16_t* out;                 // [batch, numel]
+  float* partial;                // [batch, kNormBlocksPerMatrix]
+  int64_t numel;
+  float one_minus_mu, mu;
+  int32_t nesterov;
+};
+__global__ __launch_bounds__(kNormThreads) void muon_prepare_sumsq_kernel(const MuonPrepareBatch q) {
+  __shared__ float lds[kNormThreads / 64];
+  const int64_t b = blockIdx.y;
+  uint16_t* mom = reinterpret_cast<uint16_t*>(q.momentum_ptrs[b]);
+  const uint16_t* grad = reinterpret_cast<const uint16_t*>(q.grad_ptrs[b]);
+  uint16_t* out = q.out + b * q.numel;
+  const int64_t groups = q.numel / 8;
+  const int64_t per = ceil_div(groups, (int64_t)kNormBlocksPerMatrix);
+  const int64_t begin = blockIdx.x * per;
+  const int64_t end = (begin + per) < groups ? (begin + per) : groups;
+  float s = 0.0f;
+  // Four 16-byte groups per pass, all eight loads issued before the first
+  // store: the tables give the compiler no aliasing information, so a plain
+  // loop would hold every load back behind the previous group's stores.  The
+  // squares are still added group by group in walk order.
+  constexpr int kUnroll = 4;
+  int64_t g = begin + threadIdx.x;
+  for (; g + (kUnroll - 1) * kNormThreads < end; g += kUnroll * kNormThreads) {
+    u32x4 mraw[kUnroll], graw[kUnroll];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float lo = u32_as_f32(d[j] << 16), hi = u32_as_f32(d[j] & 0xFFFF0000u);
-      s += lo * lo;
-      s += hi * hi;
+    for (int k = 0; k < kUnroll; ++k) {
+      mraw[k] = load_stream_u32x4(mom + (g + k * kNormThreads) * 8);
+      graw[k] = load_stream_u32x4(grad + (g + k * kNormThreads) * 8);
+    }
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+      float mv[8], gv[8];
+      unpack8(mraw[k], mv);
+      unpack8(graw[k], gv);
+      uint32_t mb[8], ob[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) muon_prepare_one(mv[j], gv[j], q.one_minus_mu, q.mu, q.nesterov, &mb[j], &ob[j]);
+      store_stream_u32x4(mom + (g + k * kNormThreads) * 8, pack8(mb));
+      const u32x4 u = pack8(ob);
+      store_stream_u32x4(out + (g + k * kNormThreads) * 8, u);
+      s = add_squares8(s, u);
     }
   }
-  s = wave_sum_f32(s);
-  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = s;
-  __syncthreads();
-  if (threadIdx.x == 0) partial[b * kNormBlocksPerMatrix + blockIdx.x] = (lds[0] + lds[1]) + (lds[2] + lds[3]);
+  for (; g < end; g += kNormThreads) {
+    float mv[8], gv[8];
+    unpack8(load_stream_u32x4(mom + g * 8), mv);
+    unpack8(load_stream_u32x4(grad + g * 8), gv);
+    uint32_t mb[8], ob[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) muon_prepare_one(mv[j], gv[j], q.one_minus_mu, q.mu, q.nesterov, &mb[j], &ob[j]);
+    store_stream_u32x4(mom + g * 8, pack8(mb));
+    const u32x4 u = pack8(ob);
+    store_stream_u32x4(out + g * 8, u);
+    s = add_squares8(s, u);
+  }
+  store_block_partial(s, lds, &q.partial[b * kNormBlocksPerMatrix + blockIdx.x]);
+}
+
+// The update of Muon for the same batch: parameter b (a separate allocation)
+// takes the direction in slot b of the batch buffer,
+//   p = bf16(p * decay);  p = bf16(p + neg_lr * d)   (d first scaled and rounded if scale != 1).
+struct MuonApplyBatch {
+  const int64_t* param_ptrs;  // device table [batch]
+  const uint16_t* direction;  // [batch, numel]
+  int64_t numel;
+  float decay, neg_lr, dir_scale;
+};
+__global__ __launch_bounds__(kNormThreads) void muon_apply_batch_kernel(const MuonApplyBatch q) {
+  const int64_t b = blockIdx.y;
+  uint16_t* param = reinterpret_cast<uint16_t*>(q.param_ptrs[b]);
+  const uint16_t* dir = q.direction + b * q.numel;
+  const int64_t groups = q.numel / 8;
+  // A block owns runs of four consecutive 4 KiB pieces; a thread's four
+  // loads of the parameter and of the direction go out before its stores.
+  constexpr int kUnroll = 4;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kNormThreads * kUnroll;
+  for (int64_t g0 = static_cast<int64_t>(blockIdx.x) * kNormThreads * kUnroll + threadIdx.x; g0 < groups; g0 += stride) {
+    u32x4 praw[kUnroll], draw[kUnroll];
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+      const int64_t g = g0 + k * kNormThreads;
+      if (g < groups) {
+        praw[k] = load_stream_u32x4(param + g * 8);
+        draw[k] = load_stream_u32x4(dir + g * 8);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+      const int64_t g = g0 + k * kNormThreads;
+      if (g < groups) {
+        float pv[8], dv[8];
+        unpack8(praw[k], pv);
+        unpack8(draw[k], dv);
+        uint32_t pb[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pb[j] = muon_apply_one(pv[j], dv[j], q.decay, q.neg_lr, q.dir_scale);
+        store_stream_u32x4(param + g * 8, pack8(pb));
+      }
+    }
+  }
 }
 
 // Reads matrix b of `in` ([rows, cols]), divides by max(||.||_F, eps) as bf16
@@ -1011,7 +1135,16 @@ struct NsState {
   bool single;  // only X^T is carried from step to step (G = X X^T is then computed from its k-major rows)
 };
 
-int ns_begin(const fsh_ns_problem& q, int32_t steps, float eps, hipStream_t stream, NsState* st) {
+// Workspace offset of the [batch, 64] norm partials.
+int64_t ns_partial_offset(int64_t batch, int64_t rows, int64_t cols) {
+  const int64_t s = rows < cols ? rows : cols, l = rows < cols ? cols : rows;
+  return 2 * align256(batch * s * l * 2) + 2 * align256(batch * s * s * 2);
+}
+
+// `partials_ready`: the norm partials of x are in the workspace already (the
+// fused momentum kernel wrote them), so x is not read for its norm.
+int ns_begin(const fsh_ns_problem& q, int32_t steps, float eps, hipStream_t stream, NsState* st,
+             bool partials_ready = false) {
   const int64_t batch = q.batch, rows = q.rows, cols = q.cols;
   if (batch <= 0 || rows <= 0 || cols <= 0)
     return fail(FSH_EINVAL, "newton_schulz: bad sizes (batch %lld, rows %lld, cols %lld)", (long long)batch,
@@ -1052,9 +1185,11 @@ int ns_begin(const fsh_ns_problem& q, int32_t steps, float eps, hipStream_t stre
   st->cur = steps & 1;
   st->tall = tall;
 
-  hipLaunchKernelGGL(sumsq_partial_kernel, dim3(kNormBlocksPerMatrix, static_cast<uint32_t>(batch)),
-                     dim3(kNormThreads), 0, stream, x, rows * cols, partial);
-  if (int rc = check_launch("sumsq_partial_kernel")) return rc;
+  if (!partials_ready) {
+    hipLaunchKernelGGL(sumsq_partial_kernel, dim3(kNormBlocksPerMatrix, static_cast<uint32_t>(batch)),
+                       dim3(kNormThreads), 0, stream, x, rows * cols, partial);
+    if (int rc = check_launch("sumsq_partial_kernel")) return rc;
+  }
   // Input is [rows, cols]; "same orientation" output is X for a wide input
   // and X^T for a tall one.
   uint16_t* same = tall ? st->XT[st->cur] : st->X;
@@ -1118,20 +1253,8 @@ fsh_gemm_desc ns_product(const NsState& st, int which, float a, float b, float c
   return g;
 }
 
-}  // namespace
-}  // namespace fsh
-
-FSH_API int fsh_newton_schulz_multi(const fsh_ns_problem* problems, int32_t count, float a, float b, float c,
-                                    int32_t steps, float eps, void* stream_) {
-  using namespace fsh;
-  if (count < 0 || count > FSH_MAX_NS_PROBLEMS || (count > 0 && problems == nullptr))
-    return fail(FSH_EINVAL, "fsh_newton_schulz_multi: count %d outside [0, %d] or null list", count,
-                FSH_MAX_NS_PROBLEMS);
-  if (steps < 0) return fail(FSH_EINVAL, "fsh_newton_schulz_multi: negative step count %d", steps);
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
-  NsState st[FSH_MAX_NS_PROBLEMS];
-  for (int i = 0; i < count; ++i)
-    if (int rc = ns_begin(problems[i], steps, eps, stream, &st[i])) return rc;
+// The iteration proper for `count` normalized problems.
+int ns_iterate(NsState* st, int count, float a, float b, float c, int32_t steps, hipStream_t stream) {
   fsh_gemm_desc descs[FSH_MAX_NS_PROBLEMS];
   for (int step = 0; step < steps; ++step) {
     // The same product of every problem goes out together: problems are
@@ -1147,6 +1270,23 @@ FSH_API int fsh_newton_schulz_multi(const fsh_ns_problem* problems, int32_t coun
   return FSH_OK;
 }
 
+}  // namespace
+}  // namespace fsh
+
+FSH_API int fsh_newton_schulz_multi(const fsh_ns_problem* problems, int32_t count, float a, float b, float c,
+                                    int32_t steps, float eps, void* stream_) {
+  using namespace fsh;
+  if (count < 0 || count > FSH_MAX_NS_PROBLEMS || (count > 0 && problems == nullptr))
+    return fail(FSH_EINVAL, "fsh_newton_schulz_multi: count %d outside [0, %d] or null list", count,
+                FSH_MAX_NS_PROBLEMS);
+  if (steps < 0) return fail(FSH_EINVAL, "fsh_newton_schulz_multi: negative step count %d", steps);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  NsState st[FSH_MAX_NS_PROBLEMS];
+  for (int i = 0; i < count; ++i)
+    if (int rc = ns_begin(problems[i], steps, eps, stream, &st[i])) return rc;
+  return ns_iterate(st, count, a, b, c, steps, stream);
+}
+
 FSH_API int fsh_newton_schulz(void* x_dev, int64_t batch, int64_t rows, int64_t cols, float a, float b,
                               float c, int32_t steps, float eps, void* workspace_dev,
                               int64_t workspace_nbytes, void* stream_) {
@@ -1158,6 +1298,76 @@ FSH_API int fsh_newton_schulz(void* x_dev, int64_t batch, int64_t rows, int64_t 
   q.workspace_dev = workspace_dev;
   q.workspace_nbytes = workspace_nbytes;
   return fsh_newton_schulz_multi(&q, 1, a, b, c, steps, eps, stream_);
+}
+
+// One Muon step over whole matrices grouped by shape: momentum (fused with
+// the sum of squares), Newton-Schulz over all groups together, update.
+FSH_API int fsh_muon_step(const fsh_muon_group* groups, int32_t count, float lerp_weight, float nesterov_weight,
+                          int32_t nesterov, float decay_factor, float a, float b, float c, int32_t steps, float eps,
+                          void* stream_) {
+  using namespace fsh;
+  if (count < 0 || count > FSH_MAX_NS_PROBLEMS || (count > 0 && groups == nullptr))
+    return fail(FSH_EINVAL, "fsh_muon_step: count %d outside [0, %d] or null list", count, FSH_MAX_NS_PROBLEMS);
+  if (steps < 0) return fail(FSH_EINVAL, "fsh_muon_step: negative step count %d", steps);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  fsh_ns_problem problems[FSH_MAX_NS_PROBLEMS];
+  for (int i = 0; i < count; ++i) {
+    const fsh_muon_group& g = groups[i];
+    if (g.batch <= 0 || g.batch > 65535 || g.rows <= 0 || g.cols <= 0 || g.rows % 8 || g.cols % 8)
+      return fail(FSH_EINVAL, "fsh_muon_step: group %d has bad sizes (batch %lld, rows %lld, cols %lld; rows and cols "
+                  "must be multiples of 8)", i, (long long)g.batch, (long long)g.rows, (long long)g.cols);
+    if (!g.param_ptrs_dev || !g.grad_ptrs_dev || !g.momentum_ptrs_dev || !g.batch_dev || !g.workspace_dev)
+      return fail(FSH_EINVAL, "fsh_muon_step: group %d has a null pointer", i);
+    if (!aligned(g.batch_dev, 16) || !aligned(g.workspace_dev, 256))
+      return fail(FSH_EINVAL, "fsh_muon_step: group %d: batch buffer must be 16-byte and workspace 256-byte aligned", i);
+    if (g.workspace_nbytes < fsh_newton_schulz_workspace_bytes(g.batch, g.rows, g.cols))
+      return fail(FSH_EINVAL, "fsh_muon_step: group %d: workspace of %lld bytes, need %lld", i,
+                  (long long)g.workspace_nbytes, (long long)fsh_newton_schulz_workspace_bytes(g.batch, g.rows, g.cols));
+    problems[i].x_dev = g.batch_dev;
+    problems[i].batch = g.batch;
+    problems[i].rows = g.rows;
+    problems[i].cols = g.cols;
+    problems[i].workspace_dev = g.workspace_dev;
+    problems[i].workspace_nbytes = g.workspace_nbytes;
+  }
+  for (int i = 0; i < count; ++i) {
+    const fsh_muon_group& g = groups[i];
+    MuonPrepareBatch q;
+    q.momentum_ptrs = g.momentum_ptrs_dev;
+    q.grad_ptrs = g.grad_ptrs_dev;
+    q.out = static_cast<uint16_t*>(g.batch_dev);
+    q.partial = reinterpret_cast<float*>(static_cast<uint8_t*>(g.workspace_dev) +
+                                         ns_partial_offset(g.batch, g.rows, g.cols));
+    q.numel = g.rows * g.cols;
+    q.one_minus_mu = lerp_weight;
+    q.mu = nesterov_weight;
+    q.nesterov = nesterov;
+    hipLaunchKernelGGL(muon_prepare_sumsq_kernel, dim3(kNormBlocksPerMatrix, static_cast<uint32_t>(g.batch)),
+                       dim3(kNormThreads), 0, stream, q);
+    if (int rc = check_launch("muon_prepare_sumsq_kernel")) return rc;
+  }
+  NsState st[FSH_MAX_NS_PROBLEMS];
+  for (int i = 0; i < count; ++i)
+    if (int rc = ns_begin(problems[i], steps, eps, stream, &st[i], /*partials_ready=*/true)) return rc;
+  if (int rc = ns_iterate(st, count, a, b, c, steps, stream)) return rc;
+  for (int i = 0; i < count; ++i) {
+    const fsh_muon_group& g = groups[i];
+    MuonApplyBatch q;
+    q.param_ptrs = g.param_ptrs_dev;
+    q.direction = static_cast<const uint16_t*>(g.batch_dev);
+    q.numel = g.rows * g.cols;
+    q.decay = decay_factor;
+    q.neg_lr = g.neg_adjusted_lr;
+    q.dir_scale = g.direction_scale;
+    const int64_t groups8 = q.numel / 8;
+    const int64_t blocks = ceil_div(groups8, (int64_t)kNormThreads * 4);  // four 16-byte groups per thread
+    hipLaunchKernelGGL(muon_apply_batch_kernel,
+                       dim3(static_cast<uint32_t>(blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks)),
+                            static_cast<uint32_t>(g.batch)),
+                       dim3(kNormThreads), 0, stream, q);
+    if (int rc = check_launch("muon_apply_batch_kernel")) return rc;
+  }
+  return FSH_OK;
 }
 
 // ------------------------------------------------------------------------

@@ -166,17 +166,21 @@ class OwnedMuon:
         self.lr, self.weight_decay, self.momentum, self.nesterov = lr, weight_decay, momentum, nesterov
         self.ns_coefficients, self.ns_steps, self.eps, self.adjust_lr_fn = ns_coefficients, ns_steps, eps, adjust_lr_fn
         self.momentum_buffers = [torch.zeros_like(p) for p in self.params]
-        # One batch buffer and one Newton-Schulz workspace per matrix shape.
+        # Matrices of one shape are orthogonalized as one batch; the step's
+        # launch tables (address tables, batch buffers, workspaces) are built once.
         self._groups: dict[tuple[int, int], list[int]] = {}
         for index, p in enumerate(self.params):
             self._groups.setdefault(tuple(p.shape), []).append(index)
-        self._batch: dict[tuple[int, int], torch.Tensor] = {}
-        self._workspace: dict[tuple[int, int], torch.Tensor] = {}
-        for shape, members in self._groups.items():
-            device = self.params[members[0]].device
-            self._batch[shape] = torch.empty((len(members), *shape), dtype=torch.bfloat16, device=device)
-            need = hip_ops.newton_schulz_workspace_bytes(len(members), *shape)
-            self._workspace[shape] = torch.empty(need, dtype=torch.uint8, device=device)
+        self._plan = hip_ops.MuonStepPlan(
+            [
+                # whole parameters are their own learning-rate reference shape: direction scale 1
+                (shape, len(members), -_adjust_muon_learning_rate(lr, adjust_lr_fn, shape), 1.0)
+                for shape, members in self._groups.items()
+            ],
+            self.params[0].device,
+        )
+        self._batch = dict(zip(self._groups, self._plan.batches))
+        self._workspace = dict(zip(self._groups, self._plan.workspaces))
 
     def flops_per_step(self) -> int:
         return 2 * sum(
@@ -194,24 +198,17 @@ class OwnedMuon:
             if g.shape != p.shape:
                 raise ValueError(f"gradient shape {tuple(g.shape)} does not match parameter {tuple(p.shape)}")
         _require_bf16_gpu(*grads)
-        # Momentum for every matrix first, then one Newton-Schulz call over all
-        # shape groups (each product of the iteration is issued for all groups
-        # together), then the updates.
-        for shape, members in self._groups.items():
-            batch = self._batch[shape]
-            for slot, index in enumerate(members):
-                _prepare_muon_input(
-                    grads[index], self.momentum_buffers[index], momentum=self.momentum, nesterov=self.nesterov,
-                    out=batch[slot],
-                )
-        hip_ops.newton_schulz_multi(
-            [(self._batch[shape], self._workspace[shape]) for shape in self._groups],
-            self.ns_coefficients, self.ns_steps, self.eps,
+        # One C call: per shape group a momentum launch over all its matrices
+        # (which also leaves the sums of squares the normalization needs),
+        # Newton-Schulz with every product issued for all groups together, and
+        # an update launch per group.  Same bits as _prepare_muon_input ->
+        # _compute_muon_direction -> _apply_muon_update per matrix.
+        members = list(self._groups.values())
+        self._plan.step(
+            [[self.params[i] for i in group] for group in members],
+            [[self.momentum_buffers[i] for i in group] for group in members],
+            [[grads[i] for i in group] for group in members],
+            lerp_weight=1 - self.momentum, nesterov_weight=self.momentum, nesterov=self.nesterov,
+            decay_factor=1 - self.lr * self.weight_decay, coefficients=self.ns_coefficients, steps=self.ns_steps,
+            eps=self.eps,
         )
-        for shape, members in self._groups.items():
-            batch = self._batch[shape]
-            for slot, index in enumerate(members):
-                _apply_muon_update(
-                    self.params[index], batch[slot], lr=self.lr, weight_decay=self.weight_decay,
-                    adjust_lr_fn=self.adjust_lr_fn, compute_matrix_shape=shape,
-                )

@@ -2,9 +2,6 @@
 under a forward and a backward on one GPU."""
 
 from .bucket_comm import (
-    AsyncReduceGradResult,
-    AsyncUnshardResult,
-    ExplicitUnshardResult,
     ReduceGradHandle,
     StreamHandoff,
     UnshardHandle,
@@ -22,8 +19,7 @@ from .checkpoint import (
 from .bucket_runtime import BucketCommContext, BucketParam, BucketRuntime, PendingReduceGrad
 
 __all__ = [
-    "AsyncReduceGradResult", "AsyncUnshardResult", "BucketCommContext", "BucketParam", "BucketRuntime",
-    "ExplicitUnshardResult", "PendingReduceGrad", "ReduceGradHandle", "StreamHandoff", "UnshardHandle",
+    "BucketCommContext", "BucketParam", "BucketRuntime", "PendingReduceGrad", "ReduceGradHandle", "StreamHandoff", "UnshardHandle",
     "begin_bucket_unshard", "begin_explicit_bucket_unshard", "begin_reduce_grad", "copy_full_into_shard",
     "copy_shard_into_full", "get_flex_shard_global_layouts", "register_optimizer_checkpoint_hook",
     "set_state_dict_global_layouts",

@@ -30,7 +30,6 @@ from .bucket_comm import (
     ReduceGradHandle,
     UnshardHandle,
     begin_bucket_unshard,
-    begin_explicit_bucket_unshard,
     begin_reduce_grad,
 )
 
@@ -235,14 +234,9 @@ class BucketRuntime:
             if not self.infos[0].placement.refills_persistent_buffers_in_finish:
                 self._alloc_persistent_storage()
             persistent_buffers = self.persistent_buffers
-        if on_current_stream:
-            return begin_explicit_bucket_unshard(
-                self._local_shards(), self.infos, self.mesh, async_op=async_op, debug_fqn=self.debug_fqn,
-                persistent_buffers=persistent_buffers,
-            )
         return begin_bucket_unshard(
-            self._local_shards(), self.infos, self.mesh, self.context.unshard_stream, debug_fqn=self.debug_fqn,
-            persistent_buffers=persistent_buffers,
+            self._local_shards(), self.infos, self.mesh, None if on_current_stream else self.context.unshard_stream,
+            debug_fqn=self.debug_fqn, persistent_buffers=persistent_buffers, async_op=async_op and on_current_stream,
         )
 
     def finish_unshard(self, result: UnshardHandle) -> None:

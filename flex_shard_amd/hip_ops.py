@@ -31,7 +31,7 @@ from ._native import (
 __all__ = [
     "DT_BF16", "DT_F32", "EPS_FP32", "EPS_INPUT_DTYPE", "REDUCE_POSTDIV", "REDUCE_POSTMUL",
     "REDUCE_PREMUL", "REDUCE_SUM", "SRC_BF16", "SRC_F32", "SRC_F32_AS_BF16",
-    "QuantChunkSpec", "QuantPackPlan", "accumulate_grad", "act_quant_128x1_transposed", "act_quant_1x128",
+    "MuonStepPlan", "QuantChunkSpec", "QuantPackPlan", "accumulate_grad", "act_quant_128x1_transposed", "act_quant_1x128",
     "copy_segments", "fp8_gemm_1x128_128x1", "fp8_gemm_1x128_128x128", "fp8_gemm_1x128_128x128_dgrad",
     "fp8_transpose", "gemm_nt", "gemm_nt_group", "muon_apply", "muon_prepare", "newton_schulz_multi",
     "newton_schulz", "newton_schulz_noalloc", "newton_schulz_workspace_bytes", "pack_segments", "quantize_pack",
@@ -645,3 +645,83 @@ def muon_apply(
         stream_ptr(param.device),
     )
     _native.check(status, "fsh_muon_apply")
+
+
+class MuonStepPlan:
+    """The launch tables of ``fsh_muon_step`` for the whole matrices of an
+    optimizer: per shape group three device tables of addresses (parameters,
+    momentum buffers, gradients), a contiguous batch buffer and the
+    Newton-Schulz workspace.  The address tables are checked on every step and
+    re-uploaded only when a tensor moved (gradients usually do, parameters and
+    momentum buffers usually do not)."""
+
+    def __init__(self, groups: Sequence[tuple[tuple[int, int], int, float, float]], device: torch.device) -> None:
+        """``groups``: per shape group (shape, matrix count, neg_adjusted_lr,
+        direction_scale)."""
+        if not groups:
+            raise ValueError("a Muon step needs at least one group")
+        if len(groups) > _native.MAX_NS_PROBLEMS:
+            raise NotImplementedError(f"at most {_native.MAX_NS_PROBLEMS} shape groups per step")
+        if device.type != "cuda":
+            raise RuntimeError("flex_shard_amd kernels run on the GPU only; there is no CPU path.")
+        self._device = device
+        self._table = (_native.MuonGroup * len(groups))()
+        self._shapes: list[tuple[int, int]] = []
+        self._address_tables: list[list[tuple[torch.Tensor, list[int]]]] = []
+        self.batches: list[torch.Tensor] = []
+        self.workspaces: list[torch.Tensor] = []
+        for slot, (shape, n, neg_lr, scale) in zip(self._table, groups):
+            if len(shape) != 2 or shape[0] % 8 or shape[1] % 8 or n <= 0:
+                raise NotImplementedError(f"whole matrices with rows and cols multiples of 8, got {n} x {tuple(shape)}")
+            batch = torch.empty((n, *shape), dtype=torch.bfloat16, device=device)
+            workspace = torch.empty(newton_schulz_workspace_bytes(n, *shape), dtype=torch.uint8, device=device)
+            tables = [(torch.zeros(n, dtype=torch.int64, device=device), [0] * n) for _ in range(3)]
+            self.batches.append(batch)
+            self.workspaces.append(workspace)
+            self._shapes.append(tuple(shape))
+            self._address_tables.append(tables)
+            slot.param_ptrs_dev, slot.momentum_ptrs_dev, slot.grad_ptrs_dev = (t.data_ptr() for t, _ in tables)
+            slot.batch_dev, slot.batch, slot.rows, slot.cols = batch.data_ptr(), n, shape[0], shape[1]
+            slot.workspace_dev, slot.workspace_nbytes = workspace.data_ptr(), workspace.numel()
+            slot.neg_adjusted_lr, slot.direction_scale = neg_lr, scale
+
+    def _refresh(self, table: torch.Tensor, current: list[int], tensors: Sequence[torch.Tensor], shape) -> None:
+        if len(tensors) != len(current):
+            raise ValueError(f"expected {len(current)} matrices of shape {shape}, got {len(tensors)}")
+        addresses = []
+        for t in tensors:
+            if t.device != self._device:
+                raise ValueError(f"all matrices of a Muon step must live on {self._device}, got {t.device}")
+            if t.dtype != torch.bfloat16 or not t.is_contiguous() or tuple(t.shape) != shape:
+                raise ValueError(f"the Muon step kernels need contiguous bf16 matrices of shape {shape}")
+            if t.data_ptr() % 16:
+                raise ValueError("the Muon step kernels need 16-byte aligned matrices")
+            addresses.append(t.data_ptr())
+        if addresses != current:
+            # A fresh pinned staging tensor per change: torch's host allocator
+            # keeps its block from reuse until the queued copy has read it, so
+            # nothing here waits for the GPU.
+            table.copy_(torch.tensor(addresses, dtype=torch.int64, pin_memory=True), non_blocking=True)
+            current[:] = addresses
+
+    def step(
+        self, params: Sequence[Sequence[torch.Tensor]], momenta: Sequence[Sequence[torch.Tensor]],
+        grads: Sequence[Sequence[torch.Tensor]], *, lerp_weight: float, nesterov_weight: float, nesterov: bool,
+        decay_factor: float, coefficients: tuple[float, float, float], steps: int, eps: float,
+    ) -> None:
+        """Per group: the parameters, their momentum buffers and their
+        gradients, one of each per matrix, in the same order.  All three are
+        read (and the first two written) by kernels queued on the current
+        stream."""
+        for name, lists in (("parameter", params), ("momentum", momenta), ("gradient", grads)):
+            if len(lists) != len(self._shapes):
+                raise ValueError(f"expected {name} lists for {len(self._shapes)} groups, got {len(lists)}")
+        for tables, shape, p, m, g in zip(self._address_tables, self._shapes, params, momenta, grads):
+            for (table, current), tensors in zip(tables, (p, m, g)):
+                self._refresh(table, current, tensors, shape)
+        a, b, c = coefficients
+        status = _native.lib().fsh_muon_step(
+            self._table, len(self._shapes), lerp_weight, nesterov_weight, 1 if nesterov else 0, decay_factor, a, b, c,
+            steps, eps, stream_ptr(self._device),
+        )
+        _native.check(status, "fsh_muon_step")

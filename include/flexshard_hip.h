@@ -344,6 +344,36 @@ int fsh_fp8_gemm_1x128_128x1(const void* aq_dev, const float* as_dev, const void
                              const float* bs_dev, void* out_dev, int64_t m, int64_t n, int64_t k,
                              int64_t ldaq, int64_t ldbq, int64_t ldo, void* stream);
 
+/* ------------------------------------------------------------------------
+ * 10. One whole Muon step over matrices grouped by shape, for an owner's whole
+ * parameters (the comm-free step of dist_muon/_optimizer_reshard_runtime.py
+ * :645-661): dist_muon/optimizer.py:2049-2068 (momentum, Nesterov), :2120-2151
+ * (Newton-Schulz) and :2100-2117 (decayed update), i.e. fsh_muon_prepare,
+ * fsh_newton_schulz_multi and fsh_muon_apply in sequence, with the same
+ * results bit for bit.  Per group there is one momentum launch for all its
+ * matrices (it also leaves the sums of squares the normalization needs, so
+ * the Newton-Schulz input is read once less) and one update launch.
+ * The parameters, gradients and momentum buffers of a group are separate
+ * allocations, named by device tables of their addresses; each must be a
+ * contiguous bf16 [rows, cols] matrix at a 16-byte aligned address.
+ * batch_dev is scratch of batch*rows*cols bf16: it holds the momentum
+ * output, then the orthogonalized direction.
+ * ---------------------------------------------------------------------- */
+typedef struct fsh_muon_group {
+  const int64_t* param_ptrs_dev;    /* [batch] addresses of the parameters, updated in place   */
+  const int64_t* grad_ptrs_dev;     /* [batch] addresses of the gradients                      */
+  const int64_t* momentum_ptrs_dev; /* [batch] addresses of the momentum buffers, updated      */
+  void* batch_dev;                  /* [batch, rows, cols] bf16 scratch                        */
+  int64_t batch, rows, cols;        /* rows, cols multiples of 8                               */
+  void* workspace_dev;              /* >= fsh_newton_schulz_workspace_bytes(batch, rows, cols) */
+  int64_t workspace_nbytes;
+  float neg_adjusted_lr;            /* -lr * shape factor of dist_muon/optimizer.py:2031-2046  */
+  float direction_scale;            /* 1, or ratio / reference_ratio of :2082-2097             */
+} fsh_muon_group;
+int fsh_muon_step(const fsh_muon_group* groups, int32_t count, float lerp_weight /* 1 - mu */,
+                  float nesterov_weight /* mu */, int32_t nesterov, float decay_factor /* 1 - lr*wd */, float a,
+                  float b, float c, int32_t steps, float eps, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -781,3 +781,41 @@ def test_owned_muon_step_config5_matches_reference_step(device, golden):
     assert opt.flops_per_step() == 2 * (
         _estimate_muon_compute_cost((24, 7168, 2048), 5) + _estimate_muon_compute_cost((24, 2048, 2048), 5)
     )
+
+
+@pytest.mark.parametrize("nesterov", [True, False])
+def test_fused_muon_step_equals_the_per_matrix_kernels(device, nesterov):
+    """OwnedMuon.step is one fsh_muon_step call (batched momentum kernel that
+    also leaves the norm partials, Newton-Schulz over all groups, batched
+    update).  It must give the bits of the per-matrix sequence
+    _prepare_muon_input -> newton_schulz_multi -> _apply_muon_update: wide,
+    tall and small matrices, a batch large enough for the large-tile
+    one-orientation flow, two steps (the second with momentum in place and
+    gradients at new addresses)."""
+    shapes = [(1024, 1280)] * 20 + [(768, 256)] * 3 + [(64, 96)] + [(256, 256)] * 2
+    start = [seeded_normal(s, 0.02, 700 + i, device) for i, s in enumerate(shapes)]
+    mine = [p.clone() for p in start]
+    theirs = [p.clone() for p in start]
+    opt = OwnedMuon(mine, nesterov=nesterov, lr=2e-3, weight_decay=0.05)
+    momenta = [torch.zeros_like(p) for p in theirs]
+    groups: dict[tuple[int, int], list[int]] = {}
+    for i, s in enumerate(shapes):
+        groups.setdefault(s, []).append(i)
+    for step in range(2):
+        grads = [seeded_normal(s, 1.0, 800 + 100 * step + i, device) for i, s in enumerate(shapes)]
+        opt.step(grads)
+        batches = {s: torch.empty((len(m), *s), dtype=torch.bfloat16, device=device) for s, m in groups.items()}
+        for s, members in groups.items():
+            for slot, i in enumerate(members):
+                _prepare_muon_input(grads[i], momenta[i], momentum=0.95, nesterov=nesterov, out=batches[s][slot])
+        hip_ops.newton_schulz_multi([(batches[s], None) for s in groups], COEFFS, 5, 1e-7)
+        for s, members in groups.items():
+            for slot, i in enumerate(members):
+                _apply_muon_update(theirs[i], batches[s][slot], lr=2e-3, weight_decay=0.05, adjust_lr_fn=None,
+                                   compute_matrix_shape=s)
+        for i in range(len(shapes)):
+            assert torch.equal(opt.momentum_buffers[i], momenta[i]), f"momentum {i} differs at step {step}"
+            assert torch.equal(mine[i], theirs[i]), f"parameter {i} differs at step {step}"
+        for s in groups:
+            assert torch.equal(opt._batch[s], batches[s])
+    assert not torch.equal(mine[0], start[0])
