@@ -332,15 +332,24 @@ struct HalfTileEpilogue {
   static constexpr int kLdsBytes = Cfg::WM * Cfg::WN * kRegion;
 };
 
-template <typename Cfg>
-__device__ inline void store_tile_in_halves(const GemmParams& p, int64_t batch, int64_t m0, int64_t n0, int wm, int wn,
-                                            int lane, bool mirror, const f32x16 (&acc)[Cfg::TM][Cfg::TN],
-                                            uint8_t* staging) {
+// kMode fixes the flags that every final depends on, so that the 256 finals
+// of a lane are straight-line code (with the flags read at run time the
+// compiler keeps a branch per group of four finals, and the waits at every
+// join serialize the epilogue):
+//   kEpiGeneric  any combination, flags read at run time
+//   kEpiPlain    C = bf16(acc): no D, no diagonal term, alpha == 1
+//   kEpiPoly     C = bf16(fma(beta, D, alpha * acc) + diag): D, alpha and the diagonal term
+constexpr int kEpiGeneric = 0, kEpiPlain = 1, kEpiPoly = 2;
+
+template <typename Cfg, int kMode>
+__device__ inline void store_tile_in_halves_as(const GemmParams& p, int64_t batch, int64_t m0, int64_t n0, int wm,
+                                               int wn, int lane, bool mirror, const f32x16 (&acc)[Cfg::TM][Cfg::TN],
+                                               uint8_t* staging) {
   using Epi = HalfTileEpilogue<Cfg>;
   using R = DRows<Cfg>;
   constexpr int TM = Cfg::TM, TN = Cfg::TN, HM = TM / 2;
   static_assert(TM % 2 == 0 && Epi::kRows == HM * 32, "two halves of whole 32-row blocks");
-  const bool has_d = p.D != nullptr;
+  const bool has_d = kMode == kEpiPlain ? false : kMode == kEpiPoly ? true : p.D != nullptr;
   uint16_t* C = p.C + batch * p.sC;
   // A symmetric product mirrors its off-diagonal tiles into the lower triangle.
   uint16_t* Ct = mirror ? C : (p.Ct ? p.Ct + batch * p.sCt : nullptr);
@@ -348,10 +357,10 @@ __device__ inline void store_tile_in_halves(const GemmParams& p, int64_t batch, 
   const int64_t wave_row = m0 + wm * Cfg::kWaveM, wave_col = n0 + wn * Cfg::kWaveN;
   uint8_t* region = staging + (wm * Cfg::WN + wn) * Epi::kRegion;
   const int r_lane = lane & 31, h = lane >> 5;
-  const bool unit_alpha = p.alpha == 1.0f;
+  const bool unit_alpha = kMode == kEpiPlain ? true : kMode == kEpiPoly ? false : p.alpha == 1.0f;
   // Block tiles and wave sub-tiles are square, so C's diagonal runs through
   // the (i, i) blocks of the diagonal sub-tiles of the diagonal tiles.
-  const bool on_diagonal = p.diag_add != 0.0f && m0 == n0 && wm == wn;
+  const bool on_diagonal = kMode != kEpiPlain && p.diag_add != 0.0f && m0 == n0 && wm == wn;
 
   // The lower half of D is requested once the upper half has left its
   // registers for LDS, and lands while the upper half is worked on.
@@ -397,10 +406,11 @@ __device__ inline void store_tile_in_halves(const GemmParams& p, int64_t batch, 
             v[2] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].y << 16), v[2]);
             v[3] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].y & 0xFFFF0000u), v[3]);
           }
-          if (on_diagonal && i == j) {
+          if (kMode != kEpiPlain && i == j) {
+            // a select per final rather than a branch per block (adding zero
+            // elsewhere would turn a -0 into +0)
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
-              if (r_lane == 8 * b + 4 * h + t) v[t] += p.diag_add;
+            for (int t = 0; t < 4; ++t) v[t] = (on_diagonal && r_lane == 8 * b + 4 * h + t) ? v[t] + p.diag_add : v[t];
           }
           fin[j][b] = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
         }
@@ -453,6 +463,20 @@ __device__ inline void store_tile_in_halves(const GemmParams& p, int64_t batch, 
   }
 }
 
+template <typename Cfg>
+__device__ inline void store_tile_in_halves(const GemmParams& p, int64_t batch, int64_t m0, int64_t n0, int wm, int wn,
+                                            int lane, bool mirror, const f32x16 (&acc)[Cfg::TM][Cfg::TN],
+                                            uint8_t* staging) {
+  // uniform over the launch's problem, so one branch per tile
+  const bool has_d = p.D != nullptr, diag = p.diag_add != 0.0f, unit_alpha = p.alpha == 1.0f;
+  if (!has_d && !diag && unit_alpha)
+    store_tile_in_halves_as<Cfg, kEpiPlain>(p, batch, m0, n0, wm, wn, lane, mirror, acc, staging);
+  else if (has_d && !unit_alpha)
+    store_tile_in_halves_as<Cfg, kEpiPoly>(p, batch, m0, n0, wm, wn, lane, mirror, acc, staging);
+  else
+    store_tile_in_halves_as<Cfg, kEpiGeneric>(p, batch, m0, n0, wm, wn, lane, mirror, acc, staging);
+}
+
 // Scheduling-group masks of __builtin_amdgcn_sched_group_barrier.
 constexpr int kSchedValu = 0x002, kSchedMfma = 0x008, kSchedVmemRead = 0x020, kSchedDsRead = 0x100, kSchedDsWrite = 0x200;
 
@@ -464,8 +488,7 @@ __device__ inline void dma_load_16(uint32_t voffset, const uint8_t* base, uint32
   asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voffset), "s"(base), "s"(lds_addr) : "memory");
 }
 __device__ inline void wait_for_dma_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-// The 4-byte form, used only to pull a cache line towards L2 ahead of time:
-// the data lands in a scrap LDS area nobody reads, so no register is tied up.
+// The 4-byte form: lane l writes LDS bytes [M0 + 4 l, M0 + 4 l + 4).
 __device__ inline void dma_touch_4(uint32_t voffset, const uint8_t* base, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" ::"v"(voffset), "s"(base), "s"(lds_addr) : "memory");
 }

@@ -365,11 +365,12 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_nt_interior_kernel(const G
 // reorders nor counts; everything else in the loop is compiler-visible and is
 // pinned around them with sched_barrier.
 //
-// The part does not hold its peak clock under this kernel (about 1.65 GHz by
-// the MFMA-busy counters against the delivered rate).  Operand requests
-// complete in order, so a k-tile waits for its slowest line: kTouchAhead
-// k-tiles ahead every line of both operand tiles is asked for once (4 bytes
-// into a scrap area), which brings it into L2 before the real request.
+// The part does not hold its peak clock under this kernel (1.5-1.6 GHz on
+// random operands, 2.3 GHz on zeros, by the shader-clock counter against the
+// 100 MHz one).  Cycle counters in the loop put under 5 % of a k-tile into the
+// wait for operands and the barrier together; asking for every operand line
+// once more, a few k-tiles ahead, to pull it into L2 (4-byte requests into a
+// scrap area) made all three products 2-5 % slower and is gone.
 struct DmaGemm {
   static constexpr int BM = 256, BN = 256, BK = 64, WM = 2, WN = 2, TM = 4, TN = 4;
   static constexpr int kThreads = 256, kWaveM = 128, kWaveN = 128, KS = BK / 16;
@@ -378,14 +379,11 @@ struct DmaGemm {
   static constexpr int kStageBytes = 2 * kOperandBytes;      // 64 KB
   static constexpr int kLoopLdsBytes = 2 * kStageBytes;
   static constexpr int kLoadsPerOperand = BM / 8 / 4;        // wave-level 1 KB loads per wave: 8
-  static constexpr int kTouchAhead = 3;                      // k-tiles between an L2 touch and the MFMAs on its data
-  static constexpr int kScrapBytes = 1024;                   // landing area of the touches, 256 B per wave
 };
 
 // LDS of the kernel: two operand stages, the epilogue's staging region from
-// stage 1 upward, and the touches' scrap area at the very end.
-constexpr int kDmaGemmLdsBytes =
-    DmaGemm::kStageBytes + max_int(DmaGemm::kStageBytes, HalfTileEpilogue<DmaGemm>::kLdsBytes) + DmaGemm::kScrapBytes;
+// stage 1 upward.
+constexpr int kDmaGemmLdsBytes = DmaGemm::kStageBytes + max_int(DmaGemm::kStageBytes, HalfTileEpilogue<DmaGemm>::kLdsBytes);
 
 // kPersistent: the grid is one workgroup per compute unit and workgroup g
 // takes the ids g, g + gridDim.x, ... of the launch (the same XCD every time,
@@ -503,7 +501,6 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
 #pragma unroll
     for (int j = 0; j < TN; ++j) b_frag_km[j] = Cfg::kOperandBytes + common + wn * 256 + ((j ^ (t >> 2)) * 64);
   }
-  constexpr int scrap_offset = kDmaGemmLdsBytes - Cfg::kScrapBytes;
 
   f32x16 acc[TM][TN];
   bf16x8 af[2][TM], bf[2][TN];
@@ -565,16 +562,11 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   //   k steps 0 .. KS-2: MFMAs while the next step's fragments are read
   //   wait for kt + 1, barrier
   //   k step KS-1: one MFMA, one fragment read of (kt + 1, 0), one pair of
-  //              requests for kt + 2 at a time, then the L2 touches
-  // L2 touches: two k-tiles ahead of the requested one, each lane asks for
-  // 4 bytes of one operand row (one 128-byte line each: 256 rows of A and of
-  // B = two requests per wave) into a scrap area, which brings the lines into
-  // L2 early.  They are issued after the real requests and may still be in
-  // flight when those are waited for (requests complete in order).
-  // (k-major: 64 rows of four lines each; thread t asks for line t & 3 of row t >> 2.)
-  const uint32_t touch_row = static_cast<uint32_t>(kKMajor ? (64 * wave + lane) >> 2 : 64 * wave + lane);
-  const uint32_t touch_col = static_cast<uint32_t>(kKMajor ? (lane & 3) * 128 : 0);
-  const uint32_t scrap_lds = lds_base + static_cast<uint32_t>(scrap_offset + wave * 256);
+  //              requests for kt + 2 at a time
+#ifdef FSH_TRACE
+  uint64_t trace_wait = 0, trace_barrier = 0, trace_ktiles = 0, trace_tile_wait = 0, trace_tile_barrier = 0, trace_tiles = 0, trace_kloop = 0, trace_epi = 0;
+  const uint64_t trace_begin = __builtin_amdgcn_s_memtime();
+#endif
   auto k_tile = [&](int64_t kt, int64_t ktiles, auto more_tag) {
     constexpr bool more = decltype(more_tag)::value;
     const int stage_off = static_cast<int>(kt & 1) * Cfg::kStageBytes;
@@ -590,12 +582,22 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
         __builtin_amdgcn_sched_group_barrier(kSchedMfma, TM * TN / (TM + TN), 0);
       }
     }
+#ifdef FSH_TRACE
+    const uint64_t tr0 = __builtin_amdgcn_s_memtime();
+#endif
     if (more) {  // this wave's part of the next tile has landed
-      // touches followed its requests iff the k-tile before this one issued them
-      if (kt >= 1 && kt + Cfg::kTouchAhead < ktiles) wait_for_dma_loads_except<2>();
-      else wait_for_dma_loads();
+      wait_for_dma_loads();
     }
+#ifdef FSH_TRACE
+    const uint64_t tr1 = __builtin_amdgcn_s_memtime();
+#endif
     __syncthreads();
+#ifdef FSH_TRACE
+    const uint64_t tr2 = __builtin_amdgcn_s_memtime();
+    trace_wait += tr1 - tr0;
+    trace_barrier += tr2 - tr1;
+    trace_ktiles += 1;
+#endif
     const bool more2 = more && kt + 2 < ktiles;
     const uint8_t* a_next = k_tile_ptr(Ab, a_row_bytes, kt + 2);
     const uint8_t* b_next = k_tile_ptr(Bb, b_row_bytes, kt + 2);
@@ -609,10 +611,6 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
       if (more2 && g % 2 == 0) issue_tile_load(a_next, b_next, a_row_bytes, b_row_bytes, stage_off, g / 2, g / 2 + 1);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (more2 && kt + 1 + Cfg::kTouchAhead < ktiles) {
-      dma_touch_4(touch_row * a_row_bytes + touch_col, k_tile_ptr(Ab, a_row_bytes, kt + 1 + Cfg::kTouchAhead), scrap_lds);
-      dma_touch_4(touch_row * b_row_bytes + touch_col, k_tile_ptr(Bb, b_row_bytes, kt + 1 + Cfg::kTouchAhead), scrap_lds);
-    }
   };
 
   while (true) {
@@ -625,9 +623,21 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
     FSH_STAMP(6);
+#ifdef FSH_TRACE
+    const uint64_t ts0 = __builtin_amdgcn_s_memtime();
+#endif
     wait_for_dma_loads();
     FSH_STAMP(7);
+#ifdef FSH_TRACE
+    const uint64_t ts1 = __builtin_amdgcn_s_memtime();
+#endif
     __syncthreads();  // also: every wave has left the previous tile's epilogue
+#ifdef FSH_TRACE
+    trace_tile_wait += ts1 - ts0;
+    trace_tile_barrier += __builtin_amdgcn_s_memtime() - ts1;
+    trace_tiles += 1;
+    const uint64_t tk0 = __builtin_amdgcn_s_memtime();
+#endif
     read_frags(0, 0, 0);
     if (ktiles > 1)
       issue_tile_load(k_tile_ptr(Ab, a_row_bytes, 1), k_tile_ptr(Bb, b_row_bytes, 1), a_row_bytes, b_row_bytes,
@@ -637,6 +647,9 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
     for (int64_t kt = 0; kt + 1 < ktiles; ++kt) k_tile(kt, ktiles, std::true_type{});
     k_tile(ktiles - 1, ktiles, std::false_type{});
     FSH_STAMP(3);
+#ifdef FSH_TRACE
+    trace_kloop += __builtin_amdgcn_s_memtime() - tk0;
+#endif
 
     // Both stages are free now.  The next tile's first operands go to stage 0
     // while the epilogue stages its output beside it, from stage 1 upward.
@@ -655,12 +668,31 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
         issue_tile_load(Ab, Bb, a_row_bytes, b_row_bytes, 0, 0, Cfg::kLoadsPerOperand);
       }
     }
+#ifdef FSH_TRACE
+    const uint64_t te0 = __builtin_amdgcn_s_memtime();
+#endif
     store_tile_in_halves<Cfg>(p, batch, static_cast<int64_t>(tm) * Cfg::BM, static_cast<int64_t>(tn) * Cfg::BN, wm,
                               wn, lane, p.symmetric && tm != tn, acc, lds_bytes + Cfg::kStageBytes);
-    FSH_STAMP(4);
 #ifdef FSH_TRACE
+    trace_epi += __builtin_amdgcn_s_memtime() - te0;
+#endif
+    FSH_STAMP(4);
+#if defined(FSH_TRACE) && !defined(FSH_TRACE_NODRAIN)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     FSH_STAMP(5);
+#endif
+#ifdef FSH_TRACE
+    if (!have_next && p.trace && threadIdx.x == 0) {
+      p.trace[blockIdx.x * 16 + 12] = __builtin_amdgcn_s_memtime() - trace_begin;
+      p.trace[blockIdx.x * 16 + 13] = trace_wait;
+      p.trace[blockIdx.x * 16 + 14] = trace_barrier;
+      p.trace[blockIdx.x * 16 + 15] = trace_ktiles;
+      p.trace[blockIdx.x * 16 + 8] = trace_tile_wait;
+      p.trace[blockIdx.x * 16 + 9] = trace_tile_barrier;
+      p.trace[blockIdx.x * 16 + 10] = trace_tiles;
+      p.trace[blockIdx.x * 16 + 11] = trace_kloop;
+      p.trace[blockIdx.x * 16 + 7] = trace_epi;
+    }
 #endif
     if (!have_next) break;
     which = next_which;
