@@ -492,15 +492,6 @@ __device__ inline void wait_for_dma_loads() { asm volatile("s_waitcnt vmcnt(0)" 
 __device__ inline void dma_touch_4(uint32_t voffset, const uint8_t* base, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" ::"v"(voffset), "s"(base), "s"(lds_addr) : "memory");
 }
-// Loads return in issue order: with `younger` requests issued after the ones
-// of interest, those are complete once at most `younger` are outstanding.
-template <int younger>
-__device__ inline void wait_for_dma_loads_except() {
-  static_assert(younger == 2 || younger == 13 || younger == 14, "one immediate per use");
-  if (younger == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-  else if (younger == 13) asm volatile("s_waitcnt vmcnt(13)" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(14)" ::: "memory");
-}
 
 constexpr int max_int(int a, int b) { return a > b ? a : b; }
 

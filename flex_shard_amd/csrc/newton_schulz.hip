@@ -439,10 +439,10 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   // [32 q + 8 wave, +8); lane l fills slot l & 7 of row l >> 3 there.
   // (k-major: load q fills k-rows [8 q + 2 wave, +2); lane l fills slot
   // l & 31 of row l >> 5 there.)
-  const int fill_row = kKMajor ? lane >> 5 : lane >> 3;
-  const uint32_t fill_row0 = static_cast<uint32_t>((kKMajor ? 2 : 8) * wave + fill_row);
-  const int fill_chunk = kKMajor ? (lane & 31) ^ (4 * static_cast<int>(fill_row0 & 3))
-                                 : (lane & 7) ^ static_cast<int>((fill_row0 >> 1) & 7);
+  // (The per-lane values of both sides are derived from the lane number again
+  // at the start of every tile, see derive_lane_values below.)
+  uint32_t fill_row0 = 0;
+  int fill_chunk = 0;
   constexpr uint32_t kRowsPerLoadStep = kKMajor ? 8 : 32;
   // M0 takes the LDS byte address relative to the workgroup's allocation.
   typedef __attribute__((address_space(3))) uint8_t* lds_address;
@@ -461,11 +461,13 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   };
   auto issue_tile_load = [&](const uint8_t* a_src, const uint8_t* b_src, uint32_t a_row_bytes, uint32_t b_row_bytes,
                              int stage_off, int q_first, int q_last) {
+    // The part of the address that depends on q goes into the scalar base, so
+    // that one lane offset per operand serves all eight loads.
+    const uint32_t a_voff = fill_row0 * a_row_bytes + fill_chunk * 16, b_voff = fill_row0 * b_row_bytes + fill_chunk * 16;
 #pragma unroll
     for (int q = q_first; q < q_last; ++q) {
-      dma_load_16((fill_row0 + kRowsPerLoadStep * q) * a_row_bytes + fill_chunk * 16, a_src,
-                  stage_off + fill_lds + q * 4096);
-      dma_load_16((fill_row0 + kRowsPerLoadStep * q) * b_row_bytes + fill_chunk * 16, b_src,
+      dma_load_16(a_voff, a_src + static_cast<uint64_t>(kRowsPerLoadStep * q) * a_row_bytes, stage_off + fill_lds + q * 4096);
+      dma_load_16(b_voff, b_src + static_cast<uint64_t>(kRowsPerLoadStep * q) * b_row_bytes,
                   stage_off + Cfg::kOperandBytes + fill_lds + q * 4096);
     }
   };
@@ -478,29 +480,39 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   // Fragment side.  Lane l reads row l & 31 of a 32-row block, k chunk
   // 2 ks + (l >> 5); its slot is that chunk XOR ((row >> 1) & 7), i.e. the
   // ks = 0 address with bits 5..6 flipped by ks.
-  const int frag_row = lane & 31;
-  const uint32_t frag_base =
-      static_cast<uint32_t>(frag_row * Cfg::kRowBytes + (((lane >> 5) ^ ((frag_row >> 1) & 7)) * 16));
   uint32_t a_frag[KS], b_frag[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    a_frag[ks] = (frag_base ^ (ks * 32)) + wm * Cfg::kWaveM * Cfg::kRowBytes;
-    b_frag[ks] = (frag_base ^ (ks * 32)) + Cfg::kOperandBytes + wn * Cfg::kWaveN * Cfg::kRowBytes;
-  }
   // k-major fragments: lane l = 16 g + t of a wave serves output row
   // 16 (g & 1) + t of a 32-row block and the k octet g >> 1 of a k step; it
   // passes the address of columns 4 (t & 3) .. + 3 of k-row (t >> 2) of its
   // octet's first half, then of its second half (4 rows = 2048 bytes down).
   // The block index enters the slot through the swizzle: i ^ (k-row & 3).
   uint32_t a_frag_km[TM], b_frag_km[TN];
-  {
-    const int t = lane & 15, g = lane >> 4;
+  // All per-lane addresses of the k loop, from the lane number.  Called with
+  // a lane number the compiler cannot see through at the start of every tile:
+  // the values then live from there to the end of the k loop only.  Kept
+  // across the epilogue (which needs every register it can get), the compiler
+  // spilled some of them and reloaded them inside the k loop, and a reload is
+  // a vector memory load: the wait for it also waited for every operand
+  // request in flight.
+  auto derive_lane_values = [&](int l) {
+    const int fill_row = kKMajor ? l >> 5 : l >> 3;
+    fill_row0 = static_cast<uint32_t>((kKMajor ? 2 : 8) * wave + fill_row);
+    fill_chunk = kKMajor ? (l & 31) ^ (4 * static_cast<int>(fill_row0 & 3)) : (l & 7) ^ static_cast<int>((fill_row0 >> 1) & 7);
+    const int frag_row = l & 31;
+    const uint32_t frag_base = static_cast<uint32_t>(frag_row * Cfg::kRowBytes + (((l >> 5) ^ ((frag_row >> 1) & 7)) * 16));
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      a_frag[ks] = (frag_base ^ (ks * 32)) + wm * Cfg::kWaveM * Cfg::kRowBytes;
+      b_frag[ks] = (frag_base ^ (ks * 32)) + Cfg::kOperandBytes + wn * Cfg::kWaveN * Cfg::kRowBytes;
+    }
+    const int t = l & 15, g = l >> 4;
     const uint32_t common = static_cast<uint32_t>(((g >> 1) * 8 + (t >> 2)) * 512 + (g & 1) * 32 + (t & 3) * 8);
 #pragma unroll
     for (int i = 0; i < TM; ++i) a_frag_km[i] = common + wm * 256 + ((i ^ (t >> 2)) * 64);
 #pragma unroll
     for (int j = 0; j < TN; ++j) b_frag_km[j] = Cfg::kOperandBytes + common + wn * 256 + ((j ^ (t >> 2)) * 64);
-  }
+  };
+  derive_lane_values(lane);
 
   f32x16 acc[TM][TN];
   bf16x8 af[2][TM], bf[2][TN];
@@ -564,15 +576,51 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   //   k step KS-1: one MFMA, one fragment read of (kt + 1, 0), one pair of
   //              requests for kt + 2 at a time
 #ifdef FSH_TRACE
-  uint64_t trace_wait = 0, trace_barrier = 0, trace_ktiles = 0, trace_tile_wait = 0, trace_tile_barrier = 0, trace_tiles = 0, trace_kloop = 0, trace_epi = 0;
+  uint64_t trace_wait = 0, trace_barrier = 0, trace_ktiles = 0, trace_tile_wait = 0, trace_tile_barrier = 0, trace_tiles = 0, trace_kloop = 0, trace_epi = 0, trace_steps = 0, trace_last = 0, trace_mark = 0;
   const uint64_t trace_begin = __builtin_amdgcn_s_memtime();
 #endif
+  // Requests for a k-tile's operands.  A wave cannot issue anything else
+  // while a request waits to be accepted, and with all four waves asking at
+  // once each request takes about 80 cycles: cycle counters put the last k
+  // step, when it carried all sixteen requests of a wave, at 1250 cycles
+  // against 512 of matrix work.  With k-contiguous operands the requests are
+  // therefore spread over two k steps, one per two MFMAs: eight behind the
+  // barrier that released their stage and eight in the first k step of the
+  // next k-tile, which still leaves them two k steps to land.  (Spread over
+  // all four k steps, the late ones were waited for; the k-major variant keeps
+  // all sixteen in the last step: its fragment reads take twice the
+  // instructions and the explicit interleaving needed here ran out of registers.)
+  constexpr bool kSplitIssue = !kKMajor;
+  // request idx (0 .. 15) of a k-tile: operand A for even idx, B for odd, wave-level load idx / 2
+  auto issue_one = [&](int idx, const uint8_t* a_src, const uint8_t* b_src, int stage) {
+    const int q = idx >> 1;
+    if (idx & 1)
+      dma_load_16(fill_row0 * b_row_bytes + fill_chunk * 16, b_src + static_cast<uint64_t>(kRowsPerLoadStep * q) * b_row_bytes,
+                  stage + Cfg::kOperandBytes + fill_lds + q * 4096);
+    else
+      dma_load_16(fill_row0 * a_row_bytes + fill_chunk * 16, a_src + static_cast<uint64_t>(kRowsPerLoadStep * q) * a_row_bytes,
+                  stage + fill_lds + q * 4096);
+  };
   auto k_tile = [&](int64_t kt, int64_t ktiles, auto more_tag) {
     constexpr bool more = decltype(more_tag)::value;
     const int stage_off = static_cast<int>(kt & 1) * Cfg::kStageBytes;
     const int next_off = stage_off ^ Cfg::kStageBytes;
 #pragma unroll
     for (int ks = 0; ks + 1 < KS; ++ks) {
+      if (kSplitIssue && ks == 0 && more && kt >= 1) {
+        // the second eight requests for k-tile kt + 1 (the first eight went out in the last k step of kt - 1)
+        const uint8_t* a_cur = k_tile_ptr(Ab, a_row_bytes, kt + 1);
+        const uint8_t* b_cur = k_tile_ptr(Bb, b_row_bytes, kt + 1);
+#pragma unroll
+        for (int g = 0; g < TM * TN; ++g) {
+          mfma(0, g / TN, g % TN);
+          if (g < TM) read_a(1, stage_off, 1, g);
+          else if (g < TM + TN) read_b(1, stage_off, 1, g - TM);
+          if (g % 2 == 0) issue_one(8 + g / 2, a_cur, b_cur, next_off);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        continue;
+      }
       read_frags((ks + 1) & 1, stage_off, ks + 1);
 #pragma unroll
       for (int g = 0; g < TM * TN; ++g) mfma(ks & 1, g / TN, g % TN);
@@ -584,6 +632,7 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
     }
 #ifdef FSH_TRACE
     const uint64_t tr0 = __builtin_amdgcn_s_memtime();
+    trace_steps += tr0 - trace_mark;
 #endif
     if (more) {  // this wave's part of the next tile has landed
       wait_for_dma_loads();
@@ -608,14 +657,26 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
         if (g < TM) read_a(0, next_off, 0, g);
         else if (g < TM + TN) read_b(0, next_off, 0, g - TM);
       }
-      if (more2 && g % 2 == 0) issue_tile_load(a_next, b_next, a_row_bytes, b_row_bytes, stage_off, g / 2, g / 2 + 1);
+      if (more2 && g % 2 == 0) {
+        if (kSplitIssue) issue_one(g / 2, a_next, b_next, stage_off);
+        else issue_tile_load(a_next, b_next, a_row_bytes, b_row_bytes, stage_off, g / 2, g / 2 + 1);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
+#ifdef FSH_TRACE
+    trace_mark = __builtin_amdgcn_s_memtime();
+    trace_last += trace_mark - tr2;
+#endif
   };
 
   while (true) {
     const GemmParams& p = launch.problem[which];
     const int64_t ktiles = p.K / Cfg::BK;
+    {
+      int lane_again = lane;
+      asm volatile("" : "+v"(lane_again));
+      derive_lane_values(lane_again);
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -637,6 +698,7 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
     trace_tile_barrier += __builtin_amdgcn_s_memtime() - ts1;
     trace_tiles += 1;
     const uint64_t tk0 = __builtin_amdgcn_s_memtime();
+    trace_mark = tk0;
 #endif
     read_frags(0, 0, 0);
     if (ktiles > 1)
@@ -692,6 +754,8 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
       p.trace[blockIdx.x * 16 + 10] = trace_tiles;
       p.trace[blockIdx.x * 16 + 11] = trace_kloop;
       p.trace[blockIdx.x * 16 + 7] = trace_epi;
+      p.trace[blockIdx.x * 16 + 5] = trace_steps;
+      p.trace[blockIdx.x * 16 + 6] = trace_last;
     }
 #endif
     if (!have_next) break;
