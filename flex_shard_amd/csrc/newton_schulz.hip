@@ -583,14 +583,11 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   // while a request waits to be accepted, and with all four waves asking at
   // once each request takes about 80 cycles: cycle counters put the last k
   // step, when it carried all sixteen requests of a wave, at 1250 cycles
-  // against 512 of matrix work.  With k-contiguous operands the requests are
-  // therefore spread over two k steps, one per two MFMAs: eight behind the
-  // barrier that released their stage and eight in the first k step of the
-  // next k-tile, which still leaves them two k steps to land.  (Spread over
-  // all four k steps, the late ones were waited for; the k-major variant keeps
-  // all sixteen in the last step: its fragment reads take twice the
-  // instructions and the explicit interleaving needed here ran out of registers.)
-  constexpr bool kSplitIssue = !kKMajor;
+  // against 512 of matrix work.  The requests are therefore spread over two k
+  // steps, one per two MFMAs: eight behind the barrier that released their
+  // stage and eight in the first k step of the next k-tile, which still
+  // leaves them two k steps to land.  (Spread over all four k steps, the late
+  // ones were waited for.)
   // request idx (0 .. 15) of a k-tile: operand A for even idx, B for odd, wave-level load idx / 2
   auto issue_one = [&](int idx, const uint8_t* a_src, const uint8_t* b_src, int stage) {
     const int q = idx >> 1;
@@ -607,7 +604,7 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
     const int next_off = stage_off ^ Cfg::kStageBytes;
 #pragma unroll
     for (int ks = 0; ks + 1 < KS; ++ks) {
-      if (kSplitIssue && ks == 0 && more && kt >= 1) {
+      if (ks == 0 && more && kt >= 1) {
         // the second eight requests for k-tile kt + 1 (the first eight went out in the last k step of kt - 1)
         const uint8_t* a_cur = k_tile_ptr(Ab, a_row_bytes, kt + 1);
         const uint8_t* b_cur = k_tile_ptr(Bb, b_row_bytes, kt + 1);
@@ -657,10 +654,7 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
         if (g < TM) read_a(0, next_off, 0, g);
         else if (g < TM + TN) read_b(0, next_off, 0, g - TM);
       }
-      if (more2 && g % 2 == 0) {
-        if (kSplitIssue) issue_one(g / 2, a_next, b_next, stage_off);
-        else issue_tile_load(a_next, b_next, a_row_bytes, b_row_bytes, stage_off, g / 2, g / 2 + 1);
-      }
+      if (more2 && g % 2 == 0) issue_one(g / 2, a_next, b_next, stage_off);
       __builtin_amdgcn_sched_barrier(0);
     }
 #ifdef FSH_TRACE
