@@ -160,25 +160,18 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         descriptors: dict
 
     @dataclass(frozen=True)
-    class _LocalPackedSourceState:
-        storage: Any
-        version: int
-        storage_offset: int
-        shape: torch.Size
-        stride: tuple[int, ...]
-        dtype: torch.dtype
-        is_conj: bool
-        is_neg: bool
-
-    @dataclass(frozen=True)
-    class _LocalPackedInfoState:
-        info: Any
-        unsharded_dtype: torch.dtype
-
-    @dataclass(frozen=True)
     class _LocalPackedCacheEntry:
-        info_states: tuple
-        source_states: tuple
+        """A forward pack a backward re-gather may take once.  ``signature``
+        names the sources (address, dtype, shape, strides, negative bit) and
+        the quantization dtypes, ``versions`` their version counters at pack
+        time; ``sources`` keeps the shards' storage alive, so that an equal
+        address still means the same memory, and ``infos`` pins the ParamInfo
+        objects by identity."""
+
+        signature: tuple
+        versions: tuple
+        sources: tuple
+        infos: tuple
         metadata: quant_plan.QuantBucketMetadata
         packed: torch.Tensor
 
@@ -426,40 +419,19 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
 
     # ------------------------------------------------ local quantize + pack
     @staticmethod
-    def _local_packed_source_state(tensor: torch.Tensor) -> "_LocalPackedSourceState":
-        # Holding the storage keeps its address from being reused by another
-        # tensor, which would otherwise look like an unchanged source.
-        return BlockwiseQuantBucketedBlockShard._LocalPackedSourceState(
-            storage=tensor.untyped_storage(),
-            version=tensor._version,
-            storage_offset=tensor.storage_offset(),
-            shape=tensor.shape,
-            stride=tensor.stride(),
-            dtype=tensor.dtype,
-            is_conj=tensor.is_conj(),
-            is_neg=tensor.is_neg(),
-        )
-
-    @staticmethod
-    def _local_packed_source_matches(tensor: torch.Tensor, state: "_LocalPackedSourceState") -> bool:
+    def _pack_signature(
+        tensors: list[torch.Tensor], infos: list["ParamInfo"], rank: int, metadata: quant_plan.QuantBucketMetadata
+    ) -> tuple:
+        """What a cached launch table and a cached payload depend on besides
+        the shards' contents: which memory the shards are (address, dtype,
+        shape, strides, negative bit; bf16 and fp32 shards have no conjugate
+        bit) and the dtype each is quantized in."""
         return (
-            tensor._version == state.version
-            and tensor.untyped_storage() is state.storage
-            and tensor.storage_offset() == state.storage_offset
-            and tensor.shape == state.shape
-            and tensor.stride() == state.stride
-            and tensor.dtype == state.dtype
-            and tensor.is_conj() == state.is_conj
-            and tensor.is_neg() == state.is_neg
+            id(metadata),
+            rank,
+            tuple((t.data_ptr(), t.dtype, t.shape, t.stride(), t.is_neg()) for t in tensors),
+            tuple(info.unsharded_dtype for info in infos),
         )
-
-    @staticmethod
-    def _local_packed_info_state(info: "ParamInfo") -> "_LocalPackedInfoState":
-        return BlockwiseQuantBucketedBlockShard._LocalPackedInfoState(info=info, unsharded_dtype=info.unsharded_dtype)
-
-    @staticmethod
-    def _local_packed_info_matches(info: "ParamInfo", state: "_LocalPackedInfoState") -> bool:
-        return info is state.info and info.unsharded_dtype == state.unsharded_dtype
 
     @staticmethod
     def _local_packed_cache_context(tensors: list[torch.Tensor]) -> tuple[torch.device, Any]:
@@ -472,9 +444,12 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         infos: list["ParamInfo"],
         rank: int,
         metadata: quant_plan.QuantBucketMetadata,
+        signature: tuple | None = None,
     ) -> torch.Tensor:
         """Quantize this rank's dense shards and pack them, in one launch, into
-        a fresh payload ``[data | pad | scales | pad]`` of the common row size."""
+        a fresh payload ``[data | pad | scales | pad]`` of the common row size.
+        ``signature``: ``_pack_signature`` of the arguments when the caller has
+        it already."""
         if len(tensors) != len(infos):
             raise ValueError(
                 f"Quantized copy-in requires one tensor per ParamInfo, got {len(tensors)} tensors and {len(infos)} infos."
@@ -483,12 +458,8 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         # Steady state: the same shards (sharded parameter storage is
         # persistent) in the same layout.  The validated launch tables are
         # reused, so a pack is one allocation and one C call.
-        signature = (
-            id(metadata),
-            rank,
-            tuple((t.data_ptr(), t.dtype, t.shape, t.stride()) for t in tensors),
-            tuple(info.unsharded_dtype for info in infos),
-        )
+        if signature is None:
+            signature = self._pack_signature(tensors, infos, rank, metadata)
         cached = self._pack_launches.get(signature)
         if cached is not None and cached[0] is metadata:
             payload = torch.empty(metadata.packed_send_nbytes_per_rank, dtype=torch.uint8, device=cached[2])
@@ -573,28 +544,29 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         device, stream = self._local_packed_cache_context(tensors)
         prefix = (rank, id(metadata))
         key = (*prefix, device, stream)
+        signature = self._pack_signature(tensors, infos, rank, metadata)
+        versions = tuple(t._version for t in tensors)
         if not _is_backward_graph_task():
-            packed = self._pack_local_quantized_chunks(tensors, infos, rank, metadata)
-            for stale in [k for k in self._local_packed_cache if k[:2] == prefix]:
-                del self._local_packed_cache[stale]
+            packed = self._pack_local_quantized_chunks(tensors, infos, rank, metadata, signature)
+            if len(self._local_packed_cache) > 1 or (self._local_packed_cache and key not in self._local_packed_cache):
+                for stale in [k for k in self._local_packed_cache if k[:2] == prefix]:
+                    del self._local_packed_cache[stale]
             self._local_packed_cache[key] = self._LocalPackedCacheEntry(
-                info_states=tuple(self._local_packed_info_state(i) for i in infos),
-                source_states=tuple(self._local_packed_source_state(t) for t in tensors),
-                metadata=metadata,
-                packed=packed,
+                signature=signature, versions=versions, sources=tuple(tensors), infos=tuple(infos),
+                metadata=metadata, packed=packed,
             )
             return packed, metadata
         entry = self._local_packed_cache.pop(key, None)
         if (
             entry is not None
             and entry.metadata is metadata
-            and len(entry.info_states) == len(infos)
-            and len(entry.source_states) == len(tensors)
-            and all(self._local_packed_info_matches(i, s) for i, s in zip(infos, entry.info_states, strict=True))
-            and all(self._local_packed_source_matches(t, s) for t, s in zip(tensors, entry.source_states, strict=True))
+            and entry.signature == signature
+            and entry.versions == versions
+            and len(entry.infos) == len(infos)
+            and all(a is b for a, b in zip(infos, entry.infos))
         ):
             return entry.packed, metadata
-        return self._pack_local_quantized_chunks(tensors, infos, rank, metadata), metadata
+        return self._pack_local_quantized_chunks(tensors, infos, rank, metadata, signature), metadata
 
     # -------------------------------------------------------- unshard lifecycle
     def prepare_unshard_bucket(

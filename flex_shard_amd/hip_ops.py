@@ -127,13 +127,16 @@ class QuantPackPlan:
                 slot.src_kind = spec.src_kind
             self._tables.append((table, len(group)))
 
-    def launch(self, payload: torch.Tensor) -> None:
+    def launch(self, payload: torch.Tensor, stream: torch.cuda.Stream | None = None) -> None:
+        """Queue the launch on ``stream`` (default: the current stream of the
+        plan's device); the caller orders the payload's allocation and the
+        shards against that stream."""
         if payload.device != self._device or payload.dtype != torch.uint8 or payload.ndim != 1:
             raise ValueError("payload must be a 1-D uint8 tensor on the plan's device")
         if not payload.is_contiguous() or payload.numel() != self._payload_nbytes:
             raise ValueError(f"payload must be contiguous with {self._payload_nbytes} bytes")
         fn = _native.lib().fsh_quantize_pack
-        stream = stream_ptr(self._device)
+        stream = stream_ptr(self._device) if stream is None else stream.cuda_stream
         ptr, nbytes = payload.data_ptr(), self._payload_nbytes
         for index, (table, count) in enumerate(self._tables):
             zr = self._zero_ranges if index == 0 else ((0, 0), (0, 0))

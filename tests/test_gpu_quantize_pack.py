@@ -238,6 +238,20 @@ def test_payload_cache_forward_backward(device):
     assert restored.buffers[0] is cached.buffers[0]
     assert again.buffers[0] is not cached.buffers[0]  # the entry is consumed once
     assert torch.equal(again.buffers[0], cached.buffers[0])
+    # a source written in place after the forward pack (version counter moved) is packed again
+    forward = pl.prepare_unshard_bucket([param.detach()], [info], mesh, None)
+    with torch.no_grad():
+        param.mul_(-2.0)
+    with patch.object(mod, "_is_backward_graph_task", return_value=True):
+        repacked = pl.prepare_unshard_bucket([param.detach()], [info], mesh, None)
+    assert repacked.buffers[0] is not forward.buffers[0]
+    assert not torch.equal(repacked.buffers[0], forward.buffers[0])
+    # ... and so is a shard of the same shape at another address
+    forward = pl.prepare_unshard_bucket([param.detach()], [info], mesh, None)
+    moved = param.detach().clone()
+    with patch.object(mod, "_is_backward_graph_task", return_value=True):
+        elsewhere = pl.prepare_unshard_bucket([moved], [info], mesh, None)
+    assert elsewhere.buffers[0] is not forward.buffers[0] and torch.equal(elsewhere.buffers[0], forward.buffers[0])
 
 
 def test_argument_errors(device):
