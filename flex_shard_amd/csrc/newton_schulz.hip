@@ -544,6 +544,12 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   auto mfma = [&](int set, int i, int j) {
     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[set][j], af[set][i], acc[i][j], 0, 0, 0);
   };
+  // The first k step of a tile starts its accumulators from a zero operand
+  // instead of from 256 cleared registers.
+  auto mfma_from_zero = [&](int set, int i, int j) {
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[set][j], af[set][i], zero, 0, 0, 0);
+  };
 
   // Current tile: plain scalars, reassigned per tile.
   int which = 0, tm = 0, tn = 0;
@@ -598,13 +604,14 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
       dma_load_16(fill_row0 * a_row_bytes + fill_chunk * 16, a_src + static_cast<uint64_t>(kRowsPerLoadStep * q) * a_row_bytes,
                   stage + fill_lds + q * 4096);
   };
-  auto k_tile = [&](int64_t kt, int64_t ktiles, auto more_tag) {
+  auto k_tile = [&](int64_t kt, int64_t ktiles, auto more_tag, auto first_tag) {
     constexpr bool more = decltype(more_tag)::value;
+    constexpr bool first = decltype(first_tag)::value;  // k-tile 0 of an output tile
     const int stage_off = static_cast<int>(kt & 1) * Cfg::kStageBytes;
     const int next_off = stage_off ^ Cfg::kStageBytes;
 #pragma unroll
     for (int ks = 0; ks + 1 < KS; ++ks) {
-      if (ks == 0 && more && kt >= 1) {
+      if (ks == 0 && more && !first) {
         // the second eight requests for k-tile kt + 1 (the first eight went out in the last k step of kt - 1)
         const uint8_t* a_cur = k_tile_ptr(Ab, a_row_bytes, kt + 1);
         const uint8_t* b_cur = k_tile_ptr(Bb, b_row_bytes, kt + 1);
@@ -620,7 +627,10 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
       }
       read_frags((ks + 1) & 1, stage_off, ks + 1);
 #pragma unroll
-      for (int g = 0; g < TM * TN; ++g) mfma(ks & 1, g / TN, g % TN);
+      for (int g = 0; g < TM * TN; ++g) {
+        if (first && ks == 0) mfma_from_zero(0, g / TN, g % TN);
+        else mfma(ks & 1, g / TN, g % TN);
+      }
 #pragma unroll
       for (int g = 0; g < TM + TN; ++g) {
         __builtin_amdgcn_sched_group_barrier(kSchedDsRead, kKMajor ? 2 : 1, 0);
@@ -671,12 +681,6 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
       asm volatile("" : "+v"(lane_again));
       derive_lane_values(lane_again);
     }
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
     FSH_STAMP(6);
 #ifdef FSH_TRACE
     const uint64_t ts0 = __builtin_amdgcn_s_memtime();
@@ -700,8 +704,13 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
                       Cfg::kStageBytes, 0, Cfg::kLoadsPerOperand);
     FSH_STAMP(2);
 
-    for (int64_t kt = 0; kt + 1 < ktiles; ++kt) k_tile(kt, ktiles, std::true_type{});
-    k_tile(ktiles - 1, ktiles, std::false_type{});
+    if (ktiles > 1) {
+      k_tile(0, ktiles, std::true_type{}, std::true_type{});
+      for (int64_t kt = 1; kt + 1 < ktiles; ++kt) k_tile(kt, ktiles, std::true_type{}, std::false_type{});
+      k_tile(ktiles - 1, ktiles, std::false_type{}, std::false_type{});
+    } else {
+      k_tile(0, ktiles, std::false_type{}, std::true_type{});
+    }
     FSH_STAMP(3);
 #ifdef FSH_TRACE
     trace_kloop += __builtin_amdgcn_s_memtime() - tk0;
