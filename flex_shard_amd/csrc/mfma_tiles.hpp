@@ -30,6 +30,14 @@ struct GemmParams {
   int32_t tiles_per_matrix;
   int64_t work_items;     // tiles_per_matrix * batch
   int64_t items_per_xcd;  // ceil(work_items / 8); the grid has 8 * items_per_xcd workgroups
+  // Muon update fused into the epilogue (large-tile kernel only).  When
+  // update_ptrs is not null, C and D are ignored: matrix b of the batch is the
+  // separately allocated parameter at update_ptrs[b] (row stride ldc), and the
+  // epilogue stores  p = bf16(bf16(p * decay) + neg_lr * d),  d = bf16(acc)
+  // (d scaled by dir_scale and rounded first when that is not 1): the
+  // product itself is never written.
+  const int64_t* update_ptrs;
+  float update_decay, update_neg_lr, update_dir_scale;
 #ifdef FSH_TRACE
   uint64_t* trace;
 #endif
@@ -176,17 +184,24 @@ struct DRows {
   u32x4 t[kPasses];
 };
 
+// `d` is matrix `batch` of D (row stride ldd elements).
+template <typename Cfg>
+__device__ __forceinline__ void load_d_rows_from(const uint16_t* d, int64_t ldd, int64_t m0, int64_t n0, int wm, int wn,
+                                                 int lane, int half, DRows<Cfg>& rows) {
+  using R = DRows<Cfg>;
+  const int r0 = lane / R::kLanesPerRow, chunk = lane % R::kLanesPerRow;
+  const uint32_t lane_off = static_cast<uint32_t>(r0) * static_cast<uint32_t>(ldd * 2) + chunk * 16;
+  const uint8_t* base = uniform_ptr(reinterpret_cast<const uint8_t*>(
+      d + (m0 + wm * Cfg::kWaveM + half * (Cfg::kWaveM / 2)) * ldd + n0 + wn * Cfg::kWaveN));
+  const int64_t pass_bytes = uniform_i64(static_cast<int64_t>(R::kRowsPerPass) * ldd * 2);
+#pragma unroll
+  for (int q = 0; q < R::kPasses; ++q) rows.t[q] = *reinterpret_cast<const u32x4*>(base + q * pass_bytes + lane_off);
+}
+
 template <typename Cfg>
 __device__ __forceinline__ void load_d_rows(const GemmParams& p, int64_t batch, int64_t m0, int64_t n0, int wm, int wn,
                                             int lane, int half, DRows<Cfg>& rows) {
-  using R = DRows<Cfg>;
-  const int r0 = lane / R::kLanesPerRow, chunk = lane % R::kLanesPerRow;
-  const uint32_t lane_off = static_cast<uint32_t>(r0) * static_cast<uint32_t>(p.ldd * 2) + chunk * 16;
-  const uint8_t* base = uniform_ptr(reinterpret_cast<const uint8_t*>(
-      p.D + batch * p.sD + (m0 + wm * Cfg::kWaveM + half * (Cfg::kWaveM / 2)) * p.ldd + n0 + wn * Cfg::kWaveN));
-  const int64_t pass_bytes = uniform_i64(static_cast<int64_t>(R::kRowsPerPass) * p.ldd * 2);
-#pragma unroll
-  for (int q = 0; q < R::kPasses; ++q) rows.t[q] = *reinterpret_cast<const u32x4*>(base + q * pass_bytes + lane_off);
+  load_d_rows_from<Cfg>(p.D + batch * p.sD, p.ldd, m0, n0, wm, wn, lane, half, rows);
 }
 
 template <typename Cfg, int kPitch>
@@ -339,33 +354,39 @@ struct HalfTileEpilogue {
 //   kEpiGeneric  any combination, flags read at run time
 //   kEpiPlain    C = bf16(acc): no D, no diagonal term, alpha == 1
 //   kEpiPoly     C = bf16(fma(beta, D, alpha * acc) + diag): D, alpha and the diagonal term
-constexpr int kEpiGeneric = 0, kEpiPlain = 1, kEpiPoly = 2;
+//   kEpiUpdate   Muon update of separately allocated parameters (see GemmParams::update_ptrs)
+constexpr int kEpiGeneric = 0, kEpiPlain = 1, kEpiPoly = 2, kEpiUpdate = 3;
 
+// (Always inlined: as a real call the accumulators and the launch's problem
+// table would have to live in scratch memory.)
 template <typename Cfg, int kMode>
-__device__ inline void store_tile_in_halves_as(const GemmParams& p, int64_t batch, int64_t m0, int64_t n0, int wm,
+__device__ __forceinline__ void store_tile_in_halves_as(const GemmParams& p, int64_t batch, int64_t m0, int64_t n0, int wm,
                                                int wn, int lane, bool mirror, const f32x16 (&acc)[Cfg::TM][Cfg::TN],
                                                uint8_t* staging) {
   using Epi = HalfTileEpilogue<Cfg>;
   using R = DRows<Cfg>;
   constexpr int TM = Cfg::TM, TN = Cfg::TN, HM = TM / 2;
   static_assert(TM % 2 == 0 && Epi::kRows == HM * 32, "two halves of whole 32-row blocks");
-  const bool has_d = kMode == kEpiPlain ? false : kMode == kEpiPoly ? true : p.D != nullptr;
-  uint16_t* C = p.C + batch * p.sC;
+  const bool has_d = kMode == kEpiPlain ? false : (kMode == kEpiPoly || kMode == kEpiUpdate) ? true : p.D != nullptr;
+  // (a pointer loaded from a table is a per-lane value to the compiler: said to be uniform here)
+  uint16_t* C = kMode == kEpiUpdate ? reinterpret_cast<uint16_t*>(uniform_i64(p.update_ptrs[batch])) : p.C + batch * p.sC;
+  const uint16_t* D = kMode == kEpiUpdate ? C : p.D + batch * p.sD;
+  const int64_t ldd = kMode == kEpiUpdate ? p.ldc : p.ldd;
   // A symmetric product mirrors its off-diagonal tiles into the lower triangle.
   uint16_t* Ct = mirror ? C : (p.Ct ? p.Ct + batch * p.sCt : nullptr);
   const int64_t ldct = mirror ? p.ldc : p.ldct;
   const int64_t wave_row = m0 + wm * Cfg::kWaveM, wave_col = n0 + wn * Cfg::kWaveN;
   uint8_t* region = staging + (wm * Cfg::WN + wn) * Epi::kRegion;
   const int r_lane = lane & 31, h = lane >> 5;
-  const bool unit_alpha = kMode == kEpiPlain ? true : kMode == kEpiPoly ? false : p.alpha == 1.0f;
+  const bool unit_alpha = (kMode == kEpiPlain || kMode == kEpiUpdate) ? true : kMode == kEpiPoly ? false : p.alpha == 1.0f;
   // Block tiles and wave sub-tiles are square, so C's diagonal runs through
   // the (i, i) blocks of the diagonal sub-tiles of the diagonal tiles.
-  const bool on_diagonal = kMode != kEpiPlain && p.diag_add != 0.0f && m0 == n0 && wm == wn;
+  const bool on_diagonal = kMode != kEpiPlain && kMode != kEpiUpdate && p.diag_add != 0.0f && m0 == n0 && wm == wn;
 
   // The lower half of D is requested once the upper half has left its
   // registers for LDS, and lands while the upper half is worked on.
   DRows<Cfg> drows[2];
-  if (has_d) load_d_rows<Cfg>(p, batch, m0, n0, wm, wn, lane, 0, drows[0]);
+  if (has_d) load_d_rows_from<Cfg>(D, ldd, m0, n0, wm, wn, lane, 0, drows[0]);
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {
     if (has_d) {
@@ -377,7 +398,7 @@ __device__ inline void store_tile_in_halves_as(const GemmParams& p, int64_t batc
         *reinterpret_cast<u32x2*>(d) = u32x2{drows[hf].t[q].x, drows[hf].t[q].y};
         *reinterpret_cast<u32x2*>(d + 8) = u32x2{drows[hf].t[q].z, drows[hf].t[q].w};
       }
-      if (hf == 0) load_d_rows<Cfg>(p, batch, m0, n0, wm, wn, lane, 1, drows[1]);
+      if (hf == 0) load_d_rows_from<Cfg>(D, ldd, m0, n0, wm, wn, lane, 1, drows[1]);
       wave_lds_sync();
     }
 #pragma unroll
@@ -400,13 +421,34 @@ __device__ inline void store_tile_in_halves_as(const GemmParams& p, int64_t batc
           float v[4];
 #pragma unroll
           for (int t = 0; t < 4; ++t) v[t] = unit_alpha ? acc[i][j][4 * b + t] : p.alpha * acc[i][j][4 * b + t];
-          if (has_d) {
+          if (kMode == kEpiUpdate) {
+            // The rounding sequence of the separate update kernel: direction
+            // to bf16 (scaled and rounded again when the scale is not 1),
+            // decayed parameter to bf16, then one multiply and one add.
+            const uint32_t d01 = pack_bf16x2(v[0], v[1]), d23 = pack_bf16x2(v[2], v[3]);
+            float d[4] = {u32_as_f32(d01 << 16), u32_as_f32(d01 & 0xFFFF0000u), u32_as_f32(d23 << 16),
+                          u32_as_f32(d23 & 0xFFFF0000u)};
+            if (p.update_dir_scale != 1.0f) {
+              const uint32_t s01 = pack_bf16x2(d[0] * p.update_dir_scale, d[1] * p.update_dir_scale);
+              const uint32_t s23 = pack_bf16x2(d[2] * p.update_dir_scale, d[3] * p.update_dir_scale);
+              d[0] = u32_as_f32(s01 << 16); d[1] = u32_as_f32(s01 & 0xFFFF0000u);
+              d[2] = u32_as_f32(s23 << 16); d[3] = u32_as_f32(s23 & 0xFFFF0000u);
+            }
+            const uint32_t p01 = pack_bf16x2(u32_as_f32(dv[j][b].x << 16) * p.update_decay,
+                                             u32_as_f32(dv[j][b].x & 0xFFFF0000u) * p.update_decay);
+            const uint32_t p23 = pack_bf16x2(u32_as_f32(dv[j][b].y << 16) * p.update_decay,
+                                             u32_as_f32(dv[j][b].y & 0xFFFF0000u) * p.update_decay);
+            v[0] = u32_as_f32(p01 << 16) + p.update_neg_lr * d[0];
+            v[1] = u32_as_f32(p01 & 0xFFFF0000u) + p.update_neg_lr * d[1];
+            v[2] = u32_as_f32(p23 << 16) + p.update_neg_lr * d[2];
+            v[3] = u32_as_f32(p23 & 0xFFFF0000u) + p.update_neg_lr * d[3];
+          } else if (has_d) {
             v[0] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].x << 16), v[0]);
             v[1] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].x & 0xFFFF0000u), v[1]);
             v[2] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].y << 16), v[2]);
             v[3] = __builtin_fmaf(p.beta, u32_as_f32(dv[j][b].y & 0xFFFF0000u), v[3]);
           }
-          if (kMode != kEpiPlain && i == j) {
+          if (kMode != kEpiPlain && kMode != kEpiUpdate && i == j) {
             // a select per final rather than a branch per block (adding zero
             // elsewhere would turn a -0 into +0)
 #pragma unroll
@@ -464,12 +506,14 @@ __device__ inline void store_tile_in_halves_as(const GemmParams& p, int64_t batc
 }
 
 template <typename Cfg>
-__device__ inline void store_tile_in_halves(const GemmParams& p, int64_t batch, int64_t m0, int64_t n0, int wm, int wn,
+__device__ __forceinline__ void store_tile_in_halves(const GemmParams& p, int64_t batch, int64_t m0, int64_t n0, int wm, int wn,
                                             int lane, bool mirror, const f32x16 (&acc)[Cfg::TM][Cfg::TN],
                                             uint8_t* staging) {
   // uniform over the launch's problem, so one branch per tile
   const bool has_d = p.D != nullptr, diag = p.diag_add != 0.0f, unit_alpha = p.alpha == 1.0f;
-  if (!has_d && !diag && unit_alpha)
+  if (p.update_ptrs != nullptr)
+    store_tile_in_halves_as<Cfg, kEpiUpdate>(p, batch, m0, n0, wm, wn, lane, mirror, acc, staging);
+  else if (!has_d && !diag && unit_alpha)
     store_tile_in_halves_as<Cfg, kEpiPlain>(p, batch, m0, n0, wm, wn, lane, mirror, acc, staging);
   else if (has_d && !unit_alpha)
     store_tile_in_halves_as<Cfg, kEpiPoly>(p, batch, m0, n0, wm, wn, lane, mirror, acc, staging);

@@ -594,6 +594,7 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
   // stage and eight in the first k step of the next k-tile, which still
   // leaves them two k steps to land.  (Spread over all four k steps, the late
   // ones were waited for.)
+  constexpr int kFirstRequests = 8, kSecondRequests = 16 - kFirstRequests;  // 6 / 10, 10 / 6 and 12 / 4 measured the same or slower
   // request idx (0 .. 15) of a k-tile: operand A for even idx, B for odd, wave-level load idx / 2
   auto issue_one = [&](int idx, const uint8_t* a_src, const uint8_t* b_src, int stage) {
     const int q = idx >> 1;
@@ -620,7 +621,8 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
           mfma(0, g / TN, g % TN);
           if (g < TM) read_a(1, stage_off, 1, g);
           else if (g < TM + TN) read_b(1, stage_off, 1, g - TM);
-          if (g % 2 == 0) issue_one(8 + g / 2, a_cur, b_cur, next_off);
+          if ((g + 1) * kSecondRequests / 16 != g * kSecondRequests / 16)
+            issue_one(kFirstRequests + g * kSecondRequests / 16, a_cur, b_cur, next_off);
           __builtin_amdgcn_sched_barrier(0);
         }
         continue;
@@ -664,7 +666,8 @@ __global__ __launch_bounds__(DmaGemm::kThreads) void gemm_nt_dma_kernel(const Ge
         if (g < TM) read_a(0, next_off, 0, g);
         else if (g < TM + TN) read_b(0, next_off, 0, g - TM);
       }
-      if (more2 && g % 2 == 0) issue_one(g / 2, a_next, b_next, stage_off);
+      if (more2 && (g + 1) * kFirstRequests / 16 != g * kFirstRequests / 16)
+        issue_one(g * kFirstRequests / 16, a_next, b_next, stage_off);
       __builtin_amdgcn_sched_barrier(0);
     }
 #ifdef FSH_TRACE
@@ -809,7 +812,14 @@ int plan_gemm_cfg(PlannedGemm* plan, int64_t batch) {
   return FSH_OK;
 }
 
-int plan_gemm(const fsh_gemm_desc& d, PlannedGemm* plan) {
+// The Muon update an epilogue applies instead of storing its product (see
+// GemmParams::update_ptrs); ptrs == nullptr: an ordinary product.
+struct GemmUpdate {
+  const int64_t* ptrs;
+  float decay, neg_lr, dir_scale;
+};
+
+int plan_gemm(const fsh_gemm_desc& d, PlannedGemm* plan, const GemmUpdate* update = nullptr) {
   if (d.m <= 0 || d.n <= 0 || d.k <= 0 || d.batch <= 0)
     return fail(FSH_EINVAL, "gemm: non-positive size (m %lld, n %lld, k %lld, batch %lld)", (long long)d.m,
                 (long long)d.n, (long long)d.k, (long long)d.batch);
@@ -837,14 +847,30 @@ int plan_gemm(const fsh_gemm_desc& d, PlannedGemm* plan) {
   p.sA = d.stride_a; p.sB = d.stride_b; p.sD = d.stride_d; p.sC = d.stride_c; p.sCt = d.stride_ct;
   p.alpha = d.alpha; p.beta = d.beta;
   p.diag_add = d.diag_add;
+  if (update != nullptr && update->ptrs != nullptr) {
+    if (d.d_dev != nullptr || d.ct_dev != nullptr || d.symmetric || d.alpha != 1.0f || d.diag_add != 0.0f)
+      return fail(FSH_EINVAL, "gemm: a fused update takes a plain product");
+    p.update_ptrs = update->ptrs;
+    p.update_decay = update->decay;
+    p.update_neg_lr = update->neg_lr;
+    p.update_dir_scale = update->dir_scale;
+  }
 #ifdef FSH_TRACE
   if (const char* e = getenv("FSH_GEMM_TRACE")) p.trace = reinterpret_cast<uint64_t*>(strtoull(e, nullptr, 0));
 #endif
   // The big tile pays off once it fills the chip at least once.
   const int64_t big_n = ceil_div(d.n, BigCfg::BN);
   const int64_t big_tiles = (d.symmetric ? big_n * (big_n + 1) / 2 : ceil_div(d.m, BigCfg::BM) * big_n) * d.batch;
-  if (big_tiles >= 192) return plan_gemm_cfg<BigCfg>(plan, d.batch);
-  return plan_gemm_cfg<SmallCfg>(plan, d.batch);
+  const int rc = big_tiles >= 192 ? plan_gemm_cfg<BigCfg>(plan, d.batch) : plan_gemm_cfg<SmallCfg>(plan, d.batch);
+  if (rc == FSH_OK && p.update_ptrs != nullptr && plan->kind != kKernelDma)
+    return fail(FSH_ENOTSUP, "gemm: only the large-tile kernel applies a fused update");
+  return rc;
+}
+
+// Whether `d` would run on the large-tile kernel (whose epilogue can apply a fused update).
+bool takes_large_tile_kernel(const fsh_gemm_desc& d) {
+  PlannedGemm plan;
+  return plan_gemm(d, &plan) == FSH_OK && plan.kind == kKernelDma;
 }
 
 // Compute units of the current device (0 when the query fails).
@@ -946,13 +972,13 @@ int launch_planned(PlannedGemm* plans, int count, hipStream_t stream) {
   return FSH_OK;
 }
 
-int launch_gemms(const fsh_gemm_desc* descs, int count, hipStream_t stream) {
+int launch_gemms(const fsh_gemm_desc* descs, int count, hipStream_t stream, const GemmUpdate* updates = nullptr) {
   constexpr int kChunk = 16;
   PlannedGemm plans[kChunk];
   for (int begin = 0; begin < count; begin += kChunk) {
     const int n = count - begin < kChunk ? count - begin : kChunk;
     for (int i = 0; i < n; ++i)
-      if (int rc = plan_gemm(descs[begin + i], &plans[i])) return rc;
+      if (int rc = plan_gemm(descs[begin + i], &plans[i], updates ? &updates[begin + i] : nullptr)) return rc;
     if (int rc = launch_planned(plans, n, stream)) return rc;
   }
   return FSH_OK;
@@ -1353,14 +1379,19 @@ fsh_gemm_desc ns_product(const NsState& st, int which, float a, float b, float c
 }
 
 // The iteration proper for `count` normalized problems.
-int ns_iterate(NsState* st, int count, float a, float b, float c, int32_t steps, hipStream_t stream) {
+// `last_updates` (one per problem, or null): the last product of a problem
+// whose entry has ptrs set applies that update to the parameters instead of
+// writing the orthogonalized matrix to the caller's buffer.
+int ns_iterate(NsState* st, int count, float a, float b, float c, int32_t steps, hipStream_t stream,
+               const GemmUpdate* last_updates = nullptr) {
   fsh_gemm_desc descs[FSH_MAX_NS_PROBLEMS];
   for (int step = 0; step < steps; ++step) {
     // The same product of every problem goes out together: problems are
     // independent of each other, the three products of one are not.
     for (int which = 0; which < 3; ++which) {
-      for (int i = 0; i < count; ++i) descs[i] = ns_product(st[i], which, a, b, c, step + 1 == steps);
-      if (int rc = launch_gemms(descs, count, stream)) return rc;
+      const bool last = step + 1 == steps;
+      for (int i = 0; i < count; ++i) descs[i] = ns_product(st[i], which, a, b, c, last);
+      if (int rc = launch_gemms(descs, count, stream, last && which == 2 ? last_updates : nullptr)) return rc;
     }
     for (int i = 0; i < count; ++i) st[i].cur ^= 1;
   }
@@ -1448,8 +1479,21 @@ FSH_API int fsh_muon_step(const fsh_muon_group* groups, int32_t count, float ler
   NsState st[FSH_MAX_NS_PROBLEMS];
   for (int i = 0; i < count; ++i)
     if (int rc = ns_begin(problems[i], steps, eps, stream, &st[i], /*partials_ready=*/true)) return rc;
-  if (int rc = ns_iterate(st, count, a, b, c, steps, stream)) return rc;
+  // A group whose last product runs on the large-tile kernel gets its update
+  // from that product's epilogue: the direction is never written and read
+  // back.  The other groups' directions land in their batch buffers and a
+  // separate launch applies them.
+  GemmUpdate updates[FSH_MAX_NS_PROBLEMS];
   for (int i = 0; i < count; ++i) {
+    const bool fused = steps > 0 && takes_large_tile_kernel(ns_product(st[i], 2, a, b, c, true));
+    updates[i].ptrs = fused ? groups[i].param_ptrs_dev : nullptr;
+    updates[i].decay = decay_factor;
+    updates[i].neg_lr = groups[i].neg_adjusted_lr;
+    updates[i].dir_scale = groups[i].direction_scale;
+  }
+  if (int rc = ns_iterate(st, count, a, b, c, steps, stream, updates)) return rc;
+  for (int i = 0; i < count; ++i) {
+    if (updates[i].ptrs != nullptr) continue;
     const fsh_muon_group& g = groups[i];
     MuonApplyBatch q;
     q.param_ptrs = g.param_ptrs_dev;

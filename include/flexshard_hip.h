@@ -352,12 +352,16 @@ int fsh_fp8_gemm_1x128_128x1(const void* aq_dev, const float* as_dev, const void
  * fsh_newton_schulz_multi and fsh_muon_apply in sequence, with the same
  * results bit for bit.  Per group there is one momentum launch for all its
  * matrices (it also leaves the sums of squares the normalization needs, so
- * the Newton-Schulz input is read once less) and one update launch.
+ * the Newton-Schulz input is read once less).  The update of a group whose
+ * matrices fill the large-tile GEMM kernel is applied by the epilogue of its
+ * last Newton-Schulz product (the orthogonalized matrix is then never
+ * written); other groups get one update launch.
  * The parameters, gradients and momentum buffers of a group are separate
  * allocations, named by device tables of their addresses; each must be a
  * contiguous bf16 [rows, cols] matrix at a 16-byte aligned address.
  * batch_dev is scratch of batch*rows*cols bf16: it holds the momentum
- * output, then the orthogonalized direction.
+ * output and, for groups updated by a separate launch, the orthogonalized
+ * direction afterwards (its contents after the call are otherwise unspecified).
  * ---------------------------------------------------------------------- */
 typedef struct fsh_muon_group {
   const int64_t* param_ptrs_dev;    /* [batch] addresses of the parameters, updated in place   */
