@@ -107,24 +107,32 @@ __global__ __launch_bounds__(kActThreads) void act_quant_1x128_kernel(const ActQ
 // 16-byte chunk c of row r in slot c ^ ((r >> 1) & 7), into one of two 64 KB
 // stages.  A lane feeds the matrix core bytes [32 h, 32 h + 32) of each half
 // of its row (h = lane / 32), i.e. chunks 2h and 2h+1 of a 64-byte half.
-struct Fp8Gemm {
-  static constexpr int BM = 256, BN = 256, BK = 128, WM = 4, WN = 2, TM = 2, TN = 4;
+//
+// TM_ = 1 is the half tile (128 x 256, waves of 32 x 128) that the tiles of a
+// last, at most half-full round are cut into; it keeps the LDS layout of the
+// whole tile and fills the first half of the A area.
+template <int TM_>
+struct Fp8GemmCfg {
+  static constexpr int BM = 128 * TM_, BN = 256, BK = 128, WM = 4, WN = 2, TM = TM_, TN = 4;
   static constexpr int kWaves = WM * WN, kThreads = 64 * kWaves, kWaveM = BM / WM, kWaveN = BN / WN;
   static constexpr int kRowBytes = 128;
-  static constexpr int kABytes = BM * kRowBytes;               // 32 KB
-  static constexpr int kStageBytes = (BM + BN) * kRowBytes;    // 64 KB
+  static constexpr int kABytes = 256 * kRowBytes;              // 32 KB (half of it used by the half tile)
+  static constexpr int kStageBytes = (256 + BN) * kRowBytes;   // 64 KB
   static constexpr int kFillRows = 8 * kWaves;                 // tile rows per wave-level load of all waves
-  static constexpr int kLoadsA = BM / kFillRows, kLoadsB = BN / kFillRows;  // per wave: 4 and 4
+  static constexpr int kLoadsA = BM / kFillRows, kLoadsB = BN / kFillRows;  // per wave: 4 (2) and 4
   static constexpr int kPitch = kWaveN * 2 + 8;                // epilogue staging, bytes
   static constexpr int kRegion = kWaveM * kPitch;              // per wave
   static constexpr int kStages = 2;
-  static constexpr int kScaleStageBytes = kWaves * kWaveM * 4;  // per stage: [wave][64] row scales
+  static constexpr int kScaleSlots = 64;                        // row scales per wave and stage (one 4-byte request per lane)
+  static constexpr int kScaleStageBytes = kWaves * kScaleSlots * 4;
   static constexpr int kScaleOffset = kStages * kStageBytes;
   static constexpr int kWeightScaleOffset = kScaleOffset + kStages * kScaleStageBytes;  // [wave][256] block scales
   static constexpr int kMaxKTilesInLds = 256;
   static constexpr int kLdsBytes = max_int(kWeightScaleOffset + kWaves * kMaxKTilesInLds * 4, kWaves * kRegion);
-  static_assert(kWaveM == 64, "one 4-byte scale request per wave covers its rows");
+  static_assert(kWaveM <= kScaleSlots, "one 4-byte scale request per lane covers the wave's rows");
 };
+using Fp8Gemm = Fp8GemmCfg<2>;
+static_assert(Fp8GemmCfg<1>::kLdsBytes <= Fp8Gemm::kLdsBytes, "the half tile lives in the whole tile's LDS");
 
 struct Fp8GemmParams {
   const uint8_t* xq;
@@ -135,30 +143,45 @@ struct Fp8GemmParams {
   uint16_t* out;
   int64_t m, n, k;
   int64_t ldxq, ldwq, ldo, ws_cb, ws_kb;
-  GemmParams schedule;  // tile order only
+  GemmParams schedule;  // tile order; its work items are the tiles computed whole
+  // Workgroups [whole_grid, ...) take the remaining tiles (in the same order)
+  // as two half tiles each, half_items in all.
+  int64_t whole_grid, half_items, half_items_per_xcd;
 };
 
 typedef int v8i32 __attribute__((ext_vector_type(8)));
 
-// kColumnScales = false: the second operand carries one scale per 128 x 128
-// tile (a prequantized weight, either orientation).  true: one scale per
-// output column and k-block (an operand quantized in 128 x 1 runs).
-template <bool kColumnScales>
-__global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(const Fp8GemmParams p) {
-  using Cfg = Fp8Gemm;
+// acc[n] += (product[n] * row_scale) * (column_scales of lane n of this lane's row of 16).
+// The broadcast is the multiply-add's own operand modifier (the compiler keeps
+// a separate move per element when given the builtin).  column_scales comes
+// from LDS, not from the vector ALU, so the modifier's read needs no wait states.
+template <int N = 0>
+__device__ __forceinline__ void fold_with_row_broadcast(f32x16& acc, const f32x16& product, float row_scale,
+                                                        float column_scales) {
+  if constexpr (N < 16) {
+    const float scaled = product[N] * row_scale;
+    float sum = acc[N];
+    asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
+        : "+v"(sum)
+        : "v"(column_scales), "v"(scaled), "n"(N));
+    acc[N] = sum;
+    fold_with_row_broadcast<N + 1>(acc, product, row_scale, column_scales);
+  }
+}
+
+// One output tile (TM_ = 2) or half tile (TM_ = 1, rows [128 half, +128) of the tile).
+template <bool kColumnScales, int TM_>
+__device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams& p, uint8_t* lds_bytes, int tm, int tn, int half) {
+  using Cfg = Fp8GemmCfg<TM_>;
   static_assert(Cfg::kStages == 2, "the loop below alternates between two stages");
-  extern __shared__ __attribute__((aligned(1024))) uint8_t lds_bytes[];
   constexpr int TM = Cfg::TM, TN = Cfg::TN;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
-  int64_t unused_batch;
-  int tm, tn;
-  if (!tile_of_workgroup(p.schedule, blockIdx.x, &unused_batch, &tm, &tn)) return;  // whole workgroup
-  tm = uniform_i32(tm);
-  tn = uniform_i32(tn);
-  const int64_t m0 = static_cast<int64_t>(tm) * Cfg::BM, n0 = static_cast<int64_t>(tn) * Cfg::BN;
+  const int64_t m0 = static_cast<int64_t>(tm) * Fp8Gemm::BM + static_cast<int64_t>(half) * Cfg::BM;
+  const int64_t n0 = static_cast<int64_t>(tn) * Cfg::BN;
+  if (m0 >= p.m) return;  // the second half of a tile that ends in its first (whole workgroup)
   const int64_t ktiles = p.k / Cfg::BK;
 
   // Load side: wave-level load q of a wave fills tile rows [64 q + 8 wave, +8);
@@ -231,8 +254,8 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
   // per-lane requests per wave and k-tile for the wave's 128 rows): a
   // compiler-visible load here would make the compiler wait for everything in
   // flight, the prefetched tile included.
-  const uint32_t scale_lds0 = lds_base + static_cast<uint32_t>(Cfg::kScaleOffset + wave * Cfg::kWaveM * 4);
-  const int64_t scale_row = m0 + wm * Cfg::kWaveM + lane;
+  const uint32_t scale_lds0 = lds_base + static_cast<uint32_t>(Cfg::kScaleOffset + wave * Cfg::kScaleSlots * 4);
+  const int64_t scale_row = m0 + wm * Cfg::kWaveM + (lane & (Cfg::kWaveM - 1));  // lanes past the wave's rows repeat them
   const uint32_t scale_voff = static_cast<uint32_t>((scale_row < p.m ? scale_row : p.m - 1) * 4);
   // Per-column scales of the workgroup's 256 columns take the same road, 64
   // columns per wave (the first four waves), into [stage][256] floats of the
@@ -250,20 +273,21 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
     issue_tile_load(kt, stage * Cfg::kStageBytes);
     issue_scale_loads(kt, stage);
   };
-  // One eighth of the wave's requests for the next k-tile; issued behind each
-  // block's MFMAs rather than all at once, which would hold up the wave's
-  // instruction issue while the matrix core runs dry.
+  // One of the wave's requests for the next k-tile; they are issued a few at
+  // a time behind the MFMAs of the first blocks rather than all at once, which
+  // would hold up the wave's instruction issue while the matrix core runs dry.
   auto issue_k_tile_part = [&](int64_t kt, int stage, int part) {
     const int stage_off = stage * Cfg::kStageBytes;
-    const int q = part >> 1;
-    if (part & 1)
+    if (part >= Cfg::kLoadsA + Cfg::kLoadsB) return;
+    if (part >= Cfg::kLoadsA) {
+      const int q = part - Cfg::kLoadsA;
       dma_load_16(b_voff[q], Bb + kt * Cfg::kRowBytes,
                   stage_off + Cfg::kABytes + fill_lds + q * Cfg::kFillRows * Cfg::kRowBytes);
-    else
-      dma_load_16(a_voff[q], Ab + kt * Cfg::kRowBytes, stage_off + fill_lds + q * Cfg::kFillRows * Cfg::kRowBytes);
+    } else {
+      dma_load_16(a_voff[part], Ab + kt * Cfg::kRowBytes, stage_off + fill_lds + part * Cfg::kFillRows * Cfg::kRowBytes);
+    }
     if (part == 0) issue_scale_loads(kt, stage);
   };
-  static_assert(Cfg::kLoadsA + Cfg::kLoadsB == Cfg::TM * Cfg::TN, "one request per block");
   // The block scales of the wave's 128 columns, one per k-tile, are copied
   // to LDS once (a load from global memory inside the loop would again wait
   // for the prefetched tile).
@@ -294,7 +318,7 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
 #pragma unroll
     for (int i = 0; i < TM; ++i)
       s[i] = *reinterpret_cast<const float*>(lds_bytes + Cfg::kScaleOffset + stage * Cfg::kScaleStageBytes +
-                                             (wave * Cfg::kWaveM + i * 32 + frag_row) * 4);
+                                             (wave * Cfg::kScaleSlots + i * 32 + frag_row) * 4);
     if (!kColumnScales) {
       const float ws_now = ws_lds[kt];
 #pragma unroll
@@ -319,7 +343,19 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
     // block's MFMAs: a fold that reads the product of the MFMA issued just
     // before it waits for the matrix core to drain (measured: 122 against 100
     // time units per block for the arrangement used here).
-    const uint8_t* cscale_lds = lds_bytes + Cfg::kWeightScaleOffset + stage * 1024 + (wn * Cfg::kWaveN + 4 * h) * 4;
+    // Per-column scales: register j holds, in every row of 16 lanes, the 16
+    // scales of column block j that the lanes of that row fold with (lane n of
+    // the row the scale of accumulator element n), so a fold takes element n's
+    // scale from lane n of its own row through the data-parallel-primitive
+    // broadcast of the multiply-add itself: no scale is read from LDS between a
+    // product and its fold.
+    float cs_rows[TN];
+    if (kColumnScales) {
+      const uint8_t* cscale_lds = lds_bytes + Cfg::kWeightScaleOffset + stage * 1024 +
+                                  (wn * Cfg::kWaveN + 8 * ((lane & 15) >> 2) + 4 * h + (lane & 3)) * 4;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) cs_rows[j] = *reinterpret_cast<const float*>(cscale_lds + j * 32 * 4);
+    }
     constexpr int kBlocks = TM * TN;
     // Blocks between a product and its fold.  One: the other wave of the SIMD
     // keeps the matrix core busy while this one waits for its own product,
@@ -329,13 +365,7 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
     auto fold = [&](int blk, const f32x16& product) {
       const int pi = blk % TM, pj = blk / TM;
       if (kColumnScales) {
-#pragma unroll
-        for (int b = 0; b < 4; ++b) {  // four column scales at a time: 16 would not fit next to the accumulators
-          const f32x4 cs = *reinterpret_cast<const f32x4*>(cscale_lds + (pj * 32 + 8 * b) * 4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            acc[pi][pj][4 * b + e] = __builtin_fmaf(product[4 * b + e] * s[pi], cs[e], acc[pi][pj][4 * b + e]);
-        }
+        fold_with_row_broadcast(acc[pi][pj], product, s[pi], cs_rows[pj]);
       } else {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[pi][pj][r] = __builtin_fmaf(product[r], s[pi], acc[pi][pj][r]);
@@ -357,6 +387,15 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
         for (int kh = 0; kh < 2; ++kh)
           bfrag[(j + 1) % kBSets][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32) + j + 1, kh);
       }
+      // Wave priority falls as the k-tile proceeds: of the two waves of a SIMD
+      // the one that is behind wins the issue slot, so both reach the barrier
+      // together (with equal priorities the older wave runs ahead and then
+      // idles at the barrier while the other finishes alone, without a
+      // partner to overlap its folds with).
+      if (blk * 4 == 0 * kBlocks) __builtin_amdgcn_s_setprio(3);
+      if (blk * 4 == 1 * kBlocks) __builtin_amdgcn_s_setprio(2);
+      if (blk * 4 == 2 * kBlocks) __builtin_amdgcn_s_setprio(1);
+      if (blk * 4 == 3 * kBlocks) __builtin_amdgcn_s_setprio(0);
       f32x16 product =
           __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag[j % kBSets][0], afrag[i][0], zero, 0, 0, 0, 0, 0, 0);
       product =
@@ -368,7 +407,16 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
         for (int kh = 0; kh < 2; ++kh)
           bfrag[0][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32) + j + 1, kh);
       }
-      if (more) issue_k_tile_part(kt + 1, stage ^ 1, blk);
+      // The next k-tile's requests leave during the first half of this one, so
+      // the data has the second half to arrive (spread over all blocks, the last
+      // requests were still in flight at the end: 0.15-0.35 us of every 2 us
+      // k-tile went to waiting for them).
+      constexpr int kIssueBlocks = kBlocks / 2;
+      constexpr int kPartsPerBlock = (Cfg::kLoadsA + Cfg::kLoadsB + kIssueBlocks - 1) / kIssueBlocks;
+      if (more && blk < kIssueBlocks) {
+#pragma unroll
+        for (int part = 0; part < kPartsPerBlock; ++part) issue_k_tile_part(kt + 1, stage ^ 1, blk * kPartsPerBlock + part);
+      }
       if (blk >= kLag) fold(blk - kLag, part[(blk - kLag) % (kLag + 1)]);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -431,6 +479,28 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
           if (col + e < p.n) dst[e] = static_cast<uint16_t>(w[e >> 1] >> (16 * (e & 1)));
       }
     }
+  }
+}
+
+// kColumnScales = false: the second operand carries one scale per 128 x 128
+// tile (a prequantized weight, either orientation).  true: one scale per
+// output column and k-block (an operand quantized in 128 x 1 runs).
+template <bool kColumnScales>
+__global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(const Fp8GemmParams p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds_bytes[];
+  int64_t unused_batch;
+  int tm, tn;
+  if (static_cast<int64_t>(blockIdx.x) < p.whole_grid) {
+    if (!tile_of_workgroup(p.schedule, blockIdx.x, &unused_batch, &tm, &tn)) return;  // whole workgroup
+    fp8_gemm_tile<kColumnScales, 2>(p, lds_bytes, uniform_i32(tm), uniform_i32(tn), 0);
+  } else {
+    // Same split over the XCDs as the whole tiles: the two halves of a tile are
+    // neighbours in an XCD's run and share the tile's second operand in its L2.
+    const int64_t id = static_cast<int64_t>(blockIdx.x) - p.whole_grid;
+    const int64_t item = (id % kXcds) * p.half_items_per_xcd + id / kXcds;
+    if (item >= p.half_items) return;
+    tile_in_order(p.schedule, static_cast<int>(p.schedule.work_items + item / 2), &tm, &tn);
+    fp8_gemm_tile<kColumnScales, 1>(p, lds_bytes, uniform_i32(tm), uniform_i32(tn), uniform_i32(static_cast<int>(item & 1)));
   }
 }
 
@@ -508,14 +578,24 @@ int launch_fp8_gemm(Fp8GemmParams& p, bool column_scales, const char* who, void*
   const int64_t tiles = static_cast<int64_t>(s.tiles_m) * s.tiles_n;
   if (tiles > 0x3FFFFFFFLL) return fail(FSH_ENOTSUP, "%s: too many tiles", who);
   s.tiles_per_matrix = static_cast<int32_t>(tiles);
-  s.work_items = tiles;
-  s.items_per_xcd = ceil_div(tiles, static_cast<int64_t>(kXcds));
+  // A workgroup holds a CU for a tile, so the tiles go through the chip in
+  // rounds of one per CU.  A last round that is at most half full is cut into
+  // half tiles, twice as many workgroups of half the length: e.g. the 896
+  // tiles of a [14336, 4096] result take 3.5 rounds instead of 4.
+  const int64_t units = compute_units();
+  const int64_t tail = units > 0 ? tiles % units : 0;
+  const int64_t cut = (tail > 0 && 2 * tail <= units) ? tail : 0;
+  s.work_items = tiles - cut;
+  s.items_per_xcd = ceil_div(s.work_items, static_cast<int64_t>(kXcds));
+  p.whole_grid = s.items_per_xcd * kXcds;
+  p.half_items = 2 * cut;
+  p.half_items_per_xcd = ceil_div(p.half_items, static_cast<int64_t>(kXcds));
   static LdsReservation reserved_block_scales, reserved_column_scales;
   if (int rc = column_scales
                    ? reserve_lds_once(reserved_column_scales, &fp8_gemm_blockwise_kernel<true>, Fp8Gemm::kLdsBytes)
                    : reserve_lds_once(reserved_block_scales, &fp8_gemm_blockwise_kernel<false>, Fp8Gemm::kLdsBytes))
     return rc;
-  const dim3 grid(static_cast<uint32_t>(s.items_per_xcd * kXcds)), block(Fp8Gemm::kThreads);
+  const dim3 grid(static_cast<uint32_t>(p.whole_grid + p.half_items_per_xcd * kXcds)), block(Fp8Gemm::kThreads);
   if (column_scales)
     hipLaunchKernelGGL(fp8_gemm_blockwise_kernel<true>, grid, block, Fp8Gemm::kLdsBytes, static_cast<hipStream_t>(stream), p);
   else

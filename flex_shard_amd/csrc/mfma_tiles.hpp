@@ -63,6 +63,16 @@ struct GemmLaunch {
 constexpr int kXcds = 8;         // accelerator dies, each with its own L2
 constexpr int kGroupTilesM = 4;  // tile rows walked together
 
+// Tile t of a (non-symmetric) matrix in the patch order described below.
+__device__ inline void tile_in_order(const GemmParams& p, int t, int* tm, int* tn) {
+  const int group_span = kGroupTilesM * p.tiles_n;
+  const int first_m = (t / group_span) * kGroupTilesM;
+  const int rows = min(p.tiles_m - first_m, kGroupTilesM);
+  const int within = t % group_span;
+  *tm = first_m + within % rows;
+  *tn = within / rows;
+}
+
 // Workgroup id -> (batch, tile row, tile column).  Workgroups are handed to
 // the 8 XCDs round-robin by id, and an XCD holds 32 of the large-tile
 // workgroups at a time (one per CU), so XCD x is given the contiguous run
@@ -90,12 +100,7 @@ __device__ inline bool tile_of_workgroup(const GemmParams& p, int64_t id, int64_
     *tn = r + t;
     return true;
   }
-  const int group_span = kGroupTilesM * p.tiles_n;
-  const int first_m = (t / group_span) * kGroupTilesM;
-  const int rows = min(p.tiles_m - first_m, kGroupTilesM);
-  const int within = t % group_span;
-  *tm = first_m + within % rows;
-  *tn = within / rows;
+  tile_in_order(p, t, tm, tn);
   return true;
 }
 
@@ -548,6 +553,19 @@ int reserve_lds(Kernel kernel, int bytes) {
   return FSH_OK;
 }
 
+
+// Compute units of the current device (0 when the query fails).
+inline int64_t compute_units() {
+  static int cached[64] = {0};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 0;
+  if (cached[device] == 0) {
+    int count = 0;
+    if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return 0;
+    cached[device] = count;
+  }
+  return cached[device];
+}
 
 // The attribute is per device and function, and sticky: it is set once per
 // device and kernel, whichever host thread gets there first (setting it

@@ -873,19 +873,6 @@ bool takes_large_tile_kernel(const fsh_gemm_desc& d) {
   return plan_gemm(d, &plan) == FSH_OK && plan.kind == kKernelDma;
 }
 
-// Compute units of the current device (0 when the query fails).
-int64_t compute_units() {
-  static int cached[64] = {0};
-  int device = 0;
-  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 0;
-  if (cached[device] == 0) {
-    int count = 0;
-    if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return 0;
-    cached[device] = count;
-  }
-  return cached[device];
-}
-
 template <typename Kernel>
 int launch_single(Kernel kernel, LdsReservation* reserved, int lds_bytes, int threads, const PlannedGemm& plan,
                   hipStream_t stream, const char* name) {

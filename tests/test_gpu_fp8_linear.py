@@ -54,7 +54,15 @@ def _small_int_fp8(shape, gen, high=4):
     return torch.randint(-high, high + 1, shape, generator=gen).to(torch.float32).to(E4M3)
 
 
-@pytest.mark.parametrize("m,n,k", [(128, 256, 128), (70, 200, 384), (300, 520, 256), (1, 8, 128), (129, 257, 1024)])
+@pytest.mark.parametrize(
+    "m,n,k",
+    [
+        (128, 256, 128), (70, 200, 384), (300, 520, 256), (1, 8, 128), (129, 257, 1024),
+        (3072, 3000, 256),  # 144 tiles on 256 CUs: more than half a round, every tile computed whole
+        (4352, 4096, 128),  # 272 tiles: one round of whole tiles, the 16 left over as 32 half tiles
+        (2200, 4096, 128),  # 144 tiles whose last tile row ends in its first half
+    ],
+)
 def test_gemm_integer_products_are_exact(device, m, n, k):
     """Small integers and power-of-two scales: every product, scaled partial
     sum and running sum is exact in fp32 whatever the order, so the output is

@@ -100,7 +100,15 @@ def test_column_scaled_gemm_integer_products_are_exact(device, m, n, k):
     assert torch.equal(got.cpu(), want.bfloat16())
 
 
-@pytest.mark.parametrize("m,n,k", [(256, 512, 512), (200, 384, 256), (1024, 1032, 2048), (77, 130, 128)])
+@pytest.mark.parametrize(
+    "m,n,k",
+    [
+        (256, 512, 512), (200, 384, 256), (1024, 1032, 2048), (77, 130, 128),
+        (3072, 3000, 256),  # 144 tiles on 256 CUs: more than half a round, every tile computed whole
+        (4352, 4096, 128),  # 272 tiles: one round of whole tiles, the 16 left over as 32 half tiles
+        (2200, 4096, 128),  # 144 tiles whose last tile row ends in its first half
+    ],
+)
 def test_column_scaled_gemm_matches_the_oracle(device, m, n, k):
     gen = torch.Generator().manual_seed(m * 3 + n + k + 1)
     a = torch.randn(k, m, generator=gen).bfloat16()
