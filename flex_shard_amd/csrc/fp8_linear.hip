@@ -182,6 +182,9 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams& p, uint8_t* l
   const int64_t m0 = static_cast<int64_t>(tm) * Fp8Gemm::BM + static_cast<int64_t>(half) * Cfg::BM;
   const int64_t n0 = static_cast<int64_t>(tn) * Cfg::BN;
   if (m0 >= p.m) return;  // the second half of a tile that ends in its first (whole workgroup)
+#ifdef FSH_TRACE
+  const uint64_t t_entry = __builtin_amdgcn_s_memrealtime();
+#endif
   const int64_t ktiles = p.k / Cfg::BK;
 
   // Load side: wave-level load q of a wave fills tile rows [64 q + 8 wave, +8);
@@ -439,7 +442,7 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams& p, uint8_t* l
 #ifdef FSH_TRACE
   if (p.schedule.trace && lane == 0) {
     uint64_t* out = p.schedule.trace + (static_cast<int64_t>(blockIdx.x) * Cfg::kWaves + wave) * 8;
-    out[0] = t_begin; out[1] = t_compute; out[2] = t_wait; out[3] = t_barrier; out[4] = t_mark;
+    out[0] = t_begin; out[1] = t_compute; out[2] = t_wait; out[3] = t_barrier; out[4] = t_mark; out[5] = t_entry;
   }
 #endif
 
@@ -480,6 +483,17 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams& p, uint8_t* l
       }
     }
   }
+#ifdef FSH_TRACE
+  if (p.schedule.trace && lane == 0) {
+    __builtin_amdgcn_s_waitcnt(0);
+    p.schedule.trace[(static_cast<int64_t>(blockIdx.x) * Cfg::kWaves + wave) * 8 + 6] = __builtin_amdgcn_s_memrealtime();
+    uint32_t hw_id;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw_id));
+    uint32_t xcc_id;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc_id));
+    p.schedule.trace[(static_cast<int64_t>(blockIdx.x) * Cfg::kWaves + wave) * 8 + 7] = (static_cast<uint64_t>(xcc_id) << 32) | hw_id;
+  }
+#endif
 }
 
 // kColumnScales = false: the second operand carries one scale per 128 x 128

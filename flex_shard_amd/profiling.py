@@ -10,9 +10,14 @@ import contextlib
 import torch
 
 
+_NO_RANGE = contextlib.nullcontext()
+
+
 def record_range(name: str, debug_fqn: str | None = None):
-    if torch.compiler.is_compiling():
-        return contextlib.nullcontext()
+    # A range costs several microseconds of host time per call even when
+    # nobody listens; torch keeps this flag current while a profiler runs.
+    if not torch.autograd.profiler._is_profiler_enabled or torch.compiler.is_compiling():
+        return _NO_RANGE
     label = name if debug_fqn is None else f"{name} ({debug_fqn})"
     return torch.profiler.record_function(label)
 
