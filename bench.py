@@ -85,6 +85,16 @@ def _event_ms(fn, steps: int, warmup: int) -> tuple[float, float]:
     return wall, start.elapsed_time(stop)
 
 
+def _steady_us(fn, reps: int, settle_ms: float = 5.0) -> float:
+    """us per call of fn(i) over `reps` calls, after untimed calls that last
+    about `settle_ms`: a compute-bound kernel runs its first milliseconds
+    after other work at a clock that is still settling."""
+    _, est_ms = _event_ms(fn, 3, 2)
+    settle = max(2, int(settle_ms / max(est_ms / 3, 1e-3)))
+    _, ms = _event_ms(fn, reps, settle)
+    return ms / reps * 1e3
+
+
 def build_quant_workload(device, layers: int, rank: int = 0, spec=None, std: float = 0.02):
     """Per layer: one rank's local shards as views of one flat bf16 storage (the
     sharded bucket storage layout), their ParamInfos, and a reusable payload."""
@@ -503,8 +513,8 @@ def bench_fp8_linear(device, tokens: int = 8192, reps: int = 10):
         _, q_ms = _event_ms(lambda i: hip_ops.act_quant_1x128(x), reps, 2)
         xq, xs = hip_ops.act_quant_1x128(x)
         y = torch.empty((tokens, n), dtype=torch.bfloat16, device=device)
-        _, g_ms = _event_ms(lambda i: hip_ops.fp8_gemm_1x128_128x128(xq, xs, wq, ws, out=y), 2 * reps, reps)
-        q_us, g_us = q_ms / reps * 1e3, g_ms / (2 * reps) * 1e3  # the GEMMs: 10 untimed + 20 timed launches (the clock settles over the first few ms)
+        g_us = _steady_us(lambda i: hip_ops.fp8_gemm_1x128_128x128(xq, xs, wq, ws, out=y), 2 * reps)
+        q_us = q_ms / reps * 1e3
         flop = 2 * tokens * n * k
         out[name] = {
             "act_quant_us": q_us,
@@ -542,13 +552,11 @@ def bench_fp8_linear_backward(device, tokens: int = 8192, reps: int = 10):
         us["quant_x_t"] = ms / reps * 1e3
         wt = hip_ops.fp8_transpose(wq)
         gq, gs = hip_ops.act_quant_1x128(g)
-        _, ms = _event_ms(lambda i: hip_ops.fp8_gemm_1x128_128x128_dgrad(gq, gs, wt, ws), 2 * reps, reps)
-        us["dgrad_gemm"] = ms / (2 * reps) * 1e3
+        us["dgrad_gemm"] = _steady_us(lambda i: hip_ops.fp8_gemm_1x128_128x128_dgrad(gq, gs, wt, ws), 2 * reps)
         del wt, gq, gs
         gtq, gts = hip_ops.act_quant_128x1_transposed(g)
         xtq, xts = hip_ops.act_quant_128x1_transposed(x)
-        _, ms = _event_ms(lambda i: hip_ops.fp8_gemm_1x128_128x1(gtq, gts, xtq, xts), 2 * reps, reps)
-        us["wgrad_gemm"] = ms / (2 * reps) * 1e3
+        us["wgrad_gemm"] = _steady_us(lambda i: hip_ops.fp8_gemm_1x128_128x1(gtq, gts, xtq, xts), 2 * reps)
         flop = 2 * tokens * n * k
         out[name] = {
             "transpose_us": us["transpose"],
