@@ -14,6 +14,10 @@ per second over the whole timed region, inputs resident in HBM.
 One JSON line is printed.  Besides the contract fields it carries
   roofline      the dominant kernel against the 8 TB/s HBM peak, timed with
                 events on the launch stream over the same timed region
+  contract_entry / two_buckets_in_flight
+                the same launches through `prepare_unshard_bucket` itself
+                (host time of the contract included) and alternating over two
+                streams (the per-launch ramp of one overlaps the other's tail)
   cpu_baseline  the oracle's eager-torch restatement of the reference path on
                 the host cores, on the same rank-0 share (the gradient path
                 and Newton-Schulz have their own CPU legs under `secondary`)
