@@ -131,3 +131,22 @@ def test_forward_of_the_prequantized_linear(device):
         gemms.forward(x.to(device)[:, :128].contiguous(), flat)
     with pytest.raises(ValueError, match="block_size"):
         Fp8BlockwiseGemms(block_size=64).backward(x.to(device), x.to(device), flat, True, True)
+
+
+def test_gemm_rejects_what_the_kernel_cannot_take(device):
+    """k that is not a multiple of 128, and a contraction longer than the
+    block-scale variant keeps weight scales for (32 768), fail with a message
+    instead of launching."""
+    xq = torch.zeros((8, 192), dtype=torch.uint8, device=device)
+    xs = torch.ones((1, 8), dtype=torch.float32, device=device)
+    wq = torch.zeros((8, 192), dtype=torch.uint8, device=device)
+    ws = torch.ones((1, 1), dtype=torch.float32, device=device)
+    with pytest.raises(RuntimeError, match="multiple of 128"):
+        hip_ops.fp8_gemm_1x128_128x128(xq, xs, wq, ws)
+    k = 32768 + 128
+    xq = torch.zeros((8, k), dtype=torch.uint8, device=device)
+    xs = torch.ones((k // 128, 8), dtype=torch.float32, device=device)
+    wq = torch.zeros((8, k), dtype=torch.uint8, device=device)
+    ws = torch.ones((1, k // 128), dtype=torch.float32, device=device)
+    with pytest.raises(RuntimeError, match="at most 32768"):
+        hip_ops.fp8_gemm_1x128_128x128(xq, xs, wq, ws)

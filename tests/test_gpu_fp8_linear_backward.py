@@ -89,7 +89,13 @@ def test_token_run_quantizer_strided_rows_and_eps_switch(device):
         hip_ops.act_quant_128x1_transposed(torch.zeros(128, 12, dtype=torch.bfloat16, device=device))
 
 
-@pytest.mark.parametrize("m,n,k", [(128, 256, 128), (70, 200, 384), (300, 520, 256), (1, 8, 128), (129, 257, 1024)])
+@pytest.mark.parametrize(
+    "m,n,k",
+    [
+        (128, 256, 128), (70, 200, 384), (300, 520, 256), (1, 8, 128), (129, 257, 1024),
+        (128, 256, 32768 + 128),  # more tokens than the block-scale variant's k limit: this variant takes any length
+    ],
+)
 def test_column_scaled_gemm_integer_products_are_exact(device, m, n, k):
     gen = torch.Generator().manual_seed(m + n + k + 1)
     aq, bq = _small_int_fp8((m, k), gen), _small_int_fp8((n, k), gen)
