@@ -462,7 +462,7 @@ def bench_gradients(device, reps=5):
     }
 
 
-def bench_muon(device, reps=3):
+def bench_muon(device, reps=4):
     """Config 5: 24 x [7168, 2048] + 24 x [2048, 2048] bf16 whole matrices, one
     Muon step (momentum, Nesterov, 5 Newton-Schulz steps, update)."""
     from flex_shard_amd.dist_muon import OwnedMuon
@@ -472,7 +472,7 @@ def bench_muon(device, reps=3):
     params = [seeded_normal(s, 0.02, 2000 + i, device) for i, s in enumerate(shapes)]
     grads = [seeded_normal(s, 1.0, 3000 + i, device) for i, s in enumerate(shapes)]
     opt = OwnedMuon(params)
-    _, ms = _event_ms(lambda i: opt.step(grads), reps, 1)
+    _, ms = _event_ms(lambda i: opt.step(grads), reps, 2)  # two untimed steps: the clock settles over the first
     per = ms / reps
     flops = opt.flops_per_step()
     # The orthogonalization alone (normalization + 5 iterations on all 48
