@@ -434,9 +434,11 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         )
 
     @staticmethod
-    def _local_packed_cache_context(tensors: list[torch.Tensor]) -> tuple[torch.device, Any]:
+    def _local_packed_cache_context(tensors: list[torch.Tensor]) -> tuple[torch.device, int]:
+        """Device and raw current stream: a cached payload is only valid for
+        consumers ordered after the stream it was packed on."""
         device = next((t.device for t in tensors if t.numel() > 0), tensors[0].device)
-        return device, torch.cuda.current_stream(device)
+        return device, hip_ops.stream_ptr(device)
 
     def _pack_local_quantized_chunks(
         self,
@@ -539,12 +541,13 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         metadata = self._quant_metadata_from_infos(infos)
         if torch.compiler.is_compiling():
             return self._pack_local_quantized_chunks(tensors, infos, rank, metadata), metadata
-        for tensor in tensors:
-            _require_gpu_rows(tensor, "Quantized copy-in")
+        signature = self._pack_signature(tensors, infos, rank, metadata)
+        if signature not in self._pack_launches:  # shards behind a cached launch table were checked when it was built
+            for tensor in tensors:
+                _require_gpu_rows(tensor, "Quantized copy-in")
         device, stream = self._local_packed_cache_context(tensors)
         prefix = (rank, id(metadata))
         key = (*prefix, device, stream)
-        signature = self._pack_signature(tensors, infos, rank, metadata)
         versions = tuple(t._version for t in tensors)
         if not _is_backward_graph_task():
             packed = self._pack_local_quantized_chunks(tensors, infos, rank, metadata, signature)

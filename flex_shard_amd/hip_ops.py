@@ -53,8 +53,10 @@ def _require_gpu(*tensors: torch.Tensor) -> torch.device:
 
 
 def stream_ptr(device: torch.device) -> int:
-    """The raw hipStream_t of torch's current stream on ``device``."""
-    return torch.cuda.current_stream(device).cuda_stream
+    """The raw hipStream_t of torch's current stream on ``device`` (torch's own
+    accessor for kernel launchers: no Stream object is built)."""
+    index = device.index
+    return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device() if index is None else index)
 
 
 def _dt(dtype: torch.dtype) -> int:
