@@ -313,53 +313,70 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams& p, uint8_t* l
     t_mark = now;
   };
 #endif
-  int stage = 0;
-  for (int64_t kt = 0; kt < ktiles; ++kt) {
-    const int stage_off = stage * Cfg::kStageBytes;
-    const bool more = kt + 1 < ktiles;  // the next k-tile's stage was released by the barrier that ended kt - 1
-    float s[TM];
+  // The k loop is rotated by one block: the barrier that hands over k-tile
+  // kt + 1 sits before the last 32x32 block of k-tile kt, and behind that
+  // block's MFMAs the wave already reads what the first block of kt + 1 needs
+  // (its first A and B fragments).  The first MFMAs after a
+  // barrier thus never wait for an LDS read, which every wave of the
+  // workgroup would otherwise do at the same moment.
+  //   carried into a k-tile: afrag[0], bfrag[0]
+  constexpr int kBSets = kColumnScales ? 1 : 2;  // the per-column variant has registers for one set of B fragments only
+  constexpr int kBlocks = TM * TN;
+  v8i32 afrag[TM][2], bfrag[kBSets][2];
+  float s[TM], cs_rows[TN];
+  // Row scales of the wave's rows for the k-tile in `stage`, times the weight
+  // block's scale in the block-scale variant.
+  auto read_row_scales = [&](float (&dst)[TM], int stage, int64_t kt) {
 #pragma unroll
     for (int i = 0; i < TM; ++i)
-      s[i] = *reinterpret_cast<const float*>(lds_bytes + Cfg::kScaleOffset + stage * Cfg::kScaleStageBytes +
-                                             (wave * Cfg::kScaleSlots + i * 32 + frag_row) * 4);
+      dst[i] = *reinterpret_cast<const float*>(lds_bytes + Cfg::kScaleOffset + stage * Cfg::kScaleStageBytes +
+                                               (wave * Cfg::kScaleSlots + i * 32 + frag_row) * 4);
     if (!kColumnScales) {
       const float ws_now = ws_lds[kt];
 #pragma unroll
-      for (int i = 0; i < TM; ++i) s[i] *= ws_now;
+      for (int i = 0; i < TM; ++i) dst[i] *= ws_now;
     }
-    // Fragments are read in the order the blocks need them: the first column
-    // block's B and the first row block's A before the first MFMA, the other
-    // A row blocks under the MFMAs of the first column block (they stay for
-    // the whole k-tile), each further B column block while the previous one is
-    // multiplied.
-    // The per-column variant has registers for one set of B fragments only.
-    constexpr int kBSets = kColumnScales ? 1 : 2;
-    v8i32 afrag[TM][2], bfrag[kBSets][2];
-#pragma unroll
-    for (int kh = 0; kh < 2; ++kh) bfrag[0][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32), kh);
-#pragma unroll
-    for (int kh = 0; kh < 2; ++kh) afrag[0][kh] = read_frag(stage_off, 0, wm * (Cfg::kWaveM / 32), kh);
-    // The wave's eight 32x32 blocks, column block by column block: two MFMAs, back
-    // to back, give a block's partial product for this scale block.  It is
-    // folded into the result (16 fused multiply-adds, or multiply + fused
-    // multiply-add with per-column scales) two blocks later, behind that
-    // block's MFMAs: a fold that reads the product of the MFMA issued just
-    // before it waits for the matrix core to drain (measured: 122 against 100
-    // time units per block for the arrangement used here).
-    // Per-column scales: register j holds, in every row of 16 lanes, the 16
-    // scales of column block j that the lanes of that row fold with (lane n of
-    // the row the scale of accumulator element n), so a fold takes element n's
-    // scale from lane n of its own row through the data-parallel-primitive
-    // broadcast of the multiply-add itself: no scale is read from LDS between a
-    // product and its fold.
-    float cs_rows[TN];
+  };
+  // Per-column scales: register j holds, in every row of 16 lanes, the 16
+  // scales of column block j that the lanes of that row fold with (lane n of
+  // the row the scale of accumulator element n), so a fold takes element n's
+  // scale from lane n of its own row through the data-parallel-primitive
+  // broadcast of the multiply-add itself: no scale is read from LDS between a
+  // product and its fold.
+  auto read_column_scales = [&](float (&dst)[TN], int stage) {
     if (kColumnScales) {
       const uint8_t* cscale_lds = lds_bytes + Cfg::kWeightScaleOffset + stage * 1024 +
                                   (wn * Cfg::kWaveN + 8 * ((lane & 15) >> 2) + 4 * h + (lane & 3)) * 4;
 #pragma unroll
-      for (int j = 0; j < TN; ++j) cs_rows[j] = *reinterpret_cast<const float*>(cscale_lds + j * 32 * 4);
+      for (int j = 0; j < TN; ++j) dst[j] = *reinterpret_cast<const float*>(cscale_lds + j * 32 * 4);
     }
-    constexpr int kBlocks = TM * TN;
+  };
+  auto read_first_frags = [&](int stage_off) {
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh) bfrag[0][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32), kh);
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh) afrag[0][kh] = read_frag(stage_off, 0, wm * (Cfg::kWaveM / 32), kh);
+  };
+  read_first_frags(0);
+
+  int stage = 0;
+  for (int64_t kt = 0; kt < ktiles; ++kt) {
+    const int stage_off = stage * Cfg::kStageBytes;
+    const bool more = kt + 1 < ktiles;  // the next k-tile's stage was released by the barrier inside kt - 1
+    // The scales are first needed by the fold behind the second block's MFMAs.
+    read_row_scales(s, stage, kt);
+    read_column_scales(cs_rows, stage);
+    // Fragments are read in the order the blocks need them: the other A row
+    // blocks under the MFMAs of the first column block (they stay for the
+    // whole k-tile), each further B column block while the previous one is
+    // multiplied.
+    // The wave's eight 32x32 blocks, column block by column block: two MFMAs, back
+    // to back, give a block's partial product for this scale block.  It is
+    // folded into the result (16 fused multiply-adds, or multiply + fused
+    // multiply-add with per-column scales) one block later, behind that
+    // block's MFMAs: a fold that reads the product of the MFMA issued just
+    // before it waits for the matrix core to drain (measured: 122 against 100
+    // time units per block for the arrangement used here).
     // Blocks between a product and its fold.  One: the other wave of the SIMD
     // keeps the matrix core busy while this one waits for its own product,
     // and the registers of a third product are needed elsewhere.
@@ -381,6 +398,20 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams& p, uint8_t* l
     for (int blk = 0; blk < kBlocks; ++blk) {
       const int i = blk % TM, j = blk / TM;
       const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (blk == kBlocks - 1) {
+        // Every fragment of this k-tile is in registers: hand the stage over.
+#ifdef FSH_TRACE
+        lap(t_compute);
+#endif
+        if (more) wait_for_dma_loads();  // this wave's part of k-tile kt + 1 has landed
+#ifdef FSH_TRACE
+        lap(t_wait);
+#endif
+        __syncthreads();
+#ifdef FSH_TRACE
+        lap(t_barrier);
+#endif
+      }
       if (j == 0 && i + 1 < TM) {  // next row block's A fragments
 #pragma unroll
         for (int kh = 0; kh < 2; ++kh) afrag[i + 1][kh] = read_frag(stage_off, 0, wm * (Cfg::kWaveM / 32) + i + 1, kh);
@@ -410,10 +441,15 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams& p, uint8_t* l
         for (int kh = 0; kh < 2; ++kh)
           bfrag[0][kh] = read_frag(stage_off, Cfg::kABytes, wn * (Cfg::kWaveN / 32) + j + 1, kh);
       }
+      if (blk == kBlocks - 1 && more) {  // behind the last MFMAs of this k-tile: what the next one starts with
+        read_first_frags(stage_off ^ Cfg::kStageBytes);
+      }
       // The next k-tile's requests leave during the first half of this one, so
       // the data has the second half to arrive (spread over all blocks, the last
-      // requests were still in flight at the end: 0.15-0.35 us of every 2 us
-      // k-tile went to waiting for them).
+      // requests were still in flight at the hand-over: 0.15-0.35 us of every
+      // 2 us k-tile went to waiting for them; moved one block earlier still,
+      // behind the hand-over barrier of the previous k-tile, the per-column
+      // variant ran out of registers).
       constexpr int kIssueBlocks = kBlocks / 2;
       constexpr int kPartsPerBlock = (Cfg::kLoadsA + Cfg::kLoadsB + kIssueBlocks - 1) / kIssueBlocks;
       if (more && blk < kIssueBlocks) {
@@ -425,18 +461,6 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams& p, uint8_t* l
     }
 #pragma unroll
     for (int blk = kBlocks - kLag; blk < kBlocks; ++blk) fold(blk, part[blk % (kLag + 1)]);
-#ifdef FSH_TRACE
-    asm volatile("" : "+v"(acc[TM - 1][TN - 1]));
-    lap(t_compute);
-#endif
-    if (kt + 1 < ktiles) wait_for_dma_loads();  // k-tile kt + 1 has landed
-#ifdef FSH_TRACE
-    lap(t_wait);
-#endif
-    __syncthreads();
-#ifdef FSH_TRACE
-    lap(t_barrier);
-#endif
     stage ^= 1;
   }
 #ifdef FSH_TRACE
