@@ -291,15 +291,16 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams& p, uint8_t* l
     }
     if (part == 0) issue_scale_loads(kt, stage);
   };
-  // The block scales of the wave's 128 columns, one per k-tile, are copied
-  // to LDS once (a load from global memory inside the loop would again wait
-  // for the prefetched tile).
+  // The first k-tile's requests go out before anything else that has to wait
+  // for memory.  The block scales of the wave's 128 columns, one per k-tile,
+  // are copied to LDS once, under those requests (a load from global memory
+  // inside the loop would again wait for the prefetched tile).
+  issue_k_tile(0, 0);
   float* ws_lds = reinterpret_cast<float*>(lds_bytes + Cfg::kWeightScaleOffset + wave * Cfg::kMaxKTilesInLds * 4);
   if (!kColumnScales) {
     const float* ws_row = p.ws + wblock * p.ws_cb;
     for (int64_t i = lane; i < ktiles; i += 64) ws_lds[i] = ws_row[i * p.ws_kb];  // ktiles <= kMaxKTilesInLds (host check)
   }
-  issue_k_tile(0, 0);
   wait_for_dma_loads();
   __syncthreads();
 
