@@ -256,7 +256,7 @@ def check_against_oracle(placement, infos, work, metadata, payloads):
         raise SystemExit("bench: GPU payload differs from the oracle; refusing to report a timing")
 
 
-def cpu_baseline_quant(work, infos, metadata, budget_s: float = 20.0):
+def cpu_baseline_quant(work, infos, metadata, budget_s: float = 10.0):
     """The reference path in eager torch on the host: per chunk quantize
     (pad, amax, clamp, fp64 divide, multiply, clamp, cast), then copy data and
     scale bytes into the payload.  Same rank-0 share as the GPU step."""
@@ -281,7 +281,7 @@ def cpu_baseline_quant(work, infos, metadata, budget_s: float = 20.0):
     run()  # warm-up
     times = []
     t_end = time.perf_counter() + budget_s
-    while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 15):
+    while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 1000):  # about 10 s of host work
         t0 = time.perf_counter()
         run()
         times.append(time.perf_counter() - t0)
@@ -289,7 +289,7 @@ def cpu_baseline_quant(work, infos, metadata, budget_s: float = 20.0):
     return times[len(times) // 2], len(times), torch.get_num_threads()
 
 
-def cpu_baseline_gradients(reps: int = 5):
+def cpu_baseline_gradients(reps: int = 15):
     """Config 4 on the host cores, on a bounded sample: one rank range
     (27 295 744 elements, an eighth of the layer bucket) through the oracle's
     eager restatement of the fp32 microbatch accumulation (4 bf16 microbatches)
