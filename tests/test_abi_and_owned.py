@@ -57,6 +57,19 @@ def test_host_side_argument_checks_need_no_gpu():
     assert lib.fsh_newton_schulz(None, 1, 7, 8, 1.0, 1.0, 1.0, 5, 1e-7, None, 0, None) == -22
     assert lib.fsh_newton_schulz_workspace_bytes(24, 7168, 2048) > 2 * 24 * 7168 * 2048 * 2
     assert lib.fsh_accumulate_grad(None, None, 0, 0, 0, None) == 0  # empty is a no-op
+    # whole Muon step: list and group checks come before any launch
+    assert lib.fsh_muon_step(None, 1, 0.05, 0.95, 1, 1.0, 1.0, 1.0, 1.0, 5, 1e-7, None) == -22
+    assert b"null list" in lib.fsh_last_error()
+    assert lib.fsh_muon_step(None, 0, 0.05, 0.95, 1, 1.0, 1.0, 1.0, 1.0, 5, 1e-7, None) == 0  # no group: nothing to do
+    group = _native.MuonGroup()
+    group.batch, group.rows, group.cols = 1, 12, 8  # rows not a multiple of 8
+    assert lib.fsh_muon_step(ctypes.byref(group), 1, 0.05, 0.95, 1, 1.0, 1.0, 1.0, 1.0, 5, 1e-7, None) == -22
+    assert b"multiples of 8" in lib.fsh_last_error()
+    group.rows = 16
+    assert lib.fsh_muon_step(ctypes.byref(group), 1, 0.05, 0.95, 1, 1.0, 1.0, 1.0, 1.0, 5, 1e-7, None) == -22
+    assert b"null pointer" in lib.fsh_last_error()
+    # FP8 GEMM limits
+    assert lib.fsh_fp8_gemm_1x128_128x1(None, None, None, None, None, 8, 8, 100, 128, 128, 8, None) == -22
 
 
 def test_no_cpu_compute_path():
