@@ -554,6 +554,10 @@ def bench_fp8_linear_backward(device, tokens: int = 8192, reps: int = 10):
         us["quant_grad_t"] = ms / reps * 1e3
         _, ms = _event_ms(lambda i: hip_ops.act_quant_128x1_transposed(x), reps, 2)
         us["quant_x_t"] = ms / reps * 1e3
+        _, ms = _event_ms(lambda i: hip_ops.act_quant_1x128(g), reps, 2)
+        us["quant_grad"] = ms / reps * 1e3
+        _, ms = _event_ms(lambda i: hip_ops.act_quant_both(g), reps, 2)
+        us["quant_grad_both"] = ms / reps * 1e3
         wt = hip_ops.fp8_transpose(wq)
         gq, gs = hip_ops.act_quant_1x128(g)
         us["dgrad_gemm"] = _steady_us(lambda i: hip_ops.fp8_gemm_1x128_128x128_dgrad(gq, gs, wt, ws), 2 * reps)
@@ -567,6 +571,10 @@ def bench_fp8_linear_backward(device, tokens: int = 8192, reps: int = 10):
             "transpose_GBps": 2 * n * k / us["transpose"] / 1e3,  # 1 B read + 1 B written per element
             "quant_grad_transposed_us": us["quant_grad_t"],
             "quant_grad_transposed_GBps": tokens * n * (3 + 4 / 128) / us["quant_grad_t"] / 1e3,
+            # the output gradient in both forms: one pass (what the backward runs) against the two separate quantizers
+            "quant_grad_both_forms_us": us["quant_grad_both"],
+            "quant_grad_both_forms_GBps": tokens * n * (4 + 8 / 128) / us["quant_grad_both"] / 1e3,  # 2 B read + 2 x (1 B + 4/128 B) written
+            "quant_grad_rows_plus_transposed_us": us["quant_grad"] + us["quant_grad_t"],
             "quant_x_transposed_us": us["quant_x_t"],
             "quant_x_transposed_GBps": tokens * k * (3 + 4 / 128) / us["quant_x_t"] / 1e3,
             "dgrad_gemm_us": us["dgrad_gemm"],

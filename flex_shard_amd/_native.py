@@ -165,6 +165,10 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "fsh_act_quant_128x1_transposed": (
         c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int32, c_void_p],
     ),
+    "fsh_act_quant_both": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int32, c_void_p],
+    ),
     "fsh_fp8_gemm_1x128_128x128_dgrad": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,

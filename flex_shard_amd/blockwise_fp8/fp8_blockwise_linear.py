@@ -109,9 +109,15 @@ class Fp8BlockwiseGemms:
             )
         grad_output_2d = _as_quantizer_input(grad_output_2d)
         grad_x = grad_weight = None
+        grad_t_fp8 = grad_t_scale = None
         if needs_x_grad:
-            # runs of 128 along the output index; the quantizer zero-pads it to whole runs
-            grad_fp8, grad_scale = hip_ops.act_quant_1x128(grad_output_2d)
+            # runs of 128 along the output index; the quantizer zero-pads it to whole runs.
+            # When the weight gradient is wanted too, the same pass over grad_output
+            # also writes its token-run form.
+            if needs_weight_grad:
+                grad_fp8, grad_scale, grad_t_fp8, grad_t_scale = hip_ops.act_quant_both(grad_output_2d)
+            else:
+                grad_fp8, grad_scale = hip_ops.act_quant_1x128(grad_output_2d)
             if in_dim % 16 or weight_matrix.stride(1) != 1 or weight_matrix.stride(0) % 16:
                 weight_matrix = _pad_last_dim_to(weight_matrix.view(torch.uint8), -(-in_dim // 16) * 16).view(
                     torch.float8_e4m3fn
@@ -122,7 +128,8 @@ class Fp8BlockwiseGemms:
             )
         if needs_weight_grad:
             # runs of 128 tokens for both operands; the quantizer pads the token count itself
-            grad_t_fp8, grad_t_scale = hip_ops.act_quant_128x1_transposed(grad_output_2d)
+            if grad_t_fp8 is None:
+                grad_t_fp8, grad_t_scale = hip_ops.act_quant_128x1_transposed(grad_output_2d)
             x_t_fp8, x_t_scale = hip_ops.act_quant_128x1_transposed(_as_quantizer_input(x_2d))
             grad_weight = hip_ops.fp8_gemm_1x128_128x1(grad_t_fp8, grad_t_scale, x_t_fp8, x_t_scale)
             grad_weight = grad_weight[:out_dim, :in_dim].to(weight.dtype).contiguous().view(weight.shape)

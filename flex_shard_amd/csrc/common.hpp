@@ -69,6 +69,15 @@ __device__ __forceinline__ uint32_t dpp_max_u32(uint32_t v) {
       __builtin_amdgcn_update_dpp(static_cast<int>(v), static_cast<int>(v), CTRL, ROW_MASK, 0xF, false));
   return o > v ? o : v;
 }
+// Maximum over each row of 16 lanes, in every lane of the row.
+__device__ __forceinline__ uint32_t row16_max_u32(uint32_t v) {
+  v = dpp_max_u32<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
+  v = dpp_max_u32<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
+  v = dpp_max_u32<0x141, 0xF>(v);  // row_half_mirror
+  v = dpp_max_u32<0x140, 0xF>(v);  // row_mirror
+  return v;
+}
+
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
   v = dpp_max_u32<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
   v = dpp_max_u32<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]

@@ -40,14 +40,6 @@ struct ActQuantParams {
   float eps;
 };
 
-__device__ __forceinline__ uint32_t row16_max_u32(uint32_t v) {
-  v = dpp_max_u32<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
-  v = dpp_max_u32<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
-  v = dpp_max_u32<0x141, 0xF>(v);  // row_half_mirror
-  v = dpp_max_u32<0x140, 0xF>(v);  // row_mirror
-  return v;
-}
-
 __global__ __launch_bounds__(kActThreads) void act_quant_1x128_kernel(const ActQuantParams p) {
   __shared__ float lds_scales[kActBlocks * kActRows];
   const int tid = threadIdx.x;

@@ -87,13 +87,23 @@ struct ActQuantTParams {
   int64_t rows, cols, ldx, ldq;
   int32_t tiles_c;
   float eps;
+  // the row-run outputs of the dual kernel: q_row [rows][ldq_row], scales_row [ldq_row / 128][rows]
+  uint8_t* q_row;
+  float* scales_row;
+  int64_t ldq_row;
 };
 
 // Thread t loads columns [8 (t & 15), +8) of tile rows (t >> 4) + 16 k, k = 0..7.
+// kAlsoRowRuns: the same tile also leaves quantized in runs of 128 along its
+// rows (the arithmetic and the outputs of act_quant_1x128_kernel), so an
+// operand needed in both forms is read once.  A tile row's 128 columns lie in
+// one row of 16 lanes, whose maximum takes four DPP steps.
+template <bool kAlsoRowRuns>
 __global__ __launch_bounds__(kTransposeThreads) void act_quant_128x1_t_kernel(const ActQuantTParams p) {
   __shared__ __attribute__((aligned(16))) uint8_t tile[kTileDim * kTilePitch];
   __shared__ __attribute__((aligned(16))) uint16_t col_max[16 * kTileDim];
   __shared__ __attribute__((aligned(16))) float col_scale[kTileDim];
+  __shared__ float row_recip[kAlsoRowRuns ? kTileDim : 1];
   const int tid = threadIdx.x;
   const int cg = tid & 15, rl = tid >> 4;
   const int64_t rb = blockIdx.x / p.tiles_c;
@@ -106,6 +116,31 @@ __global__ __launch_bounds__(kTransposeThreads) void act_quant_128x1_t_kernel(co
     const int64_t row = r0 + rl + 16 * k;
     v[k] = u32x4{0, 0, 0, 0};
     if (row < p.rows && col < p.cols) v[k] = load_stream_u32x4(p.x + (row * p.ldx + col) * 2);  // cols % 8 == 0
+  }
+  if (kAlsoRowRuns) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int64_t row = r0 + rl + 16 * k;
+      uint32_t mr = pk_max_u16(v[k].x & 0x7FFF7FFFu, v[k].y & 0x7FFF7FFFu);
+      mr = pk_max_u16(mr, v[k].z & 0x7FFF7FFFu);
+      mr = pk_max_u16(mr, v[k].w & 0x7FFF7FFFu);
+      const uint32_t lo = mr & 0xFFFFu, hi = mr >> 16;
+      mr = row16_max_u32(lo > hi ? lo : hi);
+      float scale, recip;
+      tile_scale(bf16_bits_to_f32(mr), p.eps, scale, recip);
+      if (cg == 0) row_recip[rl + 16 * k] = recip;
+      if (row < p.rows && col < p.ldq_row) {  // columns past `cols` hold zeros: the pad of the last run
+        const uint32_t d[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+        uint32_t w[2] = {0, 0};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float e0 = u32_as_f32(d[j] << 16) * scale;
+          const float e1 = u32_as_f32(d[j] & 0xFFFF0000u) * scale;
+          w[j >> 1] = cvt2_fp8(e0, e1, w[j >> 1], (j & 1) != 0);
+        }
+        store_stream_u32x2(p.q_row + row * p.ldq_row + col, w[0], w[1]);
+      }
+    }
   }
   // Largest magnitude (bf16 bit pattern) of the thread's eight rows, per column.
   uint32_t m[4] = {0, 0, 0, 0};
@@ -129,6 +164,8 @@ __global__ __launch_bounds__(kTransposeThreads) void act_quant_128x1_t_kernel(co
     tile_scale(bf16_bits_to_f32(best), p.eps, scale, recip);
     col_scale[tid] = scale;
     if (c0 + tid < p.cols) p.scales[rb * p.cols + c0 + tid] = recip;
+    // (row_recip was filled before the first barrier above)
+    if (kAlsoRowRuns && r0 + tid < p.rows) p.scales_row[(c0 / kTileDim) * p.rows + r0 + tid] = row_recip[tid];
   }
   __syncthreads();
   const f32x4 s_lo = *reinterpret_cast<const f32x4*>(col_scale + cg * 8);
@@ -213,11 +250,51 @@ FSH_API int fsh_act_quant_128x1_transposed(const void* x_dev, int64_t rows, int6
   p.scales = scales_dev;
   p.rows = rows; p.cols = cols; p.ldx = ldx; p.ldq = ldq;
   p.eps = floor_for(eps_mode);
+  p.q_row = nullptr; p.scales_row = nullptr; p.ldq_row = 0;
   const int64_t tiles_c = ceil_div(cols, (int64_t)kTileDim);
   const int64_t grid = (padded / kTileDim) * tiles_c;
   if (grid > 0x7FFFFFFFLL) return fail(FSH_ENOTSUP, "fsh_act_quant_128x1_transposed: too many tiles");
   p.tiles_c = static_cast<int32_t>(tiles_c);
-  hipLaunchKernelGGL(act_quant_128x1_t_kernel, dim3(static_cast<uint32_t>(grid)), dim3(kTransposeThreads), 0,
+  hipLaunchKernelGGL(act_quant_128x1_t_kernel<false>, dim3(static_cast<uint32_t>(grid)), dim3(kTransposeThreads), 0,
                      static_cast<hipStream_t>(stream), p);
   return check_launch("act_quant_128x1_t_kernel");
+}
+
+FSH_API int fsh_act_quant_both(const void* x_dev, int64_t rows, int64_t cols, int64_t ldx, void* q_row_dev,
+                               int64_t ldq_row, float* scales_row_dev, void* q_col_dev, int64_t ldq_col,
+                               float* scales_col_dev, int32_t eps_mode, void* stream) {
+  using namespace fsh;
+  if (rows < 0 || cols < 0) return fail(FSH_EINVAL, "fsh_act_quant_both: negative shape");
+  if (rows == 0 || cols == 0) return FSH_OK;
+  if (!x_dev || !q_row_dev || !scales_row_dev || !q_col_dev || !scales_col_dev)
+    return fail(FSH_EINVAL, "fsh_act_quant_both: null pointer");
+  if (eps_mode != FSH_EPS_INPUT_DTYPE && eps_mode != FSH_EPS_FP32)
+    return fail(FSH_EINVAL, "fsh_act_quant_both: unknown eps_mode %d", eps_mode);
+  const int64_t padded_rows = ceil_div(rows, (int64_t)kTileDim) * kTileDim;
+  const int64_t padded_cols = ceil_div(cols, (int64_t)kTileDim) * kTileDim;
+  if (ldx < cols || ldq_col != padded_rows || ldq_row != padded_cols)
+    return fail(FSH_EINVAL,
+                "fsh_act_quant_both: ldx %lld < cols %lld, ldq_col %lld is not rows rounded up to 128 (%lld), or "
+                "ldq_row %lld is not cols rounded up to 128 (%lld)",
+                (long long)ldx, (long long)cols, (long long)ldq_col, (long long)padded_rows, (long long)ldq_row,
+                (long long)padded_cols);
+  if (cols % 8 || ldx % 8 || !aligned(x_dev, 16) || !aligned(q_col_dev, 16) || !aligned(q_row_dev, 8) ||
+      !aligned(scales_row_dev, 4) || !aligned(scales_col_dev, 4))
+    return fail(FSH_ENOTSUP, "fsh_act_quant_both: cols and ldx must be multiples of 8, x and q_col 16-byte and q_row 8-byte aligned");
+  ActQuantTParams p;
+  p.x = static_cast<const uint8_t*>(x_dev);
+  p.q = static_cast<uint8_t*>(q_col_dev);
+  p.scales = scales_col_dev;
+  p.rows = rows; p.cols = cols; p.ldx = ldx; p.ldq = ldq_col;
+  p.eps = floor_for(eps_mode);
+  p.q_row = static_cast<uint8_t*>(q_row_dev);
+  p.scales_row = scales_row_dev;
+  p.ldq_row = ldq_row;
+  const int64_t tiles_c = padded_cols / kTileDim;
+  const int64_t grid = (padded_rows / kTileDim) * tiles_c;
+  if (grid > 0x7FFFFFFFLL) return fail(FSH_ENOTSUP, "fsh_act_quant_both: too many tiles");
+  p.tiles_c = static_cast<int32_t>(tiles_c);
+  hipLaunchKernelGGL(act_quant_128x1_t_kernel<true>, dim3(static_cast<uint32_t>(grid)), dim3(kTransposeThreads), 0,
+                     static_cast<hipStream_t>(stream), p);
+  return check_launch("act_quant_128x1_t_kernel<true>");
 }

@@ -568,6 +568,32 @@ def act_quant_128x1_transposed(x: torch.Tensor, *, eps_fp32: bool = True) -> tup
     return q, scales
 
 
+def act_quant_both(
+    x: torch.Tensor, *, eps_fp32: bool = True
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """:func:`act_quant_1x128` and :func:`act_quant_128x1_transposed` of the same
+    bf16 matrix in one pass over it: returns ``(q_rows, scales_rows, q_cols,
+    scales_cols)``, each pair bit for bit what the respective function returns."""
+    _require_gpu(x)
+    if x.dtype != torch.bfloat16 or x.ndim != 2 or x.stride(1) != 1:
+        raise ValueError("x must be a bf16 matrix with contiguous rows")
+    rows, cols = x.shape
+    padded_rows, padded_cols = -(-rows // 128) * 128, -(-cols // 128) * 128
+    q_rows = torch.empty((rows, padded_cols), dtype=torch.float8_e4m3fn, device=x.device)
+    scales_rows = torch.empty((padded_cols // 128, rows), dtype=torch.float32, device=x.device)
+    q_cols = torch.empty((cols, padded_rows), dtype=torch.float8_e4m3fn, device=x.device)
+    scales_cols = torch.empty((padded_rows // 128, cols), dtype=torch.float32, device=x.device)
+    if rows == 0 or cols == 0:
+        return q_rows, scales_rows, q_cols, scales_cols
+    status = _native.lib().fsh_act_quant_both(
+        x.data_ptr(), rows, cols, x.stride(0), q_rows.data_ptr(), padded_cols, scales_rows.data_ptr(),
+        q_cols.data_ptr(), padded_rows, scales_cols.data_ptr(), EPS_FP32 if eps_fp32 else EPS_INPUT_DTYPE,
+        stream_ptr(x.device),
+    )
+    _native.check(status, "fsh_act_quant_both")
+    return q_rows, scales_rows, q_cols, scales_cols
+
+
 def fp8_gemm_1x128_128x128_dgrad(
     gq: torch.Tensor, gs: torch.Tensor, wtq: torch.Tensor, ws: torch.Tensor, in_dim: int | None = None
 ) -> torch.Tensor:

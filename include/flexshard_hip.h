@@ -318,6 +318,15 @@ int fsh_fp8_gemm_1x128_128x128(const void* xq_dev, const float* xs_dev, const vo
  * q[c][r], ldq = rows rounded up to 128 with the pad written as zero;
  * scales_dev is the [ldq / 128, cols] table of 1.0f / scale.
  *
+ * fsh_act_quant_both: the output gradient is needed in both forms (runs along
+ * the output index for the input gradient, :107-110; runs of 128 tokens,
+ * transposed, for the weight gradient, :134-138).  One pass over x writes what
+ * fsh_act_quant_1x128 (q_row_dev [rows, ldq_row], scales_row_dev
+ * [ldq_row / 128, rows]; ldq_row = cols rounded up to 128) and
+ * fsh_act_quant_128x1_transposed (q_col_dev [cols, ldq_col], scales_col_dev
+ * [ldq_col / 128, cols]; ldq_col = rows rounded up to 128) would write, bit
+ * for bit, reading x once instead of twice.
+ *
  * fsh_fp8_gemm_1x128_128x128_dgrad:
  *   out[i][j] = bf16( sum over ob of dot(gq[i][ob], wtq[j][ob])
  *                                  * (gs[ob][i] * ws[ob][j / 128]) ),
@@ -336,6 +345,9 @@ int fsh_fp8_transpose(const void* src_dev, int64_t rows, int64_t cols, int64_t l
                       int64_t ld_dst, void* stream);
 int fsh_act_quant_128x1_transposed(const void* x_dev, int64_t rows, int64_t cols, int64_t ldx, void* q_dev,
                                    int64_t ldq, float* scales_dev, int32_t eps_mode, void* stream);
+int fsh_act_quant_both(const void* x_dev, int64_t rows, int64_t cols, int64_t ldx, void* q_row_dev,
+                       int64_t ldq_row, float* scales_row_dev, void* q_col_dev, int64_t ldq_col,
+                       float* scales_col_dev, int32_t eps_mode, void* stream);
 int fsh_fp8_gemm_1x128_128x128_dgrad(const void* gq_dev, const float* gs_dev, const void* wtq_dev,
                                      const float* ws_dev, void* out_dev, int64_t m, int64_t in_dim,
                                      int64_t out_dim, int64_t ldgq, int64_t ldwt, int64_t ldo,

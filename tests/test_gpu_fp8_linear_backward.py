@@ -74,6 +74,37 @@ def test_token_run_quantizer_is_bit_exact(device, rows, cols):
     assert torch.equal(_bits(s.cpu()), _bits(os_))
 
 
+@pytest.mark.parametrize("rows,cols", [(128, 128), (256, 384), (130, 136), (77, 8), (1000, 520), (4096, 256), (1, 128)])
+def test_both_forms_in_one_pass_equal_the_two_quantizers(device, rows, cols):
+    """One read of the matrix, both outputs: bit for bit what the row-run and
+    the token-run quantizer write on their own (pads included), and the
+    oracle's bytes."""
+    gen = torch.Generator().manual_seed(rows * 7 + cols)
+    x = (torch.randn(rows, cols, generator=gen) * 0.5).bfloat16()
+    x[torch.rand(rows, cols, generator=gen) < 0.002] *= 60
+    if rows >= 256:
+        x[128:256, cols // 2] = 0
+        x[3, :] = 0  # an all-zero row run
+    x[rows - 1, cols - 1] = 3.0e38
+    xd = x.to(device)
+    q_rows, s_rows, q_cols, s_cols = hip_ops.act_quant_both(xd)
+    want_q_rows, want_s_rows = hip_ops.act_quant_1x128(xd)
+    want_q_cols, want_s_cols = hip_ops.act_quant_128x1_transposed(xd)
+    for got, want in ((q_rows, want_q_rows), (q_cols, want_q_cols)):
+        assert got.shape == want.shape and torch.equal(got.view(torch.uint8), want.view(torch.uint8))
+    for got, want in ((s_rows, want_s_rows), (s_cols, want_s_cols)):
+        assert got.shape == want.shape and torch.equal(_bits(got.cpu()), _bits(want.cpu()))
+    oq, os_ = eager.act_quant_1x128(x)
+    assert torch.equal(q_rows.cpu().view(torch.uint8), oq.view(torch.uint8)) and torch.equal(_bits(s_rows.cpu()), _bits(os_))
+    # strided rows and the bf16-rounded floor
+    wide = torch.randn(300, 640, generator=gen).bfloat16().to(device)
+    view = wide[:, 128:512]
+    a = hip_ops.act_quant_both(view, eps_fp32=False)
+    b = hip_ops.act_quant_1x128(view, eps_fp32=False) + hip_ops.act_quant_128x1_transposed(view, eps_fp32=False)
+    assert all(torch.equal(u.view(torch.uint8) if u.dtype != torch.float32 else u, v.view(torch.uint8) if v.dtype != torch.float32 else v)
+               for u, v in zip(a, b))
+
+
 def test_token_run_quantizer_strided_rows_and_eps_switch(device):
     gen = torch.Generator().manual_seed(4)
     wide = torch.randn(300, 640, generator=gen).bfloat16().to(device)
