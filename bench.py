@@ -125,27 +125,29 @@ def build_quant_workload(device, layers: int, rank: int = 0, spec=None, std: flo
 
 def bench_quant_pack(device, steps, warmup, layers, rank: int = 0, spec=None, std: float = 0.02, extras: bool = False):
     """One step = one pass over the `layers` layer buckets: one fused
-    quantize+pack launch per bucket through the placement."""
+    quantize+pack launch per bucket through the placement's contract entry,
+    `prepare_unshard_bucket` (payload-cache bookkeeping, the launch, the
+    W x row gather output).  The two most recent prepared unshards are held,
+    as a runtime with one bucket prefetched holds them."""
+    import collections
+
     placement, mesh, infos, work = build_quant_workload(device, layers, rank, spec, std)
     metadata = placement._quant_metadata_from_infos(infos)
     plan = metadata.rank_pack_plans[rank]
     elems = plan.qdata_numel
     scales = sum(sum(c.scale_numels) for c in plan.chunks)
     algo_bytes = 3 * elems + 4 * scales  # 2 B read + 1 B write per element, 4 B per tile scale
-    payloads = [torch.empty(metadata.packed_send_nbytes_per_rank, dtype=torch.uint8, device=device) for _ in work]
+    held = collections.deque(maxlen=2)
 
     def launch(layer):
-        # The placement's pack step; the payload buffer is recycled the way the
-        # caching allocator recycles it in a training loop.
-        payloads[layer] = placement._pack_local_quantized_chunks(work[layer][1], infos, rank, metadata)
+        held.append(placement.prepare_unshard_bucket(work[layer][1], infos, mesh, None))
 
     def step(i):
         for layer in range(len(work)):
             launch(layer)
 
-    # Steady state first, independent of --warmup: every bucket's launch table
-    # is built and cached and every payload block has been through the
-    # allocator before the clock starts.
+    # Steady state first, independent of --warmup: every bucket's launch is
+    # stored and the recycled buffers exist before the clock starts.
     for _ in range(2):
         step(0)
     torch.cuda.synchronize()
@@ -158,7 +160,7 @@ def bench_quant_pack(device, steps, warmup, layers, rank: int = 0, spec=None, st
         "event_ms": event_ms,
         "payload_nbytes": metadata.packed_send_nbytes_per_rank,
         "chunks": len(plan.chunks),
-        "work": (placement, infos, work, metadata, payloads),
+        "work": (placement, infos, work, metadata, mesh),
     }
     if not extras:
         return out
@@ -167,54 +169,50 @@ def bench_quant_pack(device, steps, warmup, layers, rank: int = 0, spec=None, st
     _, hot_ms = _event_ms(lambda i: launch(0), n, 5)
     out["hot_us"] = hot_ms / n * 1e3
 
-    # The contract entry: prepare_unshard_bucket = payload-cache bookkeeping,
-    # pack, and the allocation of the W x row gather output.  Host time is the
-    # time the calls take to issue (nothing waits for the GPU inside them).
-    for layer in range(len(work)):
-        placement.prepare_unshard_bucket(work[layer][1], infos, mesh, None)
+    # Host time of the contract entry: the time the calls take to issue
+    # (nothing waits for the GPU inside them), the queue drained first.
     torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    start.record()
-    for i in range(n):
-        placement.prepare_unshard_bucket(work[i % len(work)][1], infos, mesh, None)
-    t_issued = time.perf_counter()
-    stop.record()
-    torch.cuda.synchronize()
-    out["contract_us"] = start.elapsed_time(stop) / n * 1e3
-    out["contract_host_us"] = (t_issued - t0) / n * 1e6
     t0 = time.perf_counter()
     for i in range(n):
         launch(i % len(work))
-    out["pack_host_us"] = (time.perf_counter() - t0) / n * 1e6
+    out["contract_host_us"] = (time.perf_counter() - t0) / n * 1e6
     torch.cuda.synchronize()
 
-    # Two buckets in flight on two streams of the same (default) priority, the
-    # way a prefetching runtime issues the next bucket's pack while the current
-    # one drains: launches alternate between the streams.  The cached launch
-    # tables are launched directly on each stream into payloads allocated
-    # beforehand (a stream switch through torch costs more host time than the
-    # kernel runs), so what is timed is the overlap of the kernels.
-    plans = [placement._pack_launches[sig][1] for sig in list(placement._pack_launches)][-len(work):]
-    if len(plans) != len(work):
-        raise SystemExit("bench: expected one cached pack launch per layer bucket")
+    # Two buckets in flight: the same contract calls with torch's current
+    # stream alternating between two side streams of the same (default)
+    # priority, the way a runtime that prefetches the next bucket issues them;
+    # the ramp and drain of one launch overlap the other's.  Payloads and
+    # gather outputs come from each stream's own recycled buffers.
     streams = [torch.cuda.Stream(device), torch.cuda.Stream(device)]
-    spare = [torch.empty_like(payloads[0]) for _ in range(2 * len(work))]
-    torch.cuda.synchronize()
-    for rep in range(2):  # the first repetition warms both streams
-        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record(streams[0])
-        fence = torch.cuda.Event()
-        fence.record(streams[0])
-        streams[1].wait_event(fence)
-        for i in range(n):
-            plans[i % len(work)].launch(spare[i % len(spare)], stream=streams[i % 2])
-        joined = torch.cuda.Event()
-        joined.record(streams[1])
-        streams[0].wait_event(joined)
-        stop.record(streams[0])
-        torch.cuda.synchronize()
+    main = torch.cuda.current_stream(device)
+    held2 = [collections.deque(maxlen=2), collections.deque(maxlen=2)]
+
+    def issue(i):
+        torch.cuda.set_stream(streams[i % 2])
+        held2[i % 2].append(placement.prepare_unshard_bucket(work[i % len(work)][1], infos, mesh, None))
+
+    try:
+        for rep in range(2):  # the first repetition creates both streams' buffers
+            torch.cuda.synchronize()
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record(streams[0])
+            fence = torch.cuda.Event()
+            fence.record(streams[0])
+            streams[1].wait_event(fence)
+            t0 = time.perf_counter()
+            for i in range(n):
+                issue(i)
+            host = time.perf_counter() - t0
+            joined = torch.cuda.Event()
+            joined.record(streams[1])
+            streams[0].wait_event(joined)
+            stop.record(streams[0])
+            torch.cuda.synchronize()
+    finally:
+        torch.cuda.set_stream(main)
     out["two_stream_us"] = start.elapsed_time(stop) / n * 1e3
+    out["two_stream_host_us"] = host / n * 1e6
+    out["two_stream_last"] = (held2, streams)
     return out
 
 
@@ -239,13 +237,17 @@ def bench_other_shares(device):
     return out
 
 
-def check_against_oracle(placement, infos, work, metadata, payloads):
-    """Bit-exactness gate before any timing is reported: one chunk of the last
-    payload against the C oracle."""
+def check_against_oracle(placement, infos, work, metadata, mesh, prepared=None):
+    """Bit-exactness gate before any timing is reported: one chunk of a
+    payload produced through the contract entry against the C oracle.
+    `prepared`: a prepared unshard of layer bucket 0 to check instead of a
+    fresh one."""
     from oracle import cport
 
     storage, shards = work[0]
-    payload = placement._pack_local_quantized_chunks(shards, infos, 0, metadata).cpu()
+    if prepared is None:
+        prepared = placement.prepare_unshard_bucket(shards, infos, mesh, None)
+    payload = prepared.buffers[0].cpu()
     k = shards[1].detach().cpu().flatten(0, -2)
     oq, osc = cport.quantize_blockwise(k, 128)
     start = shards[0].numel()
@@ -640,8 +642,9 @@ def main() -> None:
     if args.calibrate_copy:
         calibrate_copy(device)
     q = bench_quant_pack(device, args.steps, args.warmup, args.layers, extras=True)
-    placement, infos, work, metadata, payloads = q.pop("work")
-    check_against_oracle(placement, infos, work, metadata, payloads)
+    placement, infos, work, metadata, mesh = q.pop("work")
+    check_against_oracle(placement, infos, work, metadata, mesh)
+    q.pop("two_stream_last")
     launches = args.steps * q["launches_per_step"]
     step_bytes = q["algo_bytes"] * q["launches_per_step"]
     ms_per_step = q["wall_ms"] / args.steps
@@ -690,16 +693,17 @@ def main() -> None:
         # time either call takes to issue, and the rate with two buckets in
         # flight on two default-priority streams.
         "contract_entry": {
-            "prepare_unshard_bucket_us_per_call": round(q["contract_us"], 2),
-            "prepare_unshard_bucket_GBps": round(q["algo_bytes"] / q["contract_us"] / 1e3, 1),
+            "entry": "Fp8BucketedBlockShard.prepare_unshard_bucket (what `value` and `roofline` are timed through)",
             "prepare_unshard_bucket_host_us_per_call": round(q["contract_host_us"], 2),
-            "pack_step_host_us_per_call": round(q["pack_host_us"], 2),
-        },
-        "two_buckets_in_flight": {
-            "streams": 2,
-            "us_per_launch": round(q["two_stream_us"], 2),
-            "GBps": round(q["algo_bytes"] / q["two_stream_us"] / 1e3, 1),
-            "frac_of_hbm_peak": round(q["algo_bytes"] / q["two_stream_us"] / 1e3 / HBM_PEAK_GBPS, 4),
+            "two_buckets_in_flight": {
+                "how": "the same calls with torch's current stream alternating between two default-priority "
+                "side streams (torch.cuda.set_stream), payloads from each stream's recycled buffers",
+                "streams": 2,
+                "us_per_launch": round(q["two_stream_us"], 2),
+                "host_us_per_call": round(q["two_stream_host_us"], 2),
+                "GBps": round(q["algo_bytes"] / q["two_stream_us"] / 1e3, 1),
+                "frac_of_hbm_peak": round(q["algo_bytes"] / q["two_stream_us"] / 1e3 / HBM_PEAK_GBPS, 4),
+            },
         },
     }
     if not args.skip_cpu:
@@ -712,7 +716,7 @@ def main() -> None:
             "sample": f"eager-torch restatement of the reference path on the same rank-0 share "
             f"({q['elems']} elements), median of {reps} runs, {threads} threads of {os.cpu_count()} logical CPUs",
         }
-    del work, payloads
+    del work
     torch.cuda.empty_cache()
     if not args.skip_secondary:
         secondary = {}

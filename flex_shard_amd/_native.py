@@ -130,6 +130,12 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         c_int,
         [POINTER(QuantChunk), c_int32, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int32, c_int32, c_void_p],
     ),
+    "fsh_quant_pack_plan_create": (
+        c_int,
+        [POINTER(QuantChunk), c_int32, c_int64, c_int64, c_int64, c_int64, c_int64, c_int32, c_int32, POINTER(c_void_p)],
+    ),
+    "fsh_quant_pack_plan_launch": (c_int, [c_void_p, c_void_p, c_void_p]),
+    "fsh_quant_pack_plan_destroy": (None, [c_void_p]),
     "fsh_copy_segments": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_void_p]),
     "fsh_zero_segments": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_void_p]),
     "fsh_pack_segments": (

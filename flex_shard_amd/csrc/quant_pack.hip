@@ -18,6 +18,10 @@
 //            +-448 never changes a finite product: |x| <= amax bounds it by
 //            448 * (1 + 2^-23), which rounds to 448 either way)
 //   stored = 1.0f / scale                       (IEEE fp32 division)
+#include <algorithm>
+#include <new>
+#include <vector>
+
 #include "common.hpp"
 
 namespace fsh {
@@ -430,10 +434,89 @@ float bf16_round_host(float f) {
 }  // namespace
 }  // namespace fsh
 
+// A reusable launch: the arguments of fsh_quantize_pack except the payload
+// address and the stream.  More than FSH_MAX_QUANT_CHUNKS chunks become several
+// launches, the first of which also zeroes the pad ranges.
+struct fsh_quant_pack_plan {
+  std::vector<fsh_quant_chunk> chunks;
+  int64_t payload_nbytes;
+  int64_t zero[4];
+  int32_t block;
+  int32_t eps_mode;
+};
+
+static int quantize_pack_impl(const fsh_quant_chunk* chunks, int32_t nchunks, void* payload_dev,
+                              int64_t payload_nbytes, int64_t zero0_begin, int64_t zero0_end,
+                              int64_t zero1_begin, int64_t zero1_end, int32_t block,
+                              int32_t eps_mode, void* stream, bool launch);
+
 FSH_API int fsh_quantize_pack(const fsh_quant_chunk* chunks, int32_t nchunks, void* payload_dev,
                               int64_t payload_nbytes, int64_t zero0_begin, int64_t zero0_end,
                               int64_t zero1_begin, int64_t zero1_end, int32_t block,
                               int32_t eps_mode, void* stream) {
+  return quantize_pack_impl(chunks, nchunks, payload_dev, payload_nbytes, zero0_begin, zero0_end, zero1_begin,
+                            zero1_end, block, eps_mode, stream, true);
+}
+
+FSH_API int fsh_quant_pack_plan_create(const fsh_quant_chunk* chunks, int32_t nchunks, int64_t payload_nbytes,
+                                       int64_t zero0_begin, int64_t zero0_end, int64_t zero1_begin,
+                                       int64_t zero1_end, int32_t block, int32_t eps_mode, void** plan_out) {
+  using namespace fsh;
+  if (plan_out == nullptr) return fail(FSH_EINVAL, "fsh_quant_pack_plan_create: null plan_out");
+  *plan_out = nullptr;
+  if (nchunks < 0 || (nchunks > 0 && chunks == nullptr))
+    return fail(FSH_EINVAL, "fsh_quant_pack_plan_create: bad chunk table (%d chunks)", nchunks);
+  // Every launch of the plan is checked now, against a stand-in payload
+  // address with the alignment a launch will ask for; nothing is queued.
+  void* const probe = reinterpret_cast<void*>(static_cast<uintptr_t>(4096));
+  int32_t first = 0;
+  do {
+    const int32_t count = std::min<int32_t>(nchunks - first, FSH_MAX_QUANT_CHUNKS);
+    const bool lead = first == 0;
+    const int status = quantize_pack_impl(chunks + first, count, payload_nbytes > 0 ? probe : nullptr, payload_nbytes,
+                                          lead ? zero0_begin : 0, lead ? zero0_end : 0, lead ? zero1_begin : 0,
+                                          lead ? zero1_end : 0, block, eps_mode, nullptr, false);
+    if (status != FSH_OK) return status;
+    first += count;
+  } while (first < nchunks);
+  fsh_quant_pack_plan* plan = new (std::nothrow) fsh_quant_pack_plan();
+  if (plan == nullptr) return fail(FSH_EINVAL, "fsh_quant_pack_plan_create: out of host memory");
+  plan->chunks.assign(chunks, chunks + nchunks);
+  plan->payload_nbytes = payload_nbytes;
+  plan->zero[0] = zero0_begin, plan->zero[1] = zero0_end, plan->zero[2] = zero1_begin, plan->zero[3] = zero1_end;
+  plan->block = block;
+  plan->eps_mode = eps_mode;
+  *plan_out = plan;
+  return FSH_OK;
+}
+
+FSH_API int fsh_quant_pack_plan_launch(const void* plan_handle, void* payload_dev, void* stream) {
+  using namespace fsh;
+  if (plan_handle == nullptr) return fail(FSH_EINVAL, "fsh_quant_pack_plan_launch: null plan");
+  const fsh_quant_pack_plan& plan = *static_cast<const fsh_quant_pack_plan*>(plan_handle);
+  const int32_t nchunks = static_cast<int32_t>(plan.chunks.size());
+  int32_t first = 0;
+  do {
+    const int32_t count = std::min<int32_t>(nchunks - first, FSH_MAX_QUANT_CHUNKS);
+    const bool lead = first == 0;
+    const int status =
+        quantize_pack_impl(plan.chunks.data() + first, count, payload_dev, plan.payload_nbytes,
+                           lead ? plan.zero[0] : 0, lead ? plan.zero[1] : 0, lead ? plan.zero[2] : 0,
+                           lead ? plan.zero[3] : 0, plan.block, plan.eps_mode, stream, true);
+    if (status != FSH_OK) return status;
+    first += count;
+  } while (first < nchunks);
+  return FSH_OK;
+}
+
+FSH_API void fsh_quant_pack_plan_destroy(void* plan_handle) {
+  delete static_cast<fsh_quant_pack_plan*>(plan_handle);
+}
+
+static int quantize_pack_impl(const fsh_quant_chunk* chunks, int32_t nchunks, void* payload_dev,
+                              int64_t payload_nbytes, int64_t zero0_begin, int64_t zero0_end,
+                              int64_t zero1_begin, int64_t zero1_end, int32_t block,
+                              int32_t eps_mode, void* stream, bool launch) {
   using namespace fsh;
   if (nchunks < 0 || nchunks > FSH_MAX_QUANT_CHUNKS)
     return fail(FSH_EINVAL, "fsh_quantize_pack: nchunks %d outside [0, %d]", nchunks, FSH_MAX_QUANT_CHUNKS);
@@ -506,6 +589,7 @@ FSH_API int fsh_quantize_pack(const fsh_quant_chunk* chunks, int32_t nchunks, vo
   const int64_t grid = tiles + ceil_div(zero_total, kZeroChunk);
   if (grid == 0) return FSH_OK;
   if (grid > 0x7FFFFFFFLL) return fail(FSH_ENOTSUP, "fsh_quantize_pack: %lld workgroups exceed the grid limit", (long long)grid);
+  if (!launch) return FSH_OK;
   if (all_bf16_fast) {
     if (nchunks < 8)
       launch_bf16_kernel<8>(prm, tiles, grid, static_cast<hipStream_t>(stream));

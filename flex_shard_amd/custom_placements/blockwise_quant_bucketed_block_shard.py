@@ -17,6 +17,7 @@ tensors off the GPU raise.
 
 from __future__ import annotations
 
+import sys
 from collections.abc import Sequence
 from dataclasses import dataclass
 from typing import TYPE_CHECKING, Any
@@ -116,6 +117,113 @@ def _require_gpu_rows(tensor: torch.Tensor, what: str) -> None:
         )
 
 
+_getrefcount = sys.getrefcount
+_storage_use_count = torch._C._storage_Use_Count
+_raw_stream = torch._C._cuda_getCurrentRawStream
+
+PAYLOAD_RING_SLOTS = 4
+GATHER_RING_SLOTS = 2
+
+
+class _QuantUnshardState:
+    """The placement's private state of one prepared unshard."""
+
+    __slots__ = ("infos", "pg", "debug_fqn", "metadata")
+
+    def __init__(self, infos: list, pg: Any, debug_fqn: str | None, metadata: quant_plan.QuantBucketMetadata) -> None:
+        self.infos, self.pg, self.debug_fqn, self.metadata = infos, pg, debug_fqn, metadata
+
+
+class _LocalPackedCacheEntry:
+    """A forward pack a backward re-gather may take once.  ``signature`` names
+    the sources (address, dtype, shape, strides, negative bit, quantization
+    dtype of every shard that holds rows), ``versions`` their version counters
+    at pack time and ``stream`` the raw stream the pack was queued on;
+    ``sources`` keeps the shards' storage alive, so that an equal address still
+    means the same memory, and ``infos`` pins the ParamInfo objects by identity."""
+
+    __slots__ = ("signature", "versions", "stream", "metadata", "infos", "sources", "packed")
+
+    def __init__(self, signature, versions, stream, metadata, infos, sources, packed) -> None:
+        self.signature, self.versions, self.stream, self.metadata = signature, versions, stream, metadata
+        self.infos, self.sources, self.packed = infos, sources, packed
+
+
+class _BufferRing:
+    """A few recycled uint8 buffers of one size, allocated under one stream.
+
+    ``take`` hands out a buffer that nobody else refers to any more: the
+    tensor object has no other Python holder and no C++ holder (a collective's
+    work object keeps its operands), and its storage is shared by no view or
+    alias.  That makes reuse *on the ring's stream* safe under the ownership
+    rule of ``PlacementPreparedUnshard.buffers``: the runtime drops its
+    references only after every other stream that read a buffer has been
+    ordered before the stream that allocated it, which is what the caching
+    allocator needs as well.  When every slot is held, the buffer comes from
+    the allocator and is not kept, so the ring never holds more than ``slots``
+    buffers and a caller that keeps payloads (the backward cache does, one per
+    bucket) simply gets fresh ones."""
+
+    __slots__ = ("nbytes", "device", "capacity", "_slots")
+
+    def __init__(self, nbytes: int, device: torch.device, capacity: int) -> None:
+        self.nbytes, self.device, self.capacity = nbytes, device, capacity
+        self._slots: list[list] = []
+
+    def take(self) -> tuple[torch.Tensor, int]:
+        """A free buffer and its device address."""
+        for slot in self._slots:
+            if _getrefcount(slot[0]) == slot[3] and slot[0]._use_count() == 1 and _storage_use_count(slot[2]) == slot[4]:
+                return slot[0], slot[1]
+        tensor = torch.empty(self.nbytes, dtype=torch.uint8, device=self.device)
+        address = tensor.data_ptr()
+        if len(self._slots) < self.capacity:
+            storage = tensor.untyped_storage()
+            slot = [tensor, address, storage._cdata, 0, 0, storage]
+            # the counts of a free slot: what they read now, minus this frame's own reference
+            slot[3] = _getrefcount(slot[0]) - 1
+            slot[4] = _storage_use_count(slot[2])
+            self._slots.append(slot)
+        return tensor, address
+
+
+class _SteadyPack:
+    """The stored launch of one rank's quantize + pack for shards that stay
+    where they are, with the rings its payloads and gather outputs come from
+    (one pair per stream the bucket is prepared on)."""
+
+    __slots__ = (
+        "layout", "metadata", "rank", "ntensors", "infos", "live", "signature", "launch", "device", "device_index",
+        "cache_key", "payload_nbytes", "gathered_nbytes", "rings",
+    )
+
+    def __init__(self, *, layout, metadata, rank, ntensors, infos, live, signature, launch, device, world_size) -> None:
+        self.layout, self.metadata, self.rank, self.ntensors = layout, metadata, rank, ntensors
+        self.infos, self.live, self.signature, self.launch, self.device = infos, live, signature, launch, device
+        self.device_index = torch.cuda.current_device() if device.index is None else device.index
+        self.cache_key = (rank, id(metadata))
+        self.payload_nbytes = metadata.packed_send_nbytes_per_rank
+        self.gathered_nbytes = world_size * self.payload_nbytes
+        self.rings: dict[int, tuple[_BufferRing, _BufferRing]] = {}
+
+    def rings_for(self, stream: int, shared: dict) -> tuple[_BufferRing, _BufferRing]:
+        """This bucket's payload and gather-output rings on ``stream``, taken
+        from (or added to) ``shared``, the placement's rings by (device,
+        stream, size): buckets of one size, like the layers of a model, share
+        them, so the recycled memory does not grow with the number of buckets."""
+        if len(self.rings) >= 4:  # a bucket is prepared on one or two streams; do not grow without bound
+            self.rings.clear()
+        pair = []
+        for nbytes, slots in ((self.payload_nbytes, PAYLOAD_RING_SLOTS), (self.gathered_nbytes, GATHER_RING_SLOTS)):
+            key = (self.device, stream, nbytes, slots)
+            ring = shared.get(key)
+            if ring is None:
+                ring = shared[key] = _BufferRing(nbytes, self.device, slots)
+            pair.append(ring)
+        rings = self.rings[stream] = (pair[0], pair[1])
+        return rings
+
+
 class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
     """Bucketed block shard that all-gathers blockwise-quantized weights.
 
@@ -141,12 +249,7 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         bucket_layout: Any
         metadata: quant_plan.QuantBucketMetadata
 
-    @dataclass(frozen=True)
-    class _QuantUnshardState:
-        infos: list
-        pg: Any
-        debug_fqn: str | None
-        metadata: quant_plan.QuantBucketMetadata
+    _QuantUnshardState = _QuantUnshardState
 
     @dataclass(frozen=True)
     class _CopyOutPlan:
@@ -158,22 +261,6 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         regions: tuple[tuple[int, int, int, int], ...]
         vec_aligned: bool
         descriptors: dict
-
-    @dataclass(frozen=True)
-    class _LocalPackedCacheEntry:
-        """A forward pack a backward re-gather may take once.  ``signature``
-        names the sources (address, dtype, shape, strides, negative bit) and
-        the quantization dtypes, ``versions`` their version counters at pack
-        time; ``sources`` keeps the shards' storage alive, so that an equal
-        address still means the same memory, and ``infos`` pins the ParamInfo
-        objects by identity."""
-
-        signature: tuple
-        versions: tuple
-        sources: tuple
-        infos: tuple
-        metadata: quant_plan.QuantBucketMetadata
-        packed: torch.Tensor
 
     def __init__(self, *, world_size: int, shard_block_rows: int, qdata_dtype: torch.dtype) -> None:
         if world_size <= 0:
@@ -188,7 +275,8 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         self._local_packed_cache: dict = {}
         self._copy_out_plans: dict = {}
         self._unpack_tables: dict = {}
-        self._pack_launches: dict = {}
+        self._steady_packs: dict = {}
+        self._buffer_rings: dict = {}
 
     @property
     def world_size(self) -> int:
@@ -418,62 +506,57 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         return GlobalLayout(shape, tuple(g_off), tuple(l_off), tuple(sizes))
 
     # ------------------------------------------------ local quantize + pack
-    @staticmethod
-    def _pack_signature(
-        tensors: list[torch.Tensor], infos: list["ParamInfo"], rank: int, metadata: quant_plan.QuantBucketMetadata
-    ) -> tuple:
-        """What a cached launch table and a cached payload depend on besides
-        the shards' contents: which memory the shards are (address, dtype,
-        shape, strides, negative bit; bf16 and fp32 shards have no conjugate
-        bit) and the dtype each is quantized in."""
-        return (
-            id(metadata),
-            rank,
-            tuple((t.data_ptr(), t.dtype, t.shape, t.stride(), t.is_neg()) for t in tensors),
-            tuple(info.unsharded_dtype for info in infos),
-        )
+    def _shard_signature(self, tensors: list[torch.Tensor], infos: list["ParamInfo"], live: tuple[int, ...]):
+        """What a stored launch and a cached payload depend on besides the
+        shards' contents, for the shards that hold rows (``live``): which
+        memory each is (address, dtype, shape, strides, negative bit; bf16 and
+        fp32 shards have no conjugate bit) and the dtype it is quantized in.
+        Also returns the shards' version counters."""
+        signature, versions = [], []
+        for index in live:
+            t = tensors[index]
+            signature.append((t.data_ptr(), t.dtype, t.shape, t.stride(), t.is_neg(), infos[index].unsharded_dtype))
+            versions.append(t._version)
+        return signature, versions
 
-    @staticmethod
-    def _local_packed_cache_context(tensors: list[torch.Tensor]) -> tuple[torch.device, int]:
-        """Device and raw current stream: a cached payload is only valid for
-        consumers ordered after the stream it was packed on."""
-        device = next((t.device for t in tensors if t.numel() > 0), tensors[0].device)
-        return device, hip_ops.stream_ptr(device)
+    def _steady_pack_for(
+        self, tensors: list[torch.Tensor], infos: list["ParamInfo"], rank: int
+    ) -> "tuple[_SteadyPack | None, list | None, list | None]":
+        """The stored launch of these very shards, with their signature and
+        version counters; (None, None, None) when there is none (first call,
+        shards that moved, staged shards)."""
+        group = self._steady_packs.get((id(infos[0].bucket_layout), rank))
+        if group is None:
+            return None, None, None
+        live, by_first_address = group
+        steady = by_first_address.get(tensors[live[0]].data_ptr() if live else 0)
+        if steady is None or steady.layout is not infos[0].bucket_layout or len(tensors) != steady.ntensors:
+            return None, None, None
+        for index in live:
+            if infos[index] is not steady.infos[index]:
+                return None, None, None
+        signature, versions = self._shard_signature(tensors, infos, live)
+        if signature != steady.signature:
+            return None, None, None
+        return steady, signature, versions
 
-    def _pack_local_quantized_chunks(
-        self,
-        tensors: list[torch.Tensor],
-        infos: list["ParamInfo"],
-        rank: int,
-        metadata: quant_plan.QuantBucketMetadata,
-        signature: tuple | None = None,
-    ) -> torch.Tensor:
-        """Quantize this rank's dense shards and pack them, in one launch, into
-        a fresh payload ``[data | pad | scales | pad]`` of the common row size.
-        ``signature``: ``_pack_signature`` of the arguments when the caller has
-        it already."""
+    def _build_pack_launch(
+        self, tensors: list[torch.Tensor], infos: list["ParamInfo"], rank: int, metadata: quant_plan.QuantBucketMetadata
+    ) -> tuple[hip_ops.QuantPackPlan, list[torch.Tensor], torch.device]:
+        """Validate the shards against the rank's pack plan and build the
+        launch.  Returns it with the staged copies it reads (empty in the
+        normal case: every shard is read where it lies) and the device."""
         if len(tensors) != len(infos):
             raise ValueError(
                 f"Quantized copy-in requires one tensor per ParamInfo, got {len(tensors)} tensors and {len(infos)} infos."
             )
         plan = metadata.rank_pack_plans[rank]
-        # Steady state: the same shards (sharded parameter storage is
-        # persistent) in the same layout.  The validated launch tables are
-        # reused, so a pack is one allocation and one C call.
-        if signature is None:
-            signature = self._pack_signature(tensors, infos, rank, metadata)
-        cached = self._pack_launches.get(signature)
-        if cached is not None and cached[0] is metadata:
-            payload = torch.empty(metadata.packed_send_nbytes_per_rank, dtype=torch.uint8, device=cached[2])
-            cached[1].launch(payload)
-            return payload
         device = next((t.device for t in tensors if t.numel() > 0), tensors[0].device)
         if device.type != "cuda":
             raise RuntimeError(
                 "Quantized copy-in runs on the GPU through libflexshard_hip.so; got tensors on "
                 f"{device}. This package has no CPU compute path."
             )
-        payload = torch.empty(metadata.packed_send_nbytes_per_rank, dtype=torch.uint8, device=device)
         specs: list[hip_ops.QuantChunkSpec] = []
         staged: list[torch.Tensor] = []
         qdata_cursor = 0
@@ -486,12 +569,13 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
                     f"{chunk.param_index}, got {info.fqn!r}."
                 )
             source = tensors[chunk.param_index]
+            _require_gpu_rows(source, "Quantized copy-in")
             shard = source.reshape(chunk.local_shape)
             if shard.untyped_storage().data_ptr() != source.untyped_storage().data_ptr():
                 # The shard could not be viewed as [rows, in_dim] (e.g. a strided
                 # slice of a stacked parameter), so reshape made a temporary
-                # copy.  Its address must not outlive this call in a cached
-                # launch table.
+                # copy.  Its address must not outlive this call in a stored
+                # launch.
                 staged.append(shard)
             if shard.numel() != chunk.qdata_numel:
                 raise AssertionError(
@@ -502,11 +586,12 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
                 raise NotImplementedError("the fused quantize+pack kernel handles one scale tensor per chunk")
             quant_dtype = info.unsharded_dtype
             kind = self._quantize_pack_source_kind(shard.dtype, quant_dtype)
-            if kind is None or shard.stride(-1) != 1:
-                # Unusual dtype pair or a transposed view: stage a contiguous
-                # copy in the quantization dtype (the reference stages every
-                # non-contiguous or differently typed shard this way).
-                shard = shard.to(quant_dtype).contiguous()
+            if kind is None or shard.stride(-1) != 1 or shard.is_neg():
+                # Unusual dtype pair, a transposed view or a lazily negated one:
+                # stage a contiguous copy in the quantization dtype (the
+                # reference stages every non-contiguous or differently typed
+                # shard this way).
+                shard = shard.to(quant_dtype).contiguous().resolve_neg()
                 staged.append(shard)
                 kind = self._quantize_pack_source_kind(quant_dtype, quant_dtype)
                 if kind is None:
@@ -516,13 +601,59 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
             scale_cursor += chunk.scale_numels[0] * self._scale_itemsize
         if qdata_cursor != plan.qdata_numel or scale_cursor != plan.packed_nbytes:
             raise AssertionError("Quantized pack plan sizes are inconsistent with its chunks.")
-        zero_ranges = ((plan.qdata_numel, plan.scale_byte_offset), (plan.packed_nbytes, payload.numel()))
-        launch = self._make_quantize_pack_launch(specs, payload.numel(), zero_ranges, device)
+        nbytes = metadata.packed_send_nbytes_per_rank
+        zero_ranges = ((plan.qdata_numel, plan.scale_byte_offset), (plan.packed_nbytes, nbytes))
+        return self._make_quantize_pack_launch(specs, nbytes, zero_ranges, device), staged, device
+
+    def _remember_steady_pack(
+        self,
+        launch: hip_ops.QuantPackPlan,
+        tensors: list[torch.Tensor],
+        infos: list["ParamInfo"],
+        rank: int,
+        metadata: quant_plan.QuantBucketMetadata,
+        device: torch.device,
+    ) -> "_SteadyPack":
+        layout = infos[0].bucket_layout
+        live = tuple(chunk.param_index for chunk in metadata.rank_pack_plans[rank].chunks)
+        key = (id(layout), rank)
+        group = self._steady_packs.get(key)
+        if group is None or group[0] != live or len(group[1]) >= 64:
+            group = self._steady_packs[key] = (live, {})
+        signature, _ = self._shard_signature(tensors, infos, live)
+        steady = _SteadyPack(
+            layout=layout, metadata=metadata, rank=rank, ntensors=len(tensors), infos=tuple(infos), live=live,
+            signature=signature, launch=launch, device=device, world_size=len(metadata.rank_qdata_numels),
+        )
+        group[1][tensors[live[0]].data_ptr() if live else 0] = steady
+        return steady
+
+    def _pack_local_quantized_chunks(
+        self,
+        tensors: list[torch.Tensor],
+        infos: list["ParamInfo"],
+        rank: int,
+        metadata: quant_plan.QuantBucketMetadata,
+    ) -> torch.Tensor:
+        """Quantize this rank's dense shards and pack them, in one launch, into
+        a fresh payload ``[data | pad | scales | pad]`` of the common row size."""
+        if len(tensors) != len(infos):
+            raise ValueError(
+                f"Quantized copy-in requires one tensor per ParamInfo, got {len(tensors)} tensors and {len(infos)} infos."
+            )
+        nbytes = metadata.packed_send_nbytes_per_rank
+        steady = None
+        if tensors and not torch.compiler.is_compiling():
+            steady, _, _ = self._steady_pack_for(tensors, infos, rank)
+        if steady is not None and steady.metadata is metadata:
+            payload = torch.empty(nbytes, dtype=torch.uint8, device=steady.device)
+            steady.launch.launch_raw(payload.data_ptr(), _raw_stream(steady.device_index))
+            return payload
+        launch, staged, device = self._build_pack_launch(tensors, infos, rank, metadata)
+        payload = torch.empty(nbytes, dtype=torch.uint8, device=device)
         launch.launch(payload)
-        if not staged:
-            if len(self._pack_launches) >= 64:
-                self._pack_launches.clear()
-            self._pack_launches[signature] = (metadata, launch, device)
+        if not staged and not torch.compiler.is_compiling():
+            self._remember_steady_pack(launch, tensors, infos, rank, metadata, device)
         # Staged copies were allocated and are consumed on the current stream,
         # so the caching allocator may recycle them as soon as they go out of
         # scope.
@@ -533,7 +664,9 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         self, tensors: list[torch.Tensor], infos: list["ParamInfo"], rank: int
     ) -> tuple[torch.Tensor, quant_plan.QuantBucketMetadata]:
         """Forward always packs and remembers the payload; a backward re-gather
-        may take it back once if nothing about its sources changed."""
+        may take it back once if nothing about its sources changed.  This is
+        the path of a bucket's first unshard, of shards that moved and of
+        staged shards; ``_prepare_steady`` serves every later call."""
         if len(tensors) != len(infos):
             raise ValueError(
                 f"Quantized copy-in requires one tensor per ParamInfo, got {len(tensors)} tensors and {len(infos)} infos."
@@ -541,58 +674,117 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         metadata = self._quant_metadata_from_infos(infos)
         if torch.compiler.is_compiling():
             return self._pack_local_quantized_chunks(tensors, infos, rank, metadata), metadata
-        signature = self._pack_signature(tensors, infos, rank, metadata)
-        if signature not in self._pack_launches:  # shards behind a cached launch table were checked when it was built
-            for tensor in tensors:
-                _require_gpu_rows(tensor, "Quantized copy-in")
-        device, stream = self._local_packed_cache_context(tensors)
-        prefix = (rank, id(metadata))
-        key = (*prefix, device, stream)
-        versions = tuple(t._version for t in tensors)
-        if not _is_backward_graph_task():
-            packed = self._pack_local_quantized_chunks(tensors, infos, rank, metadata, signature)
-            if len(self._local_packed_cache) > 1 or (self._local_packed_cache and key not in self._local_packed_cache):
-                for stale in [k for k in self._local_packed_cache if k[:2] == prefix]:
-                    del self._local_packed_cache[stale]
-            self._local_packed_cache[key] = self._LocalPackedCacheEntry(
-                signature=signature, versions=versions, sources=tuple(tensors), infos=tuple(infos),
-                metadata=metadata, packed=packed,
-            )
-            return packed, metadata
-        entry = self._local_packed_cache.pop(key, None)
-        if (
+        live = tuple(chunk.param_index for chunk in metadata.rank_pack_plans[rank].chunks)
+        for index in live:
+            _require_gpu_rows(tensors[index], "Quantized copy-in")
+        device = tensors[live[0]].device if live else tensors[0].device
+        stream = hip_ops.stream_ptr(device) if device.type == "cuda" else 0
+        signature, versions = self._shard_signature(tensors, infos, live)
+        key = (rank, id(metadata))
+        if _is_backward_graph_task():
+            entry = self._local_packed_cache.pop(key, None)
+            if self._cache_entry_matches(entry, metadata, signature, versions, stream, infos):
+                return entry.packed, metadata
+            return self._pack_local_quantized_chunks(tensors, infos, rank, metadata), metadata
+        packed = self._pack_local_quantized_chunks(tensors, infos, rank, metadata)
+        self._local_packed_cache[key] = _LocalPackedCacheEntry(
+            signature, versions, stream, metadata, tuple(infos), tuple(tensors), packed
+        )
+        return packed, metadata
+
+    @staticmethod
+    def _cache_entry_matches(entry, metadata, signature, versions, stream: int, infos) -> bool:
+        """A cached payload may be taken back when it was packed from the same
+        memory (signature), unchanged since (version counters), for the same
+        bucket and ParamInfo objects, on the stream the consumer is ordered
+        after."""
+        return (
             entry is not None
             and entry.metadata is metadata
+            and entry.stream == stream
             and entry.signature == signature
             and entry.versions == versions
             and len(entry.infos) == len(infos)
             and all(a is b for a, b in zip(infos, entry.infos))
-        ):
-            return entry.packed, metadata
-        return self._pack_local_quantized_chunks(tensors, infos, rank, metadata, signature), metadata
+        )
+
+    def _prepare_steady(
+        self,
+        steady: "_SteadyPack",
+        signature: list,
+        versions: list,
+        tensors: list[torch.Tensor],
+        infos: list["ParamInfo"],
+        mesh: Any,
+        debug_fqn: str | None,
+        with_gathered: bool,
+    ) -> PlacementPreparedUnshard:
+        """The steady-state unshard preparation of a bucket whose launch is
+        stored: payload and gather output from this stream's rings, one C call."""
+        stream = _raw_stream(steady.device_index)
+        rings = steady.rings.get(stream)
+        if rings is None:
+            rings = steady.rings_for(stream, self._buffer_rings)
+        cache = self._local_packed_cache
+        if _is_backward_graph_task():
+            # a backward re-gather may take the forward's payload back, once
+            entry = cache.pop(steady.cache_key, None)
+            if self._cache_entry_matches(entry, steady.metadata, signature, versions, stream, infos):
+                payload = entry.packed
+            else:
+                payload, address = rings[0].take()
+                steady.launch.launch_raw(address, stream)
+        else:
+            payload, address = rings[0].take()
+            steady.launch.launch_raw(address, stream)
+            cache[steady.cache_key] = _LocalPackedCacheEntry(
+                signature, versions, stream, steady.metadata, tuple(infos), tuple(tensors), payload
+            )
+        buffers = [payload, rings[1].take()[0]] if with_gathered else [payload]
+        return PlacementPreparedUnshard(
+            self, buffers, _QuantUnshardState(infos, mesh.get_group(), debug_fqn, steady.metadata)
+        )
+
+    def release_buffer_rings(self) -> None:
+        """Drop the recycled payload and gather buffers (they are otherwise
+        held until the placement goes away)."""
+        self._buffer_rings.clear()
+        for _, by_first_address in self._steady_packs.values():
+            for steady in by_first_address.values():
+                steady.rings.clear()
 
     # -------------------------------------------------------- unshard lifecycle
     def prepare_unshard_bucket(
         self, tensors: list[torch.Tensor], infos: list["ParamInfo"], mesh: Any, debug_fqn: str | None
     ) -> PlacementPreparedUnshard:
         """Quantize + pack the local shards and allocate the gather output."""
-        prepared = self._prepare_local_unshard_payload(tensors, infos, mesh, debug_fqn)
-        local = prepared.buffers[0]
-        prepared.buffers.append(torch.empty(mesh.size() * local.numel(), dtype=local.dtype, device=local.device))
-        return prepared
+        return self._prepare_unshard(tensors, infos, mesh, debug_fqn, True)
 
     def _prepare_local_unshard_payload(
         self, tensors: list[torch.Tensor], infos: list["ParamInfo"], mesh: Any, debug_fqn: str | None
     ) -> PlacementPreparedUnshard:
+        """The same without the gather output (a mixed bucket gathers its
+        members' payloads in one buffer of its own)."""
+        return self._prepare_unshard(tensors, infos, mesh, debug_fqn, False)
+
+    def _prepare_unshard(
+        self, tensors: list[torch.Tensor], infos: list["ParamInfo"], mesh: Any, debug_fqn: str | None, with_gathered: bool
+    ) -> PlacementPreparedUnshard:
         rank = mesh.get_local_rank()
+        profiled = torch.autograd.profiler._is_profiler_enabled
+        if tensors and len(tensors) == len(infos) and not profiled and not torch.compiler.is_compiling():
+            steady, signature, versions = self._steady_pack_for(tensors, infos, rank)
+            if steady is not None:
+                return self._prepare_steady(steady, signature, versions, tensors, infos, mesh, debug_fqn, with_gathered)
         with record_copy_in():
             local, metadata = self._cached_local_quantized_chunks(tensors, infos, rank)
+        buffers = [local]
+        if with_gathered:
+            buffers.append(torch.empty(mesh.size() * local.numel(), dtype=local.dtype, device=local.device))
         return PlacementPreparedUnshard(
             placement=self,
-            buffers=[local],
-            placement_state=BlockwiseQuantBucketedBlockShard._QuantUnshardState(
-                infos=infos, pg=mesh.get_group(), debug_fqn=debug_fqn, metadata=metadata
-            ),
+            buffers=buffers,
+            placement_state=_QuantUnshardState(infos, mesh.get_group(), debug_fqn, metadata),
         )
 
     def _unshard_state(self, prepared: PlacementPreparedUnshard) -> "_QuantUnshardState":

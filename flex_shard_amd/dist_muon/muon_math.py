@@ -211,4 +211,8 @@ class OwnedMuon:
             lerp_weight=1 - self.momentum, nesterov_weight=self.momentum, nesterov=self.nesterov,
             decay_factor=1 - self.lr * self.weight_decay, coefficients=self.ns_coefficients, steps=self.ns_steps,
             eps=self.eps,
+            # lr and adjust_lr_fn are read on every step, like the weight decay
+            # beside them: a scheduler that changes opt.lr moves both halves of
+            # the update together.
+            neg_adjusted_lrs=[-_adjust_muon_learning_rate(self.lr, self.adjust_lr_fn, shape) for shape in self._groups],
         )

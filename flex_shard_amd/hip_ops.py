@@ -31,7 +31,7 @@ from ._native import (
 __all__ = [
     "DT_BF16", "DT_F32", "EPS_FP32", "EPS_INPUT_DTYPE", "REDUCE_POSTDIV", "REDUCE_POSTMUL",
     "REDUCE_PREMUL", "REDUCE_SUM", "SRC_BF16", "SRC_F32", "SRC_F32_AS_BF16",
-    "MuonStepPlan", "QuantChunkSpec", "QuantPackPlan", "accumulate_grad", "act_quant_128x1_transposed", "act_quant_1x128",
+    "MuonStepPlan", "QuantChunkSpec", "QuantPackPlan", "accumulate_grad", "act_quant_128x1_transposed", "act_quant_1x128", "act_quant_both",
     "copy_segments", "fp8_gemm_1x128_128x1", "fp8_gemm_1x128_128x128", "fp8_gemm_1x128_128x128_dgrad",
     "fp8_transpose", "gemm_nt", "gemm_nt_group", "muon_apply", "muon_prepare", "newton_schulz_multi",
     "newton_schulz", "newton_schulz_noalloc", "newton_schulz_workspace_bytes", "pack_segments", "quantize_pack",
@@ -82,12 +82,14 @@ class QuantChunkSpec:
 
 class QuantPackPlan:
     """A validated, reusable launch of the fused quantize + pack kernel for
-    fixed source shards: the ``fsh_quant_chunk`` tables are built once, so a
-    steady-state launch is one C call.  The shards' data pointers are baked
-    into the tables: the caller launches a plan only while tensors of the same
-    shape live at those addresses (``keep_alive`` makes the plan hold them)."""
+    fixed source shards (``fsh_quant_pack_plan_*``): the chunk table, the pad
+    ranges and the launch geometry are checked and stored on the C side once,
+    so a steady-state launch is one C call with three arguments.  The shards'
+    data pointers are baked into the plan: the caller launches it only while
+    tensors of the same shape live at those addresses (``keep_alive`` makes
+    the plan hold them).  Any number of chunks."""
 
-    __slots__ = ("_tables", "_zero_ranges", "_block", "_eps_mode", "_payload_nbytes", "_device", "_keep")
+    __slots__ = ("_handle", "_payload_nbytes", "_device", "_keep", "_launch_fn", "_destroy_fn")
 
     def __init__(
         self,
@@ -99,35 +101,56 @@ class QuantPackPlan:
         device: torch.device | None = None,
         keep_alive: bool = False,
     ) -> None:
+        self._handle = None
         if chunks:
             device = _require_gpu(*[c.tensor for c in chunks])
         if device is None or device.type != "cuda":
             raise RuntimeError("flex_shard_amd kernels run on the GPU only; there is no CPU path.")
         self._device = device
         self._keep = [c.tensor for c in chunks] if keep_alive else None
-        self._zero_ranges = zero_ranges
-        self._block, self._eps_mode, self._payload_nbytes = block, eps_mode, payload_nbytes
-        cap = _native.FSH_MAX_QUANT_CHUNKS
-        groups = [list(chunks[i : i + cap]) for i in range(0, len(chunks), cap)] or [[]]
-        self._tables = []
-        for group in groups:
-            table = (_native.QuantChunk * max(len(group), 1))()
-            for slot, spec in zip(table, group):
-                t = spec.tensor
-                if t.ndim != 2 or t.stride(1) != 1 or t.shape[0] <= 0 or t.shape[1] <= 0:
-                    raise ValueError(
-                        f"chunk must be a non-empty 2-D view with unit column stride, got {tuple(t.shape)} / {t.stride()}"
-                    )
-                expected = torch.bfloat16 if spec.src_kind == SRC_BF16 else torch.float32
-                if t.dtype != expected:
-                    raise ValueError(f"chunk dtype {t.dtype} does not match src_kind {spec.src_kind}")
-                slot.src_dev = t.data_ptr()
-                slot.rows, slot.in_dim = t.shape
-                slot.src_row_stride = t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
-                slot.qdata_offset = spec.qdata_offset
-                slot.scale_offset = spec.scale_offset
-                slot.src_kind = spec.src_kind
-            self._tables.append((table, len(group)))
+        self._payload_nbytes = payload_nbytes
+        table = (_native.QuantChunk * max(len(chunks), 1))()
+        for slot, spec in zip(table, chunks):
+            t = spec.tensor
+            if t.ndim != 2 or t.stride(1) != 1 or t.shape[0] <= 0 or t.shape[1] <= 0:
+                raise ValueError(
+                    f"chunk must be a non-empty 2-D view with unit column stride, got {tuple(t.shape)} / {t.stride()}"
+                )
+            expected = torch.bfloat16 if spec.src_kind == SRC_BF16 else torch.float32
+            if t.dtype != expected:
+                raise ValueError(f"chunk dtype {t.dtype} does not match src_kind {spec.src_kind}")
+            slot.src_dev = t.data_ptr()
+            slot.rows, slot.in_dim = t.shape
+            slot.src_row_stride = t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+            slot.qdata_offset = spec.qdata_offset
+            slot.scale_offset = spec.scale_offset
+            slot.src_kind = spec.src_kind
+        lib = _native.lib()
+        self._launch_fn, self._destroy_fn = lib.fsh_quant_pack_plan_launch, lib.fsh_quant_pack_plan_destroy
+        handle = ctypes.c_void_p()
+        (z0, z1) = zero_ranges
+        status = lib.fsh_quant_pack_plan_create(
+            table, len(chunks), payload_nbytes, z0[0], z0[1], z1[0], z1[1], block, eps_mode, ctypes.byref(handle)
+        )
+        _native.check(status, "fsh_quant_pack_plan_create")
+        self._handle = handle
+
+    def __del__(self) -> None:
+        if getattr(self, "_handle", None) is not None:
+            self._destroy_fn(self._handle)
+            self._handle = None
+
+    @property
+    def payload_nbytes(self) -> int:
+        return self._payload_nbytes
+
+    def launch_raw(self, payload_ptr: int, stream: int) -> None:
+        """Queue the launch into ``payload_nbytes`` bytes at the device address
+        ``payload_ptr`` (16-byte aligned) on the raw stream handle ``stream``.
+        Nothing about the payload is checked beyond its alignment."""
+        status = self._launch_fn(self._handle, payload_ptr, stream)
+        if status != 0:
+            _native.check(status, "fsh_quant_pack_plan_launch")
 
     def launch(self, payload: torch.Tensor, stream: torch.cuda.Stream | None = None) -> None:
         """Queue the launch on ``stream`` (default: the current stream of the
@@ -137,15 +160,7 @@ class QuantPackPlan:
             raise ValueError("payload must be a 1-D uint8 tensor on the plan's device")
         if not payload.is_contiguous() or payload.numel() != self._payload_nbytes:
             raise ValueError(f"payload must be contiguous with {self._payload_nbytes} bytes")
-        fn = _native.lib().fsh_quantize_pack
-        stream = stream_ptr(self._device) if stream is None else stream.cuda_stream
-        ptr, nbytes = payload.data_ptr(), self._payload_nbytes
-        for index, (table, count) in enumerate(self._tables):
-            zr = self._zero_ranges if index == 0 else ((0, 0), (0, 0))
-            status = fn(table, count, ptr, nbytes, zr[0][0], zr[0][1], zr[1][0], zr[1][1], self._block,
-                        self._eps_mode, stream)
-            if status != 0:
-                _native.check(status, "fsh_quantize_pack")
+        self.launch_raw(payload.data_ptr(), stream_ptr(self._device) if stream is None else stream.cuda_stream)
 
 
 def quantize_pack(
@@ -739,11 +754,22 @@ class MuonStepPlan:
         self, params: Sequence[Sequence[torch.Tensor]], momenta: Sequence[Sequence[torch.Tensor]],
         grads: Sequence[Sequence[torch.Tensor]], *, lerp_weight: float, nesterov_weight: float, nesterov: bool,
         decay_factor: float, coefficients: tuple[float, float, float], steps: int, eps: float,
+        neg_adjusted_lrs: Sequence[float] | None = None, direction_scales: Sequence[float] | None = None,
     ) -> None:
         """Per group: the parameters, their momentum buffers and their
         gradients, one of each per matrix, in the same order.  All three are
         read (and the first two written) by kernels queued on the current
-        stream."""
+        stream.  ``neg_adjusted_lrs`` / ``direction_scales`` (one per group)
+        replace the step sizes and direction scales the plan was built with:
+        the C call reads them from the host table at launch time, so a
+        learning-rate schedule passes the current values on every step."""
+        for name, values in (("neg_adjusted_lr", neg_adjusted_lrs), ("direction_scale", direction_scales)):
+            if values is None:
+                continue
+            if len(values) != len(self._shapes):
+                raise ValueError(f"expected one {name} per group ({len(self._shapes)}), got {len(values)}")
+            for slot, value in zip(self._table, values):
+                setattr(slot, name, float(value))
         for name, lists in (("parameter", params), ("momentum", momenta), ("gradient", grads)):
             if len(lists) != len(self._shapes):
                 raise ValueError(f"expected {name} lists for {len(self._shapes)} groups, got {len(lists)}")

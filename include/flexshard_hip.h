@@ -87,6 +87,27 @@ int fsh_quantize_pack(const fsh_quant_chunk* chunks, int32_t nchunks, void* payl
                       int64_t zero1_begin, int64_t zero1_end, int32_t block, int32_t eps_mode,
                       void* stream);
 
+/*
+ * The same launch as a reusable plan, for a bucket whose shards stay where
+ * they are from step to step (sharded parameter storage is persistent):
+ * everything but the payload address and the stream is checked and stored
+ * once, and a steady-state pack is one call with three arguments.  Serves the
+ * per-step repetition of _pack_local_quantized_chunks
+ * (custom_placements/blockwise_quant_bucketed_block_shard.py:792-897), which
+ * the reference re-derives in Python on every unshard.  Any number of chunks:
+ * more than FSH_MAX_QUANT_CHUNKS become several launches inside one call, the
+ * first of which zeroes the pad ranges.  The plan holds the chunks' source
+ * addresses: the caller launches it only while the same memory is behind
+ * them.  A plan is host memory only (no device allocation); launches of one
+ * plan may be issued from several threads and streams at once.
+ */
+int fsh_quant_pack_plan_create(const fsh_quant_chunk* chunks, int32_t nchunks, int64_t payload_nbytes,
+                               int64_t zero0_begin, int64_t zero0_end, int64_t zero1_begin,
+                               int64_t zero1_end, int32_t block, int32_t eps_mode, void** plan_out);
+/* payload_dev: payload_nbytes bytes, 16-byte aligned. */
+int fsh_quant_pack_plan_launch(const void* plan, void* payload_dev, void* stream);
+void fsh_quant_pack_plan_destroy(void* plan);
+
 /* ------------------------------------------------------------------------
  * 2. Segment copy / zero / cast-pack.
  * Replaces the Triton kernels of custom_placements/_copy_kernels.py:

@@ -254,6 +254,130 @@ def test_payload_cache_forward_backward(device):
     assert elsewhere.buffers[0] is not forward.buffers[0] and torch.equal(elsewhere.buffers[0], forward.buffers[0])
 
 
+def test_two_buckets_in_flight_with_recycled_buffers(device):
+    """Three buckets prepared over and over with the current stream alternating
+    between two side streams, every payload read on a third stream and handed
+    back the way the runtime hands buffers back (the allocation stream waits
+    for the reader, then the references go).  Payloads and gather outputs come
+    from each stream's recycled buffers, so a buffer reused before its reader
+    ran would show up as wrong bytes: every payload must equal the oracle's."""
+    from flex_shard_amd.custom_placements import blockwise_quant_bucketed_block_shard as mod
+    from flex_shard_amd.flex_shard.bucket_comm import StreamHandoff
+
+    shapes, block, world = [(512, 256), (384, 384), (130, 136)], 128, 2
+    pl = Fp8BucketedBlockShard(world_size=world, weight_factory=_factory, block_size=block)
+    mesh = FakeMesh(world, 0)
+    lay = olayout.quant_layout(shapes, block, world)
+    buckets = []
+    for b in range(3):
+        gen = torch.Generator().manual_seed(40 + b)
+        params = [(torch.randn(s, generator=gen) * 0.02).bfloat16() for s in shapes]
+        named = [(f"w{i}", nn.Parameter(p.to(device), requires_grad=False)) for i, p in enumerate(params)]
+        infos = make_param_infos(named, pl, mesh)
+        shards = [local_rows(p, i) for (_, p), i in zip(named, infos)]
+        qs, ss = zip(*[cport.quantize_blockwise(p, block) for p in params])
+        buckets.append((shards, infos, olayout.pack_rank_payload(lay, 0, list(qs), list(ss), block)))
+    sides = [torch.cuda.Stream(device), torch.cuda.Stream(device)]
+    reader = torch.cuda.Stream(device)
+    main = torch.cuda.current_stream(device)
+    rounds = 18
+    seen = torch.empty((rounds, lay.row_nbytes), dtype=torch.uint8, device=device)
+    addresses = [set(), set()]
+    gathered_addresses = [set(), set()]
+    try:
+        for i in range(rounds):
+            shards, infos, _ = buckets[i % 3]
+            side = sides[i % 2]
+            torch.cuda.set_stream(side)
+            prepared = pl.prepare_unshard_bucket(shards, infos, mesh, None)
+            packed = torch.cuda.Event()
+            packed.record(side)
+            addresses[i % 2].add(prepared.buffers[0].data_ptr())
+            gathered_addresses[i % 2].add(prepared.buffers[1].data_ptr())
+            assert prepared.buffers[1].numel() == world * lay.row_nbytes
+            torch.cuda.set_stream(reader)
+            reader.wait_event(packed)
+            seen[i].copy_(prepared.buffers[0])
+            read = torch.cuda.Event()
+            read.record(reader)
+            StreamHandoff(list(prepared.buffers), (side,)).release_after(read)
+            prepared.buffers.clear()
+            del prepared
+    finally:
+        torch.cuda.set_stream(main)
+    torch.cuda.synchronize()
+    got = seen.cpu()
+    for i in range(rounds):
+        assert torch.equal(got[i], buckets[i % 3][2]), f"round {i} (bucket {i % 3}, stream {i % 2})"
+    # the buffers really were recycled: a handful of addresses served all rounds
+    # (the forward payload cache holds one payload per bucket, the rings the rest)
+    for side_addresses in addresses:
+        assert len(side_addresses) < rounds // 2
+    for side_addresses in gathered_addresses:
+        assert len(side_addresses) <= mod.GATHER_RING_SLOTS
+
+
+def test_recycled_payload_is_not_handed_out_while_held(device):
+    """A payload (or any view of it) that somebody still holds is never handed
+    out again; once dropped, its buffer serves the next call on that stream."""
+    pl = Fp8BucketedBlockShard(world_size=1, weight_factory=_factory, block_size=4)
+    param = nn.Parameter(torch.arange(64, dtype=torch.float32, device=device).view(8, 8))
+    (info,) = make_param_infos([("w", param)], pl, FakeMesh(1))
+    mesh = FakeMesh(1)
+    shard = param.detach()
+    pl.prepare_unshard_bucket([shard], [info], mesh, None)  # first call builds and stores the launch
+    held = [pl.prepare_unshard_bucket([shard], [info], mesh, None) for _ in range(6)]
+    assert len({p.buffers[0].data_ptr() for p in held}) == 6 and len({p.buffers[1].data_ptr() for p in held}) == 6
+    view = held[2].buffers[0][4:12]
+    alias = held[3].buffers[0].detach()
+    busy = {view.untyped_storage().data_ptr(), alias.untyped_storage().data_ptr()}
+    first = held[0].buffers[0].clone()
+    del held
+    for _ in range(8):
+        again = pl.prepare_unshard_bucket([shard], [info], mesh, None)
+        assert again.buffers[0].data_ptr() not in busy
+        assert torch.equal(again.buffers[0], first)
+        del again
+    assert torch.equal(view, first[4:12]) and torch.equal(alias, first)
+
+
+def test_staged_shard_is_read_afresh_on_every_call(device):
+    """A shard that cannot be viewed as [rows, in_dim] (a strided slice of a
+    stacked parameter) is staged through a temporary copy; the launch of such
+    a call is not stored, so the next call reads the shard as it is then and
+    never the first call's temporary."""
+    pl = Fp8BucketedBlockShard(world_size=1, weight_factory=_factory, block_size=4)
+    gen = torch.Generator().manual_seed(9)
+    big = torch.randn(2, 8, 32, generator=gen).bfloat16().to(device)
+    param = nn.Parameter(torch.empty(2, 8, 16, dtype=torch.bfloat16, device=device), requires_grad=False)
+    (info,) = make_param_infos([("experts.w", param)], pl, FakeMesh(1))
+    mesh = FakeMesh(1)
+    shard = big[:, :, :16]  # [2, 8, 16] with a row stride of 32: reshape to [16, 16] must copy
+    assert not shard.is_contiguous()
+
+    def expected():
+        oq, osc = cport.quantize_blockwise(shard.cpu().reshape(16, 16), 4)
+        return torch.cat([oq.reshape(-1), osc.reshape(-1).view(torch.uint8)])
+
+    first = pl.prepare_unshard_bucket([shard], [info], mesh, None).buffers[0]
+    assert torch.equal(first.cpu()[: 256 + 64], expected())
+    # whatever now lives where the temporary was must not be read
+    junk = [torch.full((16, 16), 7.0, dtype=torch.bfloat16, device=device) for _ in range(8)]
+    big.mul_(-3.0)
+    second = pl.prepare_unshard_bucket([shard], [info], mesh, None).buffers[0]
+    assert torch.equal(second.cpu()[: 256 + 64], expected())
+    assert not torch.equal(first.cpu(), second.cpu())
+    del junk
+    # a lazily negated shard is staged as well (the kernel reads raw bits)
+    flat = torch.randn(16, 16, generator=gen).bfloat16().to(device)
+    negated = torch._neg_view(flat).view(1, 16, 16)
+    param1 = nn.Parameter(torch.empty(1, 16, 16, dtype=torch.bfloat16, device=device), requires_grad=False)
+    (info1,) = make_param_infos([("w", param1)], pl, FakeMesh(1))
+    got = pl.prepare_unshard_bucket([negated], [info1], mesh, None).buffers[0].cpu()
+    oq, osc = cport.quantize_blockwise((-flat).cpu(), 4)
+    assert torch.equal(got[:256], oq.reshape(-1))
+
+
 def test_argument_errors(device):
     pl = Fp8BucketedBlockShard(world_size=1, weight_factory=_factory, block_size=4)
     param = nn.Parameter(torch.zeros(8, 8, device=device))
