@@ -589,6 +589,145 @@ def bench_fp8_linear_backward(device, tokens: int = 8192, reps: int = 10):
     return out
 
 
+def bench_runtime_layer_step(device, tokens: int = 8192, layers: int = 2, steps: int = 5, warmup: int = 2):
+    """The pieces composed: forward + backward of `layers` blocks of the seven
+    Llama-3-8B projections at 8192 tokens, each block one FP8 bucket of rank 0
+    of an 8-rank mesh under `BucketRuntime.install_hooks` (pack -> local
+    all-gather of the 8 payload rows -> unpack -> FP8 linears forward; again in
+    the backward, then gradient copy-in and the fixed-order 8-way reduction of
+    rank 0's range, the other ranks' rows and contributions deposited once in
+    the one-GPU group).  Each block's unshard is prefetched on a side stream
+    under the previous block's compute.  Reports the span per step, the host
+    time spent inside the runtime's hooks, and the share of the span in which
+    the host was issuing work (the rest it waits for the GPU at the end)."""
+    import torch.nn as nn
+
+    from flex_shard_amd import Fp8BucketedBlockShard, GradientReduction, LocalReduceGroup
+    from flex_shard_amd.blockwise_fp8 import convert_to_flex_shard_float8_blockwise_linear, make_blockwise_fp8_weight
+    from flex_shard_amd.flex_shard import BucketCommContext, BucketRuntime
+    from flex_shard_amd.testing import LLAMA3_8B_LAYER, FakeMesh, local_rows, make_param_infos, seeded_normal
+
+    world = 8
+
+    class Projections(nn.Module):
+        """q/k/v/o and gate/up/down of one block, joined by elementwise ops
+        (attention itself and the norms are not part of the measured path)."""
+
+        def __init__(self) -> None:
+            super().__init__()
+            for name, (out_dim, in_dim) in LLAMA3_8B_LAYER:
+                setattr(self, name, nn.Linear(in_dim, out_dim, bias=False, device="meta", dtype=torch.bfloat16))
+
+        def forward(self, x):
+            kv = torch.cat([self.k(x), self.v(x)], dim=-1)
+            h = self.o(self.q(x) + kv.repeat(1, 2))
+            return self.down(self.gate(h) * self.up(h))
+
+    context = BucketCommContext.create(device)
+    blocks, runtimes, groups = [], [], []
+    for index in range(layers):
+        block = Projections()
+        for j, (name, (out_dim, in_dim)) in enumerate(LLAMA3_8B_LAYER):
+            weight = seeded_normal((out_dim, in_dim), 0.02, 7000 + 10 * index + j, device)
+            getattr(block, name).weight = nn.Parameter(weight)
+        convert_to_flex_shard_float8_blockwise_linear(block)
+        fqns = [f"{name}.weight" for name, _ in LLAMA3_8B_LAYER]
+        named = [(fqn, block.get_parameter(fqn)) for fqn in fqns]
+        placement = Fp8BucketedBlockShard(world_size=world, weight_factory=make_blockwise_fp8_weight)
+        group = LocalReduceGroup(world, 0)
+        for other in range(1, world):  # what the other ranks would send: their quantized, packed shards
+            mesh_o = FakeMesh(world, other)
+            infos_o = make_param_infos(named, placement, mesh_o)
+            shards_o = [local_rows(p, i) for (_, p), i in zip(named, infos_o)]
+            group.gather_rows[other] = placement.prepare_unshard_bucket(shards_o, infos_o, mesh_o, None).buffers[0]
+        runtime = BucketRuntime.shard_module_params(
+            block, fqns, placement, FakeMesh(world, 0, group), context, GradientReduction()
+        )
+        del named
+        blocks.append(block)
+        runtimes.append(runtime)
+        groups.append(group)
+    model = nn.Sequential(*blocks)
+    for index, (block, runtime) in enumerate(zip(blocks, runtimes)):
+        runtime.install_hooks(
+            block,
+            forward_prefetch=runtimes[index + 1] if index + 1 < layers else None,
+            backward_prefetch=runtimes[index - 1] if index > 0 else None,
+        )
+    torch.cuda.empty_cache()
+
+    # host time inside the runtime's entry points, by name
+    host_us: dict[str, float] = {}
+    calls: dict[str, int] = {}
+
+    def timed(obj, name):
+        inner = getattr(obj, name)
+
+        def wrapper(*args, **kwargs):
+            t0 = time.perf_counter()
+            try:
+                return inner(*args, **kwargs)
+            finally:
+                host_us[name] = host_us.get(name, 0.0) + (time.perf_counter() - t0) * 1e6
+                calls[name] = calls.get(name, 0) + 1
+
+        setattr(obj, name, wrapper)
+
+    for runtime in runtimes:
+        for name in ("unshard", "prefetch", "reshard", "reduce_grads"):
+            timed(runtime, name)
+
+    x = seeded_normal((tokens, 4096), 1.0, 7900, device).requires_grad_()
+    grad_out = seeded_normal((tokens, 4096), 0.01, 7901, device)
+
+    # The other ranks' reduce-scatter inputs: one [world, world x widest rank range] fp32 tensor
+    # shared by the blocks' groups; row 0 is written by every reduction's copy-in.
+    widest = max(runtimes[0].infos[0].bucket_layout.rank_numels)
+    contributions = torch.empty((world, world * widest), dtype=torch.float32, device=device)
+    contributions[1:].normal_(0.0, 1e-3)
+    for group in groups:
+        group.contributions = contributions
+
+    def step():
+        for group in groups:
+            group.mark_deposited(*range(1, world))
+        x.grad = None
+        for runtime in runtimes:
+            for p in runtime.sharded_params:
+                p.grad = None
+        model(x).backward(grad_out)
+        context.wait_and_clear_reduce_grad_states()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    host_us.clear()
+    calls.clear()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        step()
+    t_issued = time.perf_counter()
+    stop.record()
+    torch.cuda.synchronize()
+    t_done = time.perf_counter()
+    span_ms = start.elapsed_time(stop) / steps
+    flop = 3 * 2 * tokens * sum(o * i for _, (o, i) in LLAMA3_8B_LAYER) * layers
+    return {
+        "workload": f"{layers} blocks of the seven Llama-3-8B projections, {tokens} tokens, forward + backward, rank 0 of "
+        f"{world} (LocalReduceGroup), Fp8BucketedBlockShard under BucketRuntime.install_hooks with prefetch, "
+        "fp32 gradient reduction",
+        "span_ms_per_step": round(span_ms, 3),
+        "host_issue_ms_per_step": round((t_issued - t0) * 1e3 / steps, 3),
+        "host_issue_share_of_span": round((t_issued - t0) / max(t_done - t0, 1e-9), 3),
+        "gemm_flop_per_step": flop,
+        "gemm_TFLOPs_over_span": round(flop / span_ms / 1e9, 1),
+        "host_us_per_call_in_runtime_entry": {k: round(v / calls[k], 1) for k, v in sorted(host_us.items())},
+        "runtime_entry_calls_per_step": {k: v // steps for k, v in sorted(calls.items())},
+    }
+
+
 def calibrate_copy(device, nbytes: int = 256 << 20, reps: int = 4) -> None:
     """A plain copy of known size through copy_segments_kernel: reads `nbytes`
     and writes `nbytes` per launch."""
@@ -615,7 +754,7 @@ def main() -> None:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB -> 256 MiB segment copy, the known-size kernel that the "
                     "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
-    ap.add_argument("--only", choices=("muon", "fp8_linear"),
+    ap.add_argument("--only", choices=("muon", "fp8_linear", "runtime_layer_step"),
                     help="profiling aid: run only this secondary section (for counter runs, which slow "
                     "every kernel down) and print its figures instead of the benchmark line")
     args = ap.parse_args()
@@ -634,6 +773,9 @@ def main() -> None:
 
     if args.only == "muon":
         print(json.dumps({"muon_newton_schulz": bench_muon(device)}))
+        return
+    if args.only == "runtime_layer_step":
+        print(json.dumps({"runtime_layer_step": bench_runtime_layer_step(device)}))
         return
     if args.only == "fp8_linear":
         print(json.dumps({"fp8_linear_forward_8192_tokens": bench_fp8_linear(device),
@@ -743,6 +885,8 @@ def main() -> None:
         secondary["fp8_linear_backward_8192_tokens"] = {
             name: {k: round(v, 4) for k, v in d.items()} for name, d in bench_fp8_linear_backward(device).items()
         }
+        torch.cuda.empty_cache()
+        secondary["runtime_layer_step"] = bench_runtime_layer_step(device)
         result["secondary"] = secondary
     print(json.dumps(result))
 

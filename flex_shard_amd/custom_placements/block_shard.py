@@ -31,6 +31,7 @@ from ..placement_contract import (
     PlacementReduceGradResult,
     PlacementUnshardResult,
 )
+from .. import hip_ops
 from ..profiling import record_comm, record_copy_in, record_copy_out, record_range
 from ._copy_kernels import SegmentCopyDescriptor, SegmentPackDescriptor, copy_segments, pack_segments_into_flat_buffer
 from .utils import (
@@ -475,7 +476,12 @@ class BucketedBlockShard(Placement):
             if short_by > 0:
                 send = nn.functional.pad(send, (0, short_by))
             return send, scratch
-        key = (local.numel(), widest, local.device)
+        # One descriptor per source range and stream: its device table holds
+        # the source address and is refreshed by a copy queued on the current
+        # stream, so equally sized buckets (the layers of a model) or two
+        # streams sharing one table could overwrite it before the other's
+        # launch has read it.
+        key = (local.data_ptr(), local.numel(), widest, local.device, hip_ops.stream_ptr(local.device))
         descriptor = self._send_row_descriptors.get(key)
         if descriptor is None:
             pad = [(-1, 0, short_by, local.numel())] if short_by > 0 else []
@@ -488,7 +494,7 @@ class BucketedBlockShard(Placement):
                 dst_offsets=[seg[3] for seg in segments],
                 device=local.device,
             )
-            if len(self._send_row_descriptors) >= 16:
+            if len(self._send_row_descriptors) >= 256:
                 self._send_row_descriptors.clear()
             self._send_row_descriptors[key] = descriptor
         row = torch.empty(max(widest, local.numel()), dtype=dtype, device=local.device)

@@ -176,11 +176,16 @@ class LocalReduceGroup:
     ``rank``'s segment of the fixed-order sum over rows 0..W-1.
     """
 
-    def __init__(self, world_size: int, rank: int) -> None:
+    def __init__(self, world_size: int, rank: int, *, local_row_only: bool = False) -> None:
+        """``local_row_only``: the all-gather writes this rank's row and leaves
+        the other rows of the output as they are (no ``gather_rows`` needed).
+        For timing the local steps of an unshard; the output is then not a
+        gathered layout that can be unpacked."""
         if not 0 <= rank < world_size:
             raise ValueError(f"rank must be in [0, {world_size}), got {rank}")
         self._world_size = world_size
         self._rank = rank
+        self.local_row_only = local_row_only
         self.contributions: torch.Tensor | None = None
         self.deposited: set[int] = set()
         #: all-gather rows of the other ranks, by rank (see ``all_gather_rows``)
@@ -230,10 +235,13 @@ def all_gather_rows(output: torch.Tensor, input: torch.Tensor, group: Any, *, as
         world, rank = group.size(), group.rank()
         if output.numel() != world * input.numel():
             raise ValueError(f"all-gather output has {output.numel()} elements, expected {world} x {input.numel()}")
+        rows = output.view(world, input.numel())
+        if group.local_row_only:
+            rows[rank].copy_(input.reshape(-1))
+            return None
         missing = sorted(set(range(world)) - {rank} - set(group.gather_rows))
         if missing:
             raise ValueError(f"LocalReduceGroup is missing the all-gather rows of ranks {missing}.")
-        rows = output.view(world, input.numel())
         rows[rank].copy_(input.reshape(-1))
         for other, row in group.gather_rows.items():
             if other != rank:

@@ -39,6 +39,23 @@ if TYPE_CHECKING:
     from ..placement_contract import GradientReduction, Placement
 
 
+_STREAM_OBJECTS: dict[tuple[int, int, int], torch.cuda.Stream] = {}
+
+
+def _current_stream(device: torch.device | None) -> torch.cuda.Stream:
+    """``torch.cuda.current_stream(device)`` without building a new Stream
+    object per call: the objects are kept by (stream id, device index, device
+    type), which is what identifies a stream to torch."""
+    index = torch.cuda.current_device() if device is None or device.index is None else device.index
+    key = torch._C._cuda_getCurrentStream(index)
+    stream = _STREAM_OBJECTS.get(key)
+    if stream is None:
+        if len(_STREAM_OBJECTS) >= 64:
+            _STREAM_OBJECTS.clear()
+        stream = _STREAM_OBJECTS[key] = torch.cuda.Stream(stream_id=key[0], device_index=key[1], device_type=key[2])
+    return stream
+
+
 class _Fence:
     """A point in one stream's queue that other streams can be ordered after."""
 
@@ -53,6 +70,9 @@ class _Fence:
 
     def hold_back(self, *streams: torch.cuda.Stream) -> None:
         """Order each distinct stream of ``streams`` after this point."""
+        if len(streams) == 1:
+            streams[0].wait_event(self.event)
+            return
         done: set[int] = set()
         for stream in streams:
             if stream.cuda_stream not in done:
@@ -60,16 +80,31 @@ class _Fence:
                 stream.wait_event(self.event)
 
 
-@contextlib.contextmanager
-def _on_side_stream(side: torch.cuda.Stream, device: torch.device):
+class _on_side_stream:
     """Run the block on ``side`` after everything the current stream has
-    queued so far.  Yields a one-element list that holds the fence of the
-    block's end once the block has run."""
-    _Fence(torch.cuda.current_stream(device)).hold_back(side)
-    done: list[_Fence] = []
-    with torch.cuda.stream(side):
-        yield done
-        done.append(_Fence(side))
+    queued so far.  ``with _on_side_stream(side, device) as done``: ``done`` is
+    a list that holds the fence of the block's end once the block has run.
+    The current stream is switched with ``torch.cuda.set_stream`` (a fraction
+    of what the ``torch.cuda.stream`` context costs) and always restored."""
+
+    __slots__ = ("_side", "_previous", "_done")
+
+    def __init__(self, side: torch.cuda.Stream, device: torch.device) -> None:
+        self._side = side
+        self._previous = _current_stream(device)
+        self._done: list[_Fence] = []
+
+    def __enter__(self) -> list[_Fence]:
+        _Fence(self._previous).hold_back(self._side)
+        torch.cuda.set_stream(self._side)
+        return self._done
+
+    def __exit__(self, exc_type, exc, tb) -> None:
+        try:
+            if exc_type is None:
+                self._done.append(_Fence(self._side))
+        finally:
+            torch.cuda.set_stream(self._previous)
 
 
 class StreamHandoff:
@@ -97,7 +132,7 @@ class StreamHandoff:
         if self._tensors is None:
             return
         if self._tensors:
-            _Fence(torch.cuda.current_stream(self._tensors[0].device)).hold_back(*self._allocation_streams)
+            _Fence(_current_stream(self._tensors[0].device)).hold_back(*self._allocation_streams)
             self._tensors.clear()
         self._tensors = None
 
@@ -131,11 +166,12 @@ def _prepare_and_run(
     prepared = placement.prepare_unshard_bucket(tensors, infos, mesh, debug_fqn)
     prepared.persistent = True
     prepared.persistent_buffers = persistent_buffers
+    if persistent_buffers is None:
+        return prepared, placement.run_prepared_unshard(prepared, async_op=async_op)
     with contextlib.ExitStack() as guards:
-        if persistent_buffers is not None:
-            guards.enter_context(torch.inference_mode(False))
-            guards.enter_context(torch.no_grad())
-            guards.enter_context(torch.autograd._unsafe_preserve_version_counter(tuple(persistent_buffers)))
+        guards.enter_context(torch.inference_mode(False))
+        guards.enter_context(torch.no_grad())
+        guards.enter_context(torch.autograd._unsafe_preserve_version_counter(tuple(persistent_buffers)))
         work = placement.run_prepared_unshard(prepared, async_op=async_op)
     return prepared, work
 
@@ -170,7 +206,7 @@ class UnshardHandle:
             self._work.wait()
             self._work = None
         if self._fence is not None and self._device is not None:
-            torch.cuda.current_stream(self._device).wait_event(self._fence.event)
+            _current_stream(self._device).wait_event(self._fence.event)
 
     def finish(self) -> PlacementUnshardResult:
         """Copy out on the current stream and hand the temporaries back to the
@@ -198,7 +234,7 @@ class UnshardHandle:
         # Buffers of a side stream were last read by the copy-out just queued
         # on the current stream.
         if tensors and self._side_stream is not None:
-            current = torch.cuda.current_stream(tensors[0].device)
+            current = _current_stream(tensors[0].device)
             StreamHandoff(tensors, (self._side_stream, current)).release_after_current_stream()
 
 
@@ -275,7 +311,7 @@ class ReduceGradHandle:
         """Order the current stream after the reduction."""
         device = self._device()
         if device is not None and self._fence is not None:
-            torch.cuda.current_stream(device).wait_event(self._fence.event)
+            _current_stream(device).wait_event(self._fence.event)
 
     def finish(self) -> list[torch.Tensor]:
         self.wait()
@@ -318,7 +354,7 @@ def begin_reduce_grad(
     placement = _get_bucket_placement(infos, "reduce-grad")
     prepared = placement.prepare_reduce_grad(tensors, infos, mesh, debug_fqn)
     device = prepared.buffers[0].device
-    copy_in_stream = torch.cuda.current_stream(device)
+    copy_in_stream = _current_stream(device)
     with _on_side_stream(reduce_grad_stream, device) as done:
         result = placement.reduce_prepared_grad(prepared, reduction)
     return ReduceGradHandle(

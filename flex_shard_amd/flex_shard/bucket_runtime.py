@@ -86,26 +86,48 @@ class PendingReduceGrad:
 
 @dataclass
 class BucketCommContext:
-    """Streams and in-flight reductions shared by the buckets of one model."""
+    """Streams and in-flight reductions shared by the buckets of one model.
+
+    ``unshard_streams``: the side streams unshards are begun on, taken in turn
+    (``next_unshard_stream``).  With two of them, a prefetched bucket's
+    quantize + pack launch overlaps the ramp and drain of the previous
+    bucket's (an 82 MB launch alone spends a fifth of its time there); all
+    streams have the default priority."""
 
     device: torch.device
-    unshard_stream: torch.cuda.Stream
+    unshard_streams: list[torch.cuda.Stream]
     reduce_grad_stream: torch.cuda.Stream
     reduce_grad_release_stream: torch.cuda.Stream
     max_pending_reduce_grads: int = 2
     reduce_grad_states: list[PendingReduceGrad] = field(default_factory=list)
     retired_reduce_grad_states: list[PendingReduceGrad] = field(default_factory=list)
+    _unshard_turn: int = 0
 
     @classmethod
-    def create(cls, device: torch.device, max_pending_reduce_grads: int = 2) -> "BucketCommContext":
+    def create(
+        cls, device: torch.device, max_pending_reduce_grads: int = 2, unshard_streams: int = 2
+    ) -> "BucketCommContext":
+        if unshard_streams < 1:
+            raise ValueError(f"a context needs at least one unshard stream, got {unshard_streams}")
         # default priorities only
         return cls(
             device=device,
-            unshard_stream=torch.cuda.Stream(device),
+            unshard_streams=[torch.cuda.Stream(device) for _ in range(unshard_streams)],
             reduce_grad_stream=torch.cuda.Stream(device),
             reduce_grad_release_stream=torch.cuda.Stream(device),
             max_pending_reduce_grads=max_pending_reduce_grads,
         )
+
+    @property
+    def unshard_stream(self) -> torch.cuda.Stream:
+        """The first unshard stream (the only one of a one-stream context)."""
+        return self.unshard_streams[0]
+
+    def next_unshard_stream(self) -> torch.cuda.Stream:
+        """The side stream for the next unshard: the streams take turns."""
+        stream = self.unshard_streams[self._unshard_turn % len(self.unshard_streams)]
+        self._unshard_turn += 1
+        return stream
 
     def wait_and_release_reduce_grad_state(self, pending: PendingReduceGrad, *, wait_current_stream: bool) -> None:
         if wait_current_stream:
@@ -157,6 +179,8 @@ class BucketRuntime:
         debug_fqn: str | None = None,
     ) -> None:
         self.bucket_params = bucket_params
+        self._infos = [bp.info for bp in bucket_params]
+        self._sharded_params = [bp.sharded_param for bp in bucket_params]
         self.mesh = mesh
         self.context = context
         self.gradient_reduction = gradient_reduction
@@ -213,14 +237,14 @@ class BucketRuntime:
 
     @property
     def infos(self) -> list[ParamInfo]:
-        return [bp.info for bp in self.bucket_params]
+        return self._infos
 
     @property
     def sharded_params(self) -> list[nn.Parameter]:
-        return [bp.sharded_param for bp in self.bucket_params]
+        return self._sharded_params
 
     def _local_shards(self) -> list[torch.Tensor]:
-        return [p.detach() for p in self.sharded_params]
+        return [p.detach() for p in self._sharded_params]
 
     # ---------------------------------------------------------------- unshard
     def begin_unshard(self, *, on_current_stream: bool = False, async_op: bool = False) -> UnshardHandle:
@@ -235,7 +259,8 @@ class BucketRuntime:
                 self._alloc_persistent_storage()
             persistent_buffers = self.persistent_buffers
         return begin_bucket_unshard(
-            self._local_shards(), self.infos, self.mesh, None if on_current_stream else self.context.unshard_stream,
+            self._local_shards(), self.infos, self.mesh,
+            None if on_current_stream else self.context.next_unshard_stream(),
             debug_fqn=self.debug_fqn, persistent_buffers=persistent_buffers, async_op=async_op and on_current_stream,
         )
 
@@ -376,21 +401,39 @@ class BucketRuntime:
             self.context.reduce_grad_states.append(PendingReduceGrad(result))
 
     # ------------------------------------------------------------------- hooks
-    def install_hooks(self, module: nn.Module) -> None:
+    def install_hooks(
+        self,
+        module: nn.Module,
+        *,
+        forward_prefetch: "BucketRuntime | None" = None,
+        backward_prefetch: "BucketRuntime | None" = None,
+    ) -> None:
         """Unshard before ``module``'s forward, reshard after it, unshard again
         when its backward starts, and reduce + reshard once every parameter of
-        the bucket has its gradient (one use of each parameter per forward)."""
+        the bucket has its gradient (one use of each parameter per forward).
+        ``forward_prefetch`` / ``backward_prefetch``: the bucket used next in
+        the forward / in the backward; its unshard is begun on a side stream as
+        soon as this bucket's own is finished, so that its quantize + pack and
+        exchange run under this module's compute (the explicit form of the
+        reference's prefetch order, bucket_runtime.py:300-396)."""
 
         def pre_forward(mod: nn.Module, args: Any) -> None:
             self.unshard()
             self._grads_seen = 0
+            if forward_prefetch is not None:
+                forward_prefetch.prefetch()
+
+        def pre_backward(_grads: Any) -> None:
+            self.unshard()
+            if backward_prefetch is not None:
+                backward_prefetch.prefetch()
 
         def post_forward(mod: nn.Module, args: Any, output: Any) -> Any:
             self.reshard()
             tensors = [t for t in (output if isinstance(output, (tuple, list)) else (output,))
                        if isinstance(t, torch.Tensor) and t.requires_grad]
             if tensors:
-                torch.autograd.graph.register_multi_grad_hook(tensors, lambda _g: self.unshard(), mode="any")
+                torch.autograd.graph.register_multi_grad_hook(tensors, pre_backward, mode="any")
             return output
 
         self._hook_handles.append(module.register_forward_pre_hook(pre_forward))
