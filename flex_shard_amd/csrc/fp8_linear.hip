@@ -119,7 +119,7 @@ struct Fp8GemmCfg {
   static constexpr int kScaleStageBytes = kWaves * kScaleSlots * 4;
   static constexpr int kScaleOffset = kStages * kStageBytes;
   static constexpr int kWeightScaleOffset = kScaleOffset + kStages * kScaleStageBytes;  // [wave][256] block scales
-  static constexpr int kMaxKTilesInLds = 256;
+  static constexpr int kMaxKTilesInLds = 256;  // window of weight block scales kept in LDS per wave (a power of two)
   static constexpr int kLdsBytes = max_int(kWeightScaleOffset + kWaves * kMaxKTilesInLds * 4, kWaves * kRegion);
   static_assert(kWaveM <= kScaleSlots, "one 4-byte scale request per lane covers the wave's rows");
 };
@@ -162,7 +162,11 @@ __device__ __forceinline__ void fold_with_row_broadcast(f32x16& acc, const f32x1
 }
 
 // One output tile (TM_ = 2) or half tile (TM_ = 1, rows [128 half, +128) of the tile).
-template <bool kColumnScales, int TM_>
+// kLongK: the contraction is longer than one window of weight block scales
+// (kMaxKTilesInLds k-tiles); the block-scale variant then refills the window
+// inside the loop.  A separate instantiation: the refill's few instructions
+// cost the loop 12 % of its rate, which the usual lengths should not pay.
+template <bool kColumnScales, int TM_, bool kLongK>
 __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams& p, uint8_t* lds_bytes, int tm, int tn, int half) {
   using Cfg = Fp8GemmCfg<TM_>;
   static_assert(Cfg::kStages == 2, "the loop below alternates between two stages");
@@ -289,9 +293,30 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams& p, uint8_t* l
   // inside the loop would again wait for the prefetched tile).
   issue_k_tile(0, 0);
   float* ws_lds = reinterpret_cast<float*>(lds_bytes + Cfg::kWeightScaleOffset + wave * Cfg::kMaxKTilesInLds * 4);
+  // ws_lds holds the scales of k-tiles [window, window + kMaxKTilesInLds).
+  // For a contraction of at most one window they are copied once, under the
+  // first k-tile's requests.  A longer one (kLongK) refills the window when
+  // the loop reaches its last k-tile, and then the scales travel global -> LDS
+  // like everything else the loop reads (four 4-byte-per-lane requests per
+  // window): a load the compiler sees inside the loop makes it wait for all
+  // memory traffic in flight on every iteration (measured: 20 % slower).
+  const uint32_t ws_lds_addr = lds_base + static_cast<uint32_t>(Cfg::kWeightScaleOffset + wave * Cfg::kMaxKTilesInLds * 4);
+  auto issue_weight_scale_window = [&](int64_t first_kt) {
+    const uint8_t* ws_row = reinterpret_cast<const uint8_t*>(p.ws + wblock * p.ws_cb);
+#pragma unroll
+    for (int q = 0; q < Cfg::kMaxKTilesInLds / 64; ++q) {
+      int64_t kt_of_lane = first_kt + q * 64 + lane;
+      kt_of_lane = kt_of_lane < ktiles ? kt_of_lane : ktiles - 1;  // past the end: any valid entry, never read
+      dma_touch_4(static_cast<uint32_t>(kt_of_lane * p.ws_kb * 4), ws_row, ws_lds_addr + q * 256);
+    }
+  };
   if (!kColumnScales) {
-    const float* ws_row = p.ws + wblock * p.ws_cb;
-    for (int64_t i = lane; i < ktiles; i += 64) ws_lds[i] = ws_row[i * p.ws_kb];  // ktiles <= kMaxKTilesInLds (host check)
+    if (kLongK) {
+      issue_weight_scale_window(0);
+    } else {
+      const float* ws_row = p.ws + wblock * p.ws_cb;
+      for (int64_t i = lane; i < ktiles; i += 64) ws_lds[i] = ws_row[i * p.ws_kb];  // ktiles <= kMaxKTilesInLds (host)
+    }
   }
   wait_for_dma_loads();
   __syncthreads();
@@ -325,7 +350,7 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams& p, uint8_t* l
       dst[i] = *reinterpret_cast<const float*>(lds_bytes + Cfg::kScaleOffset + stage * Cfg::kScaleStageBytes +
                                                (wave * Cfg::kScaleSlots + i * 32 + frag_row) * 4);
     if (!kColumnScales) {
-      const float ws_now = ws_lds[kt];
+      const float ws_now = ws_lds[kLongK ? (kt & (Cfg::kMaxKTilesInLds - 1)) : kt];
 #pragma unroll
       for (int i = 0; i < TM; ++i) dst[i] *= ws_now;
     }
@@ -359,6 +384,13 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams& p, uint8_t* l
     // The scales are first needed by the fold behind the second block's MFMAs.
     read_row_scales(s, stage, kt);
     read_column_scales(cs_rows, stage);
+    if (kLongK && !kColumnScales && more && (kt & (Cfg::kMaxKTilesInLds - 1)) == Cfg::kMaxKTilesInLds - 1) {
+      // Last k-tile of the window (once per 32 768 of k): its scale has just
+      // been read; the next window is requested over it and lands before this
+      // k-tile's hand-over barrier, like the operands of k-tile kt + 1.
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      issue_weight_scale_window(kt + 1);
+    }
     // Fragments are read in the order the blocks need them: the other A row
     // blocks under the MFMAs of the first column block (they stay for the
     // whole k-tile), each further B column block while the previous one is
@@ -516,14 +548,14 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams& p, uint8_t* l
 // kColumnScales = false: the second operand carries one scale per 128 x 128
 // tile (a prequantized weight, either orientation).  true: one scale per
 // output column and k-block (an operand quantized in 128 x 1 runs).
-template <bool kColumnScales>
+template <bool kColumnScales, bool kLongK = false>
 __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(const Fp8GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds_bytes[];
   int64_t unused_batch;
   int tm, tn;
   if (static_cast<int64_t>(blockIdx.x) < p.whole_grid) {
     if (!tile_of_workgroup(p.schedule, blockIdx.x, &unused_batch, &tm, &tn)) return;  // whole workgroup
-    fp8_gemm_tile<kColumnScales, 2>(p, lds_bytes, uniform_i32(tm), uniform_i32(tn), 0);
+    fp8_gemm_tile<kColumnScales, 2, kLongK>(p, lds_bytes, uniform_i32(tm), uniform_i32(tn), 0);
   } else {
     // Same split over the XCDs as the whole tiles: the two halves of a tile are
     // neighbours in an XCD's run and share the tile's second operand in its L2.
@@ -531,7 +563,8 @@ __global__ __launch_bounds__(Fp8Gemm::kThreads) void fp8_gemm_blockwise_kernel(c
     const int64_t item = (id % kXcds) * p.half_items_per_xcd + id / kXcds;
     if (item >= p.half_items) return;
     tile_in_order(p.schedule, static_cast<int>(p.schedule.work_items + item / 2), &tm, &tn);
-    fp8_gemm_tile<kColumnScales, 1>(p, lds_bytes, uniform_i32(tm), uniform_i32(tn), uniform_i32(static_cast<int>(item & 1)));
+    fp8_gemm_tile<kColumnScales, 1, kLongK>(p, lds_bytes, uniform_i32(tm), uniform_i32(tn),
+                                            uniform_i32(static_cast<int>(item & 1)));
   }
 }
 
@@ -587,11 +620,9 @@ int launch_fp8_gemm(Fp8GemmParams& p, bool column_scales, const char* who, void*
   if (!p.xq || !p.xs || !p.wq || !p.out || (column_scales ? !p.cs : !p.ws)) return fail(FSH_EINVAL, "%s: null pointer", who);
   if (p.k == 0 || p.k % 128)
     return fail(FSH_ENOTSUP, "%s: k must be a positive multiple of 128 (pad the operands), got %lld", who, (long long)p.k);
-  // Only the block-scale variant keeps one weight scale per k-tile in LDS; the
-  // column-scale variant contracts over tokens and takes any length.
-  if (!column_scales && p.k / 128 > Fp8Gemm::kMaxKTilesInLds)
-    return fail(FSH_ENOTSUP, "%s: k must be at most %d, got %lld", who, 128 * Fp8Gemm::kMaxKTilesInLds, (long long)p.k);
   if (p.k >= (1LL << 31)) return fail(FSH_ENOTSUP, "%s: k must be below 2^31, got %lld", who, (long long)p.k);
+  if (!column_scales && (p.k / 128) * p.ws_kb * 4 >= (1LL << 31))
+    return fail(FSH_ENOTSUP, "%s: a row of the weight scale table spans more than 2 GiB", who);
   if (p.ldxq < p.k || p.ldwq < p.k || p.ldo < p.n)
     return fail(FSH_EINVAL, "%s: a leading dimension is smaller than its row", who);
   if (p.ldxq % 16 || p.ldwq % 16 || !aligned(p.xq, 16) || !aligned(p.wq, 16) || !aligned(p.out, 2))
@@ -621,14 +652,22 @@ int launch_fp8_gemm(Fp8GemmParams& p, bool column_scales, const char* who, void*
   p.whole_grid = s.items_per_xcd * kXcds;
   p.half_items = 2 * cut;
   p.half_items_per_xcd = ceil_div(p.half_items, static_cast<int64_t>(kXcds));
-  static LdsReservation reserved_block_scales, reserved_column_scales;
+  // The block-scale variant keeps one window of weight scales in LDS; a longer
+  // contraction takes the instantiation that refills it.
+  const bool long_k = !column_scales && p.k / 128 > Fp8Gemm::kMaxKTilesInLds;
+  static LdsReservation reserved_block_scales, reserved_block_scales_long, reserved_column_scales;
   if (int rc = column_scales
                    ? reserve_lds_once(reserved_column_scales, &fp8_gemm_blockwise_kernel<true>, Fp8Gemm::kLdsBytes)
+               : long_k
+                   ? reserve_lds_once(reserved_block_scales_long, &fp8_gemm_blockwise_kernel<false, true>, Fp8Gemm::kLdsBytes)
                    : reserve_lds_once(reserved_block_scales, &fp8_gemm_blockwise_kernel<false>, Fp8Gemm::kLdsBytes))
     return rc;
   const dim3 grid(static_cast<uint32_t>(p.whole_grid + p.half_items_per_xcd * kXcds)), block(Fp8Gemm::kThreads);
   if (column_scales)
     hipLaunchKernelGGL(fp8_gemm_blockwise_kernel<true>, grid, block, Fp8Gemm::kLdsBytes, static_cast<hipStream_t>(stream), p);
+  else if (long_k)
+    hipLaunchKernelGGL((fp8_gemm_blockwise_kernel<false, true>), grid, block, Fp8Gemm::kLdsBytes,
+                       static_cast<hipStream_t>(stream), p);
   else
     hipLaunchKernelGGL(fp8_gemm_blockwise_kernel<false>, grid, block, Fp8Gemm::kLdsBytes, static_cast<hipStream_t>(stream), p);
   return check_launch("fp8_gemm_blockwise_kernel");

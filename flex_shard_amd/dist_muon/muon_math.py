@@ -169,23 +169,30 @@ class OwnedMuon:
         # Matrices of one shape are orthogonalized as one batch; the step's
         # launch tables (address tables, batch buffers, workspaces) are built once.
         self._groups: dict[tuple[int, int], list[int]] = {}
+        # Matrices whose rows or columns are not multiples of 8 (the batched
+        # step's 16-byte rows) take the per-matrix kernels, padded inside
+        # the orthogonalization.
+        self._odd: list[int] = []
         for index, p in enumerate(self.params):
-            self._groups.setdefault(tuple(p.shape), []).append(index)
-        self._plan = hip_ops.MuonStepPlan(
-            [
-                # whole parameters are their own learning-rate reference shape: direction scale 1
-                (shape, len(members), -_adjust_muon_learning_rate(lr, adjust_lr_fn, shape), 1.0)
-                for shape, members in self._groups.items()
-            ],
-            self.params[0].device,
-        )
-        self._batch = dict(zip(self._groups, self._plan.batches))
-        self._workspace = dict(zip(self._groups, self._plan.workspaces))
+            if p.shape[0] % 8 or p.shape[1] % 8:
+                self._odd.append(index)
+            else:
+                self._groups.setdefault(tuple(p.shape), []).append(index)
+        self._plan = None
+        if self._groups:
+            self._plan = hip_ops.MuonStepPlan(
+                [
+                    # whole parameters are their own learning-rate reference shape: direction scale 1
+                    (shape, len(members), -_adjust_muon_learning_rate(lr, adjust_lr_fn, shape), 1.0)
+                    for shape, members in self._groups.items()
+                ],
+                self.params[0].device,
+            )
+            self._batch = dict(zip(self._groups, self._plan.batches))
+            self._workspace = dict(zip(self._groups, self._plan.workspaces))
 
     def flops_per_step(self) -> int:
-        return 2 * sum(
-            _estimate_muon_compute_cost((len(members), *shape), self.ns_steps) for shape, members in self._groups.items()
-        )
+        return 2 * sum(_estimate_muon_compute_cost(tuple(p.shape), self.ns_steps) for p in self.params)
 
     @torch.no_grad()
     def step(self, grads: Sequence[torch.Tensor | None]) -> None:
@@ -203,6 +210,18 @@ class OwnedMuon:
         # Newton-Schulz with every product issued for all groups together, and
         # an update launch per group.  Same bits as _prepare_muon_input ->
         # _compute_muon_direction -> _apply_muon_update per matrix.
+        for index in self._odd:
+            p, g = self.params[index], grads[index]
+            direction = _prepare_muon_input(
+                g, self.momentum_buffers[index], momentum=self.momentum, nesterov=self.nesterov, out=torch.empty_like(p)
+            )
+            _compute_muon_direction(direction, ns_coefficients=self.ns_coefficients, ns_steps=self.ns_steps, eps=self.eps)
+            _apply_muon_update(
+                p, direction, lr=self.lr, weight_decay=self.weight_decay, adjust_lr_fn=self.adjust_lr_fn,
+                compute_matrix_shape=p.shape,
+            )
+        if self._plan is None:
+            return
         members = list(self._groups.values())
         self._plan.step(
             [[self.params[i] for i in group] for group in members],

@@ -301,7 +301,9 @@ def reduce_rows(
 
 
 def newton_schulz_workspace_bytes(batch: int, rows: int, cols: int) -> int:
-    return int(_native.lib().fsh_newton_schulz_workspace_bytes(batch, rows, cols))
+    """Workspace of ``newton_schulz`` for ``batch`` matrices; rows and columns
+    count as rounded up to multiples of 8, which is how they are processed."""
+    return int(_native.lib().fsh_newton_schulz_workspace_bytes(batch, -(-rows // 8) * 8, -(-cols // 8) * 8))
 
 
 def newton_schulz(
@@ -318,6 +320,18 @@ def newton_schulz(
         raise ValueError("x must be a contiguous bf16 matrix or batch of matrices")
     batch = 1 if x.ndim == 2 else x.shape[0]
     rows, cols = x.shape[-2:]
+    if (rows % 8 or cols % 8) and x.numel():
+        # The kernels move 16-byte rows.  Zero rows and columns change nothing:
+        # the Frobenius norm is the same, X X^T and the polynomial keep them
+        # zero in every iteration, and the other entries see the same products.
+        padded = x.new_zeros((batch, -(-rows // 8) * 8, -(-cols // 8) * 8))
+        padded[:, :rows, :cols] = x.view(batch, rows, cols)
+        need = newton_schulz_workspace_bytes(batch, padded.shape[1], padded.shape[2])
+        if workspace is not None and (workspace.dtype != torch.uint8 or workspace.numel() < need):
+            workspace = None  # sized for the unpadded shape
+        newton_schulz(padded, coefficients, steps, eps, workspace)
+        x.view(batch, rows, cols).copy_(padded[:, :rows, :cols])
+        return x
     need = newton_schulz_workspace_bytes(batch, rows, cols)
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=x.device)

@@ -134,19 +134,32 @@ def test_forward_of_the_prequantized_linear(device):
 
 
 def test_gemm_rejects_what_the_kernel_cannot_take(device):
-    """k that is not a multiple of 128, and a contraction longer than the
-    block-scale variant keeps weight scales for (32 768), fail with a message
-    instead of launching."""
+    """k that is not a multiple of 128 fails with a message instead of launching."""
     xq = torch.zeros((8, 192), dtype=torch.uint8, device=device)
     xs = torch.ones((1, 8), dtype=torch.float32, device=device)
     wq = torch.zeros((8, 192), dtype=torch.uint8, device=device)
     ws = torch.ones((1, 1), dtype=torch.float32, device=device)
     with pytest.raises(RuntimeError, match="multiple of 128"):
         hip_ops.fp8_gemm_1x128_128x128(xq, xs, wq, ws)
-    k = 32768 + 128
-    xq = torch.zeros((8, k), dtype=torch.uint8, device=device)
-    xs = torch.ones((k // 128, 8), dtype=torch.float32, device=device)
-    wq = torch.zeros((8, k), dtype=torch.uint8, device=device)
-    ws = torch.ones((1, k // 128), dtype=torch.float32, device=device)
-    with pytest.raises(RuntimeError, match="at most 32768"):
-        hip_ops.fp8_gemm_1x128_128x128(xq, xs, wq, ws)
+
+
+def test_contraction_longer_than_one_window_of_weight_scales(device):
+    """The block-scale variant keeps 256 k-tiles of weight scales in LDS and
+    refills the window when the loop crosses it: k = 2 windows + 3 k-tiles,
+    every weight scale different, against the oracle's product; forward and
+    input-gradient (scale table read across) forms."""
+    gen = torch.Generator().manual_seed(5)
+    m, n, k = 96, 384, 2 * 32768 + 384
+    x = torch.randn(m, k, generator=gen).bfloat16()
+    w = (torch.randn(n, k, generator=gen) * 0.02).bfloat16()
+    xq, xs = eager.act_quant_1x128(x)
+    wq, ws = eager.quantize_blockwise(w, 128)
+    ws = ws * (1.0 + torch.arange(ws.numel(), dtype=torch.float32).view(ws.shape) / ws.numel())  # no two alike
+    want = eager.fp8_gemm_1x128_128x128(xq, xs, wq, ws, out_dtype=torch.float32)
+    got = hip_ops.fp8_gemm_1x128_128x128(xq.to(device), xs.to(device), wq.to(device), ws.to(device))
+    assert torch.allclose(got.cpu().float(), want, rtol=2.0**-7, atol=1e-3 * want.abs().max().item())
+    # the same product as an input gradient: operand w as [k, n]^T with the table [k / 128, n / 128] read across
+    got_t = hip_ops.fp8_gemm_1x128_128x128_dgrad(
+        xq.to(device), xs.to(device), wq.to(device), ws.t().contiguous().to(device), in_dim=n
+    )
+    assert torch.equal(got_t, got)

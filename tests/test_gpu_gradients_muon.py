@@ -5,6 +5,7 @@ import pytest
 import torch
 import torch.nn as nn
 
+from flex_shard_amd import _native  # noqa: E402
 from flex_shard_amd import (
     BucketedBlockShard,
     Fp8BucketedBlockShard,
@@ -420,8 +421,13 @@ def test_newton_schulz_leaves_its_input_untouched_and_handles_zero(device):
     assert torch.equal(g, keep)
     z = _zeropower_via_newtonschulz(torch.zeros(64, 128, device=device, dtype=torch.bfloat16))
     assert (z == 0).all()
-    with pytest.raises(RuntimeError, match="multiples of 8"):
-        _zeropower_via_newtonschulz(torch.randn(12, 20, device=device).bfloat16())
+    # the C entry itself works on 16-byte rows (the Python wrapper pads other shapes)
+    odd = torch.randn(1, 12, 20, device=device).bfloat16()
+    work = torch.empty(hip_ops.newton_schulz_workspace_bytes(1, 12, 20), dtype=torch.uint8, device=device)
+    status = _native.lib().fsh_newton_schulz(
+        odd.data_ptr(), 1, 12, 20, *COEFFS, 5, 1e-7, work.data_ptr(), work.numel(), hip_ops.stream_ptr(device)
+    )
+    assert status != 0 and b"multiples of 8" in _native.lib().fsh_last_error()
 
 
 def test_gemm_building_block(device):
@@ -829,3 +835,88 @@ def test_fused_muon_step_equals_the_per_matrix_kernels(device, nesterov):
             assert torch.equal(opt.momentum_buffers[i], momenta[i]), f"momentum {i} differs at step {step}"
             assert torch.equal(mine[i], theirs[i]), f"parameter {i} differs at step {step}"
     assert not torch.equal(mine[0], start[0])
+
+
+# ------------------------------------- shapes that are not multiples of 8, schedules, scaled directions
+@pytest.mark.parametrize("shape", [(100, 36), (33, 77), (130, 64), (2, 21, 50), (7, 7)])
+def test_newton_schulz_takes_any_shape(device, shape, golden):
+    """Rows or columns that are not multiples of 8 are zero-padded inside the
+    wrapper (zero rows and columns stay zero through the iteration and leave
+    the norm unchanged); against torch's own routine, the reference's bar."""
+    from torch.optim._muon import _zeropower_via_newtonschulz as torch_ns
+
+    tol = golden["muon_tolerance"]["atol"]
+    gen = torch.Generator().manual_seed(12)
+    g = torch.randn(shape, generator=gen).bfloat16()
+    on_gpu = g.to(device)
+    mine = _zeropower_via_newtonschulz(on_gpu).cpu()
+    assert mine.shape == g.shape and torch.equal(on_gpu.cpu(), g)  # the input is left as it was
+    ref = torch.stack([torch_ns(m, COEFFS, 5, 1e-7) for m in g.clone().view(-1, *shape[-2:])]).view(shape)
+    assert (mine.float() - ref.float()).abs().max().item() <= tol
+
+
+def test_owned_muon_with_odd_shapes_and_a_learning_rate_schedule(device, golden):
+    """Matrices the batched step cannot take (rows or columns not multiples of
+    8) go through the per-matrix kernels beside the batched groups, and a
+    learning rate changed between steps moves the step size and the weight
+    decay together: three steps against torch.optim.Muon under the same
+    schedule."""
+    tol = golden["muon_tolerance"]["atol"]
+    gen = torch.Generator().manual_seed(21)
+    shapes = [(256, 128), (100, 36), (128, 128), (33, 77), (256, 128)]
+    start = [(torch.randn(s, generator=gen) * 0.02).bfloat16() for s in shapes]
+    mine = [p.clone().to(device) for p in start]
+    theirs = [nn.Parameter(p.clone()) for p in start]
+    opt_mine = OwnedMuon(mine, lr=1e-3)
+    opt_theirs = torch.optim.Muon(theirs, lr=1e-3, weight_decay=0.1, momentum=0.95, nesterov=True)
+    for lr in (1e-3, 5e-2, 2e-4):
+        opt_mine.lr = lr
+        for group in opt_theirs.param_groups:
+            group["lr"] = lr
+        grads = [torch.randn(s, generator=gen).bfloat16() for s in shapes]
+        opt_mine.step([g.to(device) for g in grads])
+        for p, g in zip(theirs, grads):
+            p.grad = g.clone()
+        opt_theirs.step()
+    for a, b, p0 in zip(mine, theirs, start):
+        assert (a.cpu().float() - b.detach().float()).abs().max().item() <= tol
+        assert torch.allclose(a.cpu().float(), b.detach().float(), atol=4e-3)
+        # the 5e-2 step moved every entry by about lr x sqrt(rows/cols) x |direction|: a frozen step size would not
+        assert (a.cpu().float() - p0.float()).abs().mean().item() > 1e-3
+
+
+def test_muon_step_plan_with_scaled_directions_equals_the_per_matrix_kernels(device):
+    """A direction scale other than 1 (a matrix whose learning-rate factor
+    differs from its reference shape's): the update in the last product's
+    epilogue (large-tile group) and the batched update kernel (small group)
+    must give the bits of prepare -> Newton-Schulz -> apply(direction_scale)."""
+    groups = [((1024, 1280), 20, -3e-3, 0.75), ((64, 96), 2, -1.5e-3, 1.5)]
+    plan = hip_ops.MuonStepPlan(groups, device)
+    params, momenta, grads, ref_params, ref_momenta = [], [], [], [], []
+    for gi, (shape, n, _, _) in enumerate(groups):
+        params.append([seeded_normal(shape, 0.02, 900 + 50 * gi + i, device) for i in range(n)])
+        momenta.append([seeded_normal(shape, 0.5, 1900 + 50 * gi + i, device) for i in range(n)])
+        grads.append([seeded_normal(shape, 1.0, 2900 + 50 * gi + i, device) for i in range(n)])
+        ref_params.append([p.clone() for p in params[-1]])
+        ref_momenta.append([m.clone() for m in momenta[-1]])
+    decay = 1 - 2e-3 * 0.05
+    plan.step(params, momenta, grads, lerp_weight=0.05, nesterov_weight=0.95, nesterov=True, decay_factor=decay,
+              coefficients=COEFFS, steps=5, eps=1e-7)
+    batches = [torch.empty((n, *shape), dtype=torch.bfloat16, device=device) for shape, n, _, _ in groups]
+    for gi, (shape, n, _, _) in enumerate(groups):
+        for i in range(n):
+            _prepare_muon_input(grads[gi][i], ref_momenta[gi][i], momentum=0.95, nesterov=True, out=batches[gi][i])
+    hip_ops.newton_schulz_multi([(b, None) for b in batches], COEFFS, 5, 1e-7)
+    for gi, (shape, n, neg_lr, scale) in enumerate(groups):
+        for i in range(n):
+            hip_ops.muon_apply(ref_params[gi][i], batches[gi][i], decay_factor=decay, neg_adjusted_lr=neg_lr,
+                               direction_scale=scale)
+            assert torch.equal(momenta[gi][i], ref_momenta[gi][i]), f"momentum {gi}/{i}"
+            assert torch.equal(params[gi][i], ref_params[gi][i]), f"parameter {gi}/{i}"
+    # the per-step override replaces what the plan was built with
+    plan.step(params, momenta, grads, lerp_weight=0.05, nesterov_weight=0.95, nesterov=True, decay_factor=decay,
+              coefficients=COEFFS, steps=5, eps=1e-7, neg_adjusted_lrs=[0.0, 0.0], direction_scales=[1.0, 1.0])
+    for gi in range(len(groups)):
+        for i in range(groups[gi][1]):
+            want = (ref_params[gi][i].float() * decay).bfloat16()
+            assert torch.equal(params[gi][i], want), f"zero step size {gi}/{i}"

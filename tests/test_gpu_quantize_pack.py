@@ -472,3 +472,44 @@ def test_deepseek_expert_bucket_edge_tiles(device):
         saw_zero_tile |= bool((_bits(osc) == zero_scale_bits).any())
     assert saw_zero_tile
     assert (scales[0].view(torch.int32) == zero_scale_bits).all()
+
+
+def test_deepseek_rank_inside_w2_and_llama_down_against_the_oracle(device):
+    """Shares other than rank 0's at full size, on sampled 128-row bands
+    against the C oracle: rank 3 of the DeepSeek-V3 expert bucket (its whole
+    share lies in w2, in_dim 2048, rows of several experts) and rank 7 of the
+    Llama bucket (rows of `down`, in_dim 14336)."""
+    gen = torch.Generator().manual_seed(17)
+    for spec, std, rank, fqn, seed in (
+        (DEEPSEEK_V3_EXPERTS, 0.006, 3, "experts.w2", 310),
+        (LLAMA3_8B_LAYER, 0.02, 7, "down", 110),
+    ):
+        named = seeded_bucket(spec, std, seed, device)
+        if spec is DEEPSEEK_V3_EXPERTS:
+            for i, (_, p) in enumerate(named):
+                add_outliers_and_zero_tiles(p, 410 + i)
+        pl = Fp8BucketedBlockShard(world_size=8, weight_factory=_factory)
+        mesh = FakeMesh(8, rank)
+        infos = make_param_infos(named, pl, mesh)
+        live = [i for i in infos if i.local_numel]
+        assert [i.fqn for i in live] == [fqn], [i.fqn for i in live]
+        shards = [local_rows(p, i) for (_, p), i in zip(named, infos)]
+        prepared = pl.prepare_unshard_bucket(shards, infos, mesh, None)
+        md = prepared.placement_state.metadata
+        payload = prepared.buffers[0]
+        index = [i.fqn for i in infos].index(fqn)
+        shard = shards[index].flatten(0, -2)
+        rows, in_dim = shard.shape
+        assert rows * in_dim == md.rank_qdata_numels[rank] and rows % 128 == 0
+        tiles_c = in_dim // 128
+        s0 = md.rank_scale_byte_offsets[rank]
+        scales = payload[s0 : s0 + 4 * md.rank_scale_numels[rank]].view(torch.float32).view(rows // 128, tiles_c)
+        bands = sorted({0, rows // 128 - 1, *torch.randint(0, rows // 128, (10,), generator=gen).tolist()})
+        for band in bands:
+            oq, osc = cport.quantize_blockwise(shard[band * 128 : (band + 1) * 128].cpu(), 128)
+            got = payload[band * 128 * in_dim : (band + 1) * 128 * in_dim].view(128, in_dim).cpu()
+            assert torch.equal(got, oq), f"{fqn} band {band}"
+            assert torch.equal(_bits(scales[band].cpu()), _bits(osc.view(-1))), f"{fqn} band {band}"
+        assert (payload[md.rank_qdata_numels[rank] : s0] == 0).all()
+        del named, shards, prepared, payload
+        torch.cuda.empty_cache()

@@ -318,6 +318,17 @@ def test_llama_gathered_layout_unpack_full_size(device, golden):
         amax = p.detach().float().view(tiles_r, 128, tiles_c, 128).abs().amax(dim=(1, 3))
         bound = (amax / 16 * 1.01).repeat_interleave(128, 0).repeat_interleave(128, 1)
         assert ((deq.float() - p.detach().float()).abs() <= bound).all(), fqn
+    # anchor the widest parameter (`down`, in_dim 14336) against the CPU oracle on sampled 128-row bands
+    down = named[6][1].detach()
+    gen = torch.Generator().manual_seed(3)
+    for band in sorted({0, 31, *torch.randint(0, 32, (4,), generator=gen).tolist()}):
+        rows_cpu = down[band * 128 : (band + 1) * 128].cpu()
+        oq, osc = cport.quantize_blockwise(rows_cpu, 128)
+        got = result.full_params[6].view(torch.uint8)[band * 128 : (band + 1) * 128].cpu()
+        assert torch.equal(got, oq), f"down band {band}"
+        assert torch.equal(factory.calls[6][1][band].cpu().view(torch.int32), osc.view(-1).view(torch.int32))
+        want = cport.dequant_blockwise(oq, osc, 128)
+        assert torch.equal(dequant[6][band * 128 : (band + 1) * 128].cpu().view(torch.int16), want.view(torch.int16))
     # anchor one gathered parameter against the CPU oracle
     k = named[1][1].detach().cpu()
     oq, osc = cport.quantize_blockwise(k, 128)
