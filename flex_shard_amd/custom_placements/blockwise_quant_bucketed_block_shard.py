@@ -118,11 +118,12 @@ def _require_gpu_rows(tensor: torch.Tensor, what: str) -> None:
 
 
 _getrefcount = sys.getrefcount
+_profiler = torch.autograd.profiler
 _storage_use_count = torch._C._storage_Use_Count
 _raw_stream = torch._C._cuda_getCurrentRawStream
 
 PAYLOAD_RING_SLOTS = 4
-GATHER_RING_SLOTS = 2
+GATHER_RING_SLOTS = 3
 
 
 class _QuantUnshardState:
@@ -134,19 +135,15 @@ class _QuantUnshardState:
         self.infos, self.pg, self.debug_fqn, self.metadata = infos, pg, debug_fqn, metadata
 
 
-class _LocalPackedCacheEntry:
-    """A forward pack a backward re-gather may take once.  ``signature`` names
-    the sources (address, dtype, shape, strides, negative bit, quantization
-    dtype of every shard that holds rows), ``versions`` their version counters
-    at pack time and ``stream`` the raw stream the pack was queued on;
-    ``sources`` keeps the shards' storage alive, so that an equal address still
-    means the same memory, and ``infos`` pins the ParamInfo objects by identity."""
-
-    __slots__ = ("signature", "versions", "stream", "metadata", "infos", "sources", "packed")
-
-    def __init__(self, signature, versions, stream, metadata, infos, sources, packed) -> None:
-        self.signature, self.versions, self.stream, self.metadata = signature, versions, stream, metadata
-        self.infos, self.sources, self.packed = infos, sources, packed
+# A forward pack that a backward re-gather may take once is remembered as a
+# plain tuple (the cheapest object to build on every forward unshard):
+#   (signature, versions, stream, metadata, infos, sources, packed)
+# signature: address, dtype, shape, strides, negative bit and quantization
+# dtype of every shard that holds rows; versions: their version counters at
+# pack time; stream: the raw stream the pack was queued on; sources keeps the
+# shards' storage alive, so that an equal address still means the same memory;
+# infos pins the ParamInfo objects by identity.
+_E_SIGNATURE, _E_VERSIONS, _E_STREAM, _E_METADATA, _E_INFOS, _E_SOURCES, _E_PACKED = range(7)
 
 
 class _BufferRing:
@@ -164,26 +161,42 @@ class _BufferRing:
     buffers and a caller that keeps payloads (the backward cache does, one per
     bucket) simply gets fresh ones."""
 
-    __slots__ = ("nbytes", "device", "capacity", "_slots")
+    __slots__ = ("nbytes", "device", "capacity", "_slots", "_next")
 
     def __init__(self, nbytes: int, device: torch.device, capacity: int) -> None:
         self.nbytes, self.device, self.capacity = nbytes, device, capacity
         self._slots: list[list] = []
+        self._next = 0
 
     def take(self) -> tuple[torch.Tensor, int]:
         """A free buffer and its device address."""
-        for slot in self._slots:
+        # The slot behind the one handed out last: with buffers released in the
+        # order they were taken, it is the one released longest ago.
+        slots = self._slots
+        index = self._next
+        if index < len(slots):
+            slot = slots[index]
             if _getrefcount(slot[0]) == slot[3] and slot[0]._use_count() == 1 and _storage_use_count(slot[2]) == slot[4]:
+                self._next = index + 1 if index + 1 < len(slots) else 0
+                return slot[0], slot[1]
+        return self._take_any()
+
+    def _take_any(self) -> tuple[torch.Tensor, int]:
+        slots = self._slots
+        for index, slot in enumerate(slots):
+            if _getrefcount(slot[0]) == slot[3] and slot[0]._use_count() == 1 and _storage_use_count(slot[2]) == slot[4]:
+                self._next = index + 1 if index + 1 < len(slots) else 0
                 return slot[0], slot[1]
         tensor = torch.empty(self.nbytes, dtype=torch.uint8, device=self.device)
         address = tensor.data_ptr()
-        if len(self._slots) < self.capacity:
+        if len(slots) < self.capacity:
             storage = tensor.untyped_storage()
             slot = [tensor, address, storage._cdata, 0, 0, storage]
             # the counts of a free slot: what they read now, minus this frame's own reference
             slot[3] = _getrefcount(slot[0]) - 1
             slot[4] = _storage_use_count(slot[2])
-            self._slots.append(slot)
+            slots.append(slot)
+            self._next = 0
         return tensor, address
 
 
@@ -194,7 +207,7 @@ class _SteadyPack:
 
     __slots__ = (
         "layout", "metadata", "rank", "ntensors", "infos", "live", "signature", "launch", "device", "device_index",
-        "cache_key", "payload_nbytes", "gathered_nbytes", "rings",
+        "cache_key", "payload_nbytes", "gathered_nbytes", "rings", "launch_fn", "launch_handle",
     )
 
     def __init__(self, *, layout, metadata, rank, ntensors, infos, live, signature, launch, device, world_size) -> None:
@@ -202,6 +215,7 @@ class _SteadyPack:
         self.infos, self.live, self.signature, self.launch, self.device = infos, live, signature, launch, device
         self.device_index = torch.cuda.current_device() if device.index is None else device.index
         self.cache_key = (rank, id(metadata))
+        self.launch_fn, self.launch_handle = launch.raw_launch()
         self.payload_nbytes = metadata.packed_send_nbytes_per_rank
         self.gathered_nbytes = world_size * self.payload_nbytes
         self.rings: dict[int, tuple[_BufferRing, _BufferRing]] = {}
@@ -515,7 +529,8 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         signature, versions = [], []
         for index in live:
             t = tensors[index]
-            signature.append((t.data_ptr(), t.dtype, t.shape, t.stride(), t.is_neg(), infos[index].unsharded_dtype))
+            info = infos[index]  # param_dtype or dtype: ParamInfo.unsharded_dtype, read without the property call
+            signature.append((t.data_ptr(), t.dtype, t.shape, t.stride(), t.is_neg(), info.param_dtype or info.dtype))
             versions.append(t._version)
         return signature, versions
 
@@ -532,10 +547,16 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         steady = by_first_address.get(tensors[live[0]].data_ptr() if live else 0)
         if steady is None or steady.layout is not infos[0].bucket_layout or len(tensors) != steady.ntensors:
             return None, None, None
+        # (the loop of _shard_signature, with the identity check of the infos folded in)
+        steady_infos = steady.infos
+        signature, versions = [], []
         for index in live:
-            if infos[index] is not steady.infos[index]:
+            info = infos[index]
+            if info is not steady_infos[index]:
                 return None, None, None
-        signature, versions = self._shard_signature(tensors, infos, live)
+            t = tensors[index]
+            signature.append((t.data_ptr(), t.dtype, t.shape, t.stride(), t.is_neg(), info.param_dtype or info.dtype))
+            versions.append(t._version)
         if signature != steady.signature:
             return None, None, None
         return steady, signature, versions
@@ -684,12 +705,10 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         if _is_backward_graph_task():
             entry = self._local_packed_cache.pop(key, None)
             if self._cache_entry_matches(entry, metadata, signature, versions, stream, infos):
-                return entry.packed, metadata
+                return entry[_E_PACKED], metadata
             return self._pack_local_quantized_chunks(tensors, infos, rank, metadata), metadata
         packed = self._pack_local_quantized_chunks(tensors, infos, rank, metadata)
-        self._local_packed_cache[key] = _LocalPackedCacheEntry(
-            signature, versions, stream, metadata, tuple(infos), tuple(tensors), packed
-        )
+        self._local_packed_cache[key] = (signature, versions, stream, metadata, tuple(infos), tuple(tensors), packed)
         return packed, metadata
 
     @staticmethod
@@ -700,12 +719,12 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         after."""
         return (
             entry is not None
-            and entry.metadata is metadata
-            and entry.stream == stream
-            and entry.signature == signature
-            and entry.versions == versions
-            and len(entry.infos) == len(infos)
-            and all(a is b for a, b in zip(infos, entry.infos))
+            and entry[_E_METADATA] is metadata
+            and entry[_E_STREAM] == stream
+            and entry[_E_SIGNATURE] == signature
+            and entry[_E_VERSIONS] == versions
+            and len(entry[_E_INFOS]) == len(infos)
+            and all(a is b for a, b in zip(infos, entry[_E_INFOS]))
         )
 
     def _prepare_steady(
@@ -730,16 +749,16 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
             # a backward re-gather may take the forward's payload back, once
             entry = cache.pop(steady.cache_key, None)
             if self._cache_entry_matches(entry, steady.metadata, signature, versions, stream, infos):
-                payload = entry.packed
+                payload = entry[_E_PACKED]
             else:
                 payload, address = rings[0].take()
                 steady.launch.launch_raw(address, stream)
         else:
             payload, address = rings[0].take()
-            steady.launch.launch_raw(address, stream)
-            cache[steady.cache_key] = _LocalPackedCacheEntry(
-                signature, versions, stream, steady.metadata, tuple(infos), tuple(tensors), payload
-            )
+            status = steady.launch_fn(steady.launch_handle, address, stream)
+            if status != 0:
+                steady.launch.launch_raw(address, stream)  # raises with the library's message
+            cache[steady.cache_key] = (signature, versions, stream, steady.metadata, tuple(infos), tuple(tensors), payload)
         buffers = [payload, rings[1].take()[0]] if with_gathered else [payload]
         return PlacementPreparedUnshard(
             self, buffers, _QuantUnshardState(infos, mesh.get_group(), debug_fqn, steady.metadata)
@@ -771,8 +790,7 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         self, tensors: list[torch.Tensor], infos: list["ParamInfo"], mesh: Any, debug_fqn: str | None, with_gathered: bool
     ) -> PlacementPreparedUnshard:
         rank = mesh.get_local_rank()
-        profiled = torch.autograd.profiler._is_profiler_enabled
-        if tensors and len(tensors) == len(infos) and not profiled and not torch.compiler.is_compiling():
+        if tensors and len(tensors) == len(infos) and not _profiler._is_profiler_enabled and not torch.compiler.is_compiling():
             steady, signature, versions = self._steady_pack_for(tensors, infos, rank)
             if steady is not None:
                 return self._prepare_steady(steady, signature, versions, tensors, infos, mesh, debug_fqn, with_gathered)

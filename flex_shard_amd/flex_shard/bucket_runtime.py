@@ -9,7 +9,7 @@ Mirror of the reference's ``flex_shard/bucket_runtime.py``: ``begin_unshard``
 persistent storage (:951-980), ``_accumulate_sharded_grads`` (:1686-1724) and
 the reduce-grad bookkeeping of ``BucketCommContext`` (:524-576).  What is not
 here: prefetch ordering, module-tree hook discovery, activation-checkpoint
-recompute, deferred gradient upcasts, ``torch.compile`` capture and the storage
+recompute, ``torch.compile`` capture and the storage
 engine -- a bucket is built from an explicit list of parameters of one module,
 and one pair of hooks (``install_hooks``) covers one forward and one backward
 per step.
@@ -194,6 +194,10 @@ class BucketRuntime:
         self._grads_seen = 0
         self._reduce_when_grads_arrive = False
         self._pending_unshard: UnshardHandle | None = None
+        #: False: backwards keep their full-parameter gradients (microbatch
+        #: accumulation); the next backward with this set reduces them.
+        self.requires_gradient_sync = True
+        self.needs_sync = False
 
     # ------------------------------------------------------------ construction
     @classmethod
@@ -400,6 +404,43 @@ class BucketRuntime:
                 result.record_sharded_grads(_accumulate_sharded_grads(sharded_params, sharded_grads), stream)
             self.context.reduce_grad_states.append(PendingReduceGrad(result))
 
+    def set_requires_gradient_sync(self, requires_gradient_sync: bool) -> None:
+        """Whether a backward reduces this bucket's gradients (the last
+        microbatch) or only accumulates them on the unsharded parameters."""
+        self.requires_gradient_sync = requires_gradient_sync
+
+    def _set_unsharded_grad_dtypes(self, *, defer_upcast: bool) -> None:
+        """Defer or restore the upcast of gradients that accumulate in a wider
+        dtype than the parameter computes in (reference:
+        ``_set_unsharded_grad_dtypes``, bucket_runtime.py:1062-1108).
+
+        Deferred (``grad_dtype = None``), in a backward that reduces or that
+        adds to a kept gradient, autograd leaves the gradients in the compute
+        dtype: the reduce-scatter copy-in widens them as it copies (one cast
+        launch per parameter less, and half the bytes read by the copy-in) and
+        AccumulateGrad adds them in place to a wider kept gradient.  A backward
+        without sync that starts a gradient keeps the upcast, so that the sum
+        over microbatches is taken in the wider dtype.  Restoring upcasts a new
+        gradient that was not reduced, once."""
+        for bp, param in zip(self.bucket_params, self.unsharded_params or [], strict=False):
+            dtype, compute_dtype = bp.info.unsharded_grad_dtype, bp.info.unsharded_dtype
+            if (
+                dtype is None
+                or not param.requires_grad
+                or not dtype.is_floating_point
+                or not compute_dtype.is_floating_point
+                or dtype.itemsize <= compute_dtype.itemsize
+            ):
+                continue
+            if defer_upcast:
+                if param.grad is not None or self.requires_gradient_sync:
+                    param.grad_dtype = None
+                continue
+            grad = param.grad
+            if grad is not None and grad.dtype != dtype:
+                param.grad = grad.to(dtype)
+            param.grad_dtype = dtype
+
     # ------------------------------------------------------------------- hooks
     def install_hooks(
         self,
@@ -425,6 +466,7 @@ class BucketRuntime:
 
         def pre_backward(_grads: Any) -> None:
             self.unshard()
+            self._set_unsharded_grad_dtypes(defer_upcast=True)
             if backward_prefetch is not None:
                 backward_prefetch.prefetch()
 
@@ -446,8 +488,16 @@ class BucketRuntime:
         self._grads_seen += 1
         expected = sum(1 for p in self.unsharded_params if p.requires_grad)
         if self._grads_seen == expected:
-            self.reduce_grads()
-            self.reshard()
+            if self.requires_gradient_sync:
+                self.needs_sync = False
+                self.reduce_grads()  # takes the gradients; the copy-in casts them to the reduce dtype
+                self._set_unsharded_grad_dtypes(defer_upcast=False)
+                self.reshard()
+            else:
+                self.needs_sync = True
+                self.reshard()
+                # after the reshard, so that a deferred gradient's upcast never coexists with the full parameters
+                self._set_unsharded_grad_dtypes(defer_upcast=False)
 
     def _register_grad_hooks(self) -> None:
         for param in self.unsharded_params:

@@ -144,6 +144,12 @@ class QuantPackPlan:
     def payload_nbytes(self) -> int:
         return self._payload_nbytes
 
+    def raw_launch(self) -> tuple[object, object]:
+        """``(function, handle)``: ``function(handle, payload_ptr, stream)`` is
+        the C call of :meth:`launch_raw` (status 0 on success) for callers that
+        count microseconds; the plan must outlive every such call."""
+        return self._launch_fn, self._handle
+
     def launch_raw(self, payload_ptr: int, stream: int) -> None:
         """Queue the launch into ``payload_nbytes`` bytes at the device address
         ``payload_ptr`` (16-byte aligned) on the raw stream handle ``stream``.

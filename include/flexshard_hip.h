@@ -395,6 +395,12 @@ int fsh_fp8_gemm_1x128_128x1(const void* aq_dev, const float* as_dev, const void
  * batch_dev is scratch of batch*rows*cols bf16: it holds the momentum
  * output and, for groups updated by a separate launch, the orthogonalized
  * direction afterwards (its contents after the call are otherwise unspecified).
+ * Errors: the argument checks (list, groups, sizes, workspaces) come before
+ * any launch.  A failure after them (a launch the runtime rejects, a product
+ * the GEMM planner cannot place, an LDS reservation refused) leaves the step
+ * half done: the momentum buffers have been advanced, no parameter, or only
+ * some, updated.  Treat it as fatal for the optimizer state; do not retry
+ * the step.
  * ---------------------------------------------------------------------- */
 typedef struct fsh_muon_group {
   const int64_t* param_ptrs_dev;    /* [batch] addresses of the parameters, updated in place   */

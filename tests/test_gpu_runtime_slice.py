@@ -358,3 +358,54 @@ def test_checkpoint_layouts_of_sharded_buckets(device):
         copy_full_into_shard(tensor, saved[name], get_global_layout(tensor))
     assert all(torch.equal(p.view(full[name].shape), full[name]) for name, p in model.named_parameters())
     torch.cuda.synchronize()
+
+
+def test_microbatches_without_sync_accumulate_in_fp32_and_the_upcast_is_deferred(device):
+    """Two microbatches: the first backward runs without gradient sync and
+    keeps its full-parameter gradients upcast to fp32; the second one syncs,
+    its bf16 gradients are added in place to the kept fp32 ones (no separate
+    cast), and the reduction's copy-in reads them.  A single syncing backward
+    hands autograd's bf16 gradients straight to the copy-in.  Both against the
+    kernels called directly."""
+    gen = torch.Generator().manual_seed(5)
+    model = _mlp(device, gen)
+    full = [p.detach().clone() for p in model.parameters()]
+    convert_to_flex_shard_float8_blockwise_linear(model)
+    mesh = FakeMesh(1, 0, LocalReduceGroup(1, 0))
+    placement = Fp8BucketedBlockShard(world_size=1, weight_factory=make_blockwise_fp8_weight)
+    context = BucketCommContext.create(device)
+    runtime = BucketRuntime.shard_module_params(model, ["0.weight", "1.weight"], placement, mesh, context)
+    runtime.install_hooks(model)
+    xs = [torch.randn(64, 256, generator=gen).bfloat16().to(device) for _ in range(2)]
+    gos = [(torch.randn(64, 256, generator=gen) * 0.01).bfloat16().to(device) for _ in range(2)]
+    wants = [_direct(full, x, go)[2] for x, go in zip(xs, gos)]
+
+    seen_dtypes = []
+    runtime.set_requires_gradient_sync(False)
+    model(xs[0]).backward(gos[0])
+    assert runtime.needs_sync and not runtime.is_unsharded
+    kept = [p.grad for p in runtime.unsharded_params]
+    assert all(g.dtype == torch.float32 for g in kept)  # a backward that starts a gradient keeps the upcast
+    assert all(torch.equal(g, w.float()) for g, w in zip(kept, wants[0]))
+    runtime.set_requires_gradient_sync(True)
+    for p in runtime.unsharded_params:
+        p.register_hook(lambda g: seen_dtypes.append(g.dtype))
+    model(xs[1]).backward(gos[1])
+    context.wait_and_clear_reduce_grad_states()
+    assert seen_dtypes and all(d == torch.bfloat16 for d in seen_dtypes)  # the upcast was deferred
+    assert not runtime.needs_sync and all(p.grad is None for p in runtime.unsharded_params)
+    assert all(p.grad_dtype == torch.float32 for p in runtime.unsharded_params)  # restored for the next backward
+    for shard, w0, w1 in zip(runtime.sharded_params, wants[0], wants[1]):
+        want = (w0.float() + w1.float()).bfloat16()  # summed in fp32, stored in the shard's dtype
+        assert torch.equal(shard.grad.view(want.shape), want)
+
+    # one syncing backward: bf16 gradients reach the copy-in as they are
+    for p in runtime.sharded_params:
+        p.grad = None
+    seen_dtypes.clear()
+    model(xs[0]).backward(gos[0])
+    context.wait_and_clear_reduce_grad_states()
+    assert seen_dtypes and all(d == torch.bfloat16 for d in seen_dtypes)
+    for shard, w0 in zip(runtime.sharded_params, wants[0]):
+        assert torch.equal(shard.grad.view(w0.shape), w0)
+    torch.cuda.synchronize()
