@@ -44,6 +44,43 @@ def _pad_last_dim_to(tensor: torch.Tensor, target_dim: int) -> torch.Tensor:
     return padded
 
 
+class _SharedActivationQuantizer:
+    """The last quantization of an activation in each of the two forms (runs
+    along a row for the forward, runs of tokens for the weight gradient).
+
+    Projections that read the same activation (q, k and v; gate and up)
+    quantize it with the same arithmetic, so the second and third ask for the
+    very bytes the first produced: the result is kept until another tensor is
+    quantized in that form and handed out again when the request names the
+    same memory (address, shape, strides), unchanged since (version counter),
+    on the same stream.  The entry holds the activation itself, so its memory
+    cannot have been handed to another tensor in the meantime; that keeps at
+    most one activation per form alive a little longer.  Only the saving is
+    new: the outputs are the ones the quantizer would write again."""
+
+    def __init__(self) -> None:
+        self._entries: dict[str, tuple] = {}
+        self.enabled = True
+
+    def quantize(self, form: str, x: torch.Tensor, quantizer) -> tuple[torch.Tensor, torch.Tensor]:
+        if not self.enabled or torch.compiler.is_compiling():
+            return quantizer(x)
+        key = (x.data_ptr(), x._version, x.shape, x.stride(), x.dtype, hip_ops.stream_ptr(x.device))
+        entry = self._entries.get(form)
+        if entry is not None and entry[0] == key:
+            return entry[2]
+        result = quantizer(x)
+        self._entries[form] = (key, x, result)
+        return result
+
+    def clear(self) -> None:
+        self._entries.clear()
+
+
+#: shared by every ``Fp8BlockwiseGemms`` (the linears of a model create one per call)
+shared_activation_quantizer = _SharedActivationQuantizer()
+
+
 @dataclass(frozen=True)
 class Fp8BlockwiseGemms:
     """1x128 activation / 128x128 weight blockwise FP8 GEMMs."""
@@ -69,7 +106,7 @@ class Fp8BlockwiseGemms:
             x_2d = _pad_last_dim_to(x_2d, -(-in_dim // 8) * 8)
         # The quantizer pads the activation to whole 128-element runs itself;
         # only a weight whose rows are not whole runs has to be copied.
-        x_fp8, x_scale = hip_ops.act_quant_1x128(x_2d)
+        x_fp8, x_scale = shared_activation_quantizer.quantize("rows", x_2d, hip_ops.act_quant_1x128)
         padded_in_dim = x_fp8.shape[1]
         if weight_matrix.shape[1] != padded_in_dim or weight_matrix.stride(1) != 1 or weight_matrix.stride(0) % 16:
             weight_matrix = _pad_last_dim_to(weight_matrix.view(torch.uint8), padded_in_dim).view(torch.float8_e4m3fn)
@@ -130,7 +167,9 @@ class Fp8BlockwiseGemms:
             # runs of 128 tokens for both operands; the quantizer pads the token count itself
             if grad_t_fp8 is None:
                 grad_t_fp8, grad_t_scale = hip_ops.act_quant_128x1_transposed(grad_output_2d)
-            x_t_fp8, x_t_scale = hip_ops.act_quant_128x1_transposed(_as_quantizer_input(x_2d))
+            x_t_fp8, x_t_scale = shared_activation_quantizer.quantize(
+                "token_runs", _as_quantizer_input(x_2d), hip_ops.act_quant_128x1_transposed
+            )
             grad_weight = hip_ops.fp8_gemm_1x128_128x1(grad_t_fp8, grad_t_scale, x_t_fp8, x_t_scale)
             grad_weight = grad_weight[:out_dim, :in_dim].to(weight.dtype).contiguous().view(weight.shape)
         return grad_x, grad_weight
@@ -242,5 +281,5 @@ def _convert_child(parent: nn.Module, name: str, child: nn.Module, fqn: str, fil
 
 __all__ = [
     "FlexShardFloat8BlockwiseLinear", "Fp8BlockwiseGemms", "convert_to_flex_shard_float8_blockwise_linear",
-    "prequantized_linear",
+    "prequantized_linear", "shared_activation_quantizer",
 ]

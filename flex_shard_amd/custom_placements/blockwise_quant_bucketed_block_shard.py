@@ -687,7 +687,7 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         """Forward always packs and remembers the payload; a backward re-gather
         may take it back once if nothing about its sources changed.  This is
         the path of a bucket's first unshard, of shards that moved and of
-        staged shards; ``_prepare_steady`` serves every later call."""
+        staged shards; the steady-state branch of ``_prepare_unshard`` serves every later call."""
         if len(tensors) != len(infos):
             raise ValueError(
                 f"Quantized copy-in requires one tensor per ParamInfo, got {len(tensors)} tensors and {len(infos)} infos."
@@ -727,43 +727,6 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
             and all(a is b for a, b in zip(infos, entry[_E_INFOS]))
         )
 
-    def _prepare_steady(
-        self,
-        steady: "_SteadyPack",
-        signature: list,
-        versions: list,
-        tensors: list[torch.Tensor],
-        infos: list["ParamInfo"],
-        mesh: Any,
-        debug_fqn: str | None,
-        with_gathered: bool,
-    ) -> PlacementPreparedUnshard:
-        """The steady-state unshard preparation of a bucket whose launch is
-        stored: payload and gather output from this stream's rings, one C call."""
-        stream = _raw_stream(steady.device_index)
-        rings = steady.rings.get(stream)
-        if rings is None:
-            rings = steady.rings_for(stream, self._buffer_rings)
-        cache = self._local_packed_cache
-        if _is_backward_graph_task():
-            # a backward re-gather may take the forward's payload back, once
-            entry = cache.pop(steady.cache_key, None)
-            if self._cache_entry_matches(entry, steady.metadata, signature, versions, stream, infos):
-                payload = entry[_E_PACKED]
-            else:
-                payload, address = rings[0].take()
-                steady.launch.launch_raw(address, stream)
-        else:
-            payload, address = rings[0].take()
-            status = steady.launch_fn(steady.launch_handle, address, stream)
-            if status != 0:
-                steady.launch.launch_raw(address, stream)  # raises with the library's message
-            cache[steady.cache_key] = (signature, versions, stream, steady.metadata, tuple(infos), tuple(tensors), payload)
-        buffers = [payload, rings[1].take()[0]] if with_gathered else [payload]
-        return PlacementPreparedUnshard(
-            self, buffers, _QuantUnshardState(infos, mesh.get_group(), debug_fqn, steady.metadata)
-        )
-
     def release_buffer_rings(self) -> None:
         """Drop the recycled payload and gather buffers (they are otherwise
         held until the placement goes away)."""
@@ -791,9 +754,60 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
     ) -> PlacementPreparedUnshard:
         rank = mesh.get_local_rank()
         if tensors and len(tensors) == len(infos) and not _profiler._is_profiler_enabled and not torch.compiler.is_compiling():
-            steady, signature, versions = self._steady_pack_for(tensors, infos, rank)
-            if steady is not None:
-                return self._prepare_steady(steady, signature, versions, tensors, infos, mesh, debug_fqn, with_gathered)
+            # Steady state (every unshard of a bucket after its first): the
+            # launch is stored, so this is one pass over the shards that hold
+            # rows to see that they are the memory the launch reads, a payload
+            # and a gather output from this stream's recycled buffers, and one
+            # C call.  Written out in one piece: at a few microseconds per
+            # call, every Python call and temporary counts.
+            layout = infos[0].bucket_layout
+            group = self._steady_packs.get((id(layout), rank))
+            if group is not None:
+                live, by_first_address = group
+                steady = by_first_address.get(tensors[live[0]].data_ptr() if live else 0)
+                if steady is not None and steady.layout is layout and len(tensors) == steady.ntensors:
+                    versions = []
+                    for index, want in zip(live, steady.signature):
+                        info, t = infos[index], tensors[index]
+                        if (
+                            info is not steady.infos[index]
+                            or t.data_ptr() != want[0]
+                            or t.dtype != want[1]
+                            or t.shape != want[2]
+                            or t.stride() != want[3]
+                            or t.is_neg() != want[4]
+                            or (info.param_dtype or info.dtype) != want[5]
+                        ):
+                            break
+                        versions.append(t._version)
+                    else:
+                        signature = steady.signature  # equal to these shards', entry by entry
+                        stream = _raw_stream(steady.device_index)
+                        rings = steady.rings.get(stream)
+                        if rings is None:
+                            rings = steady.rings_for(stream, self._buffer_rings)
+                        cache = self._local_packed_cache
+                        payload = None
+                        if _is_backward_graph_task():
+                            # a backward re-gather may take the forward's payload back, once
+                            entry = cache.pop(steady.cache_key, None)
+                            if self._cache_entry_matches(entry, steady.metadata, signature, versions, stream, infos):
+                                payload = entry[_E_PACKED]
+                            else:
+                                payload, address = rings[0].take()
+                                steady.launch.launch_raw(address, stream)
+                        else:
+                            payload, address = rings[0].take()
+                            if steady.launch_fn(steady.launch_handle, address, stream) != 0:
+                                steady.launch.launch_raw(address, stream)  # raises with the library's message
+                            cache[steady.cache_key] = (
+                                signature, versions, stream, steady.metadata, tuple(infos), tuple(tensors), payload
+                            )
+                        return PlacementPreparedUnshard(
+                            self,
+                            [payload, rings[1].take()[0]] if with_gathered else [payload],
+                            _QuantUnshardState(infos, mesh.get_group(), debug_fqn, steady.metadata),
+                        )
         with record_copy_in():
             local, metadata = self._cached_local_quantized_chunks(tensors, infos, rank)
         buffers = [local]

@@ -10,6 +10,11 @@ as a substring of the kernel name; ``--per-step`` launches per step): the
 first ``--skip-steps`` steps are dropped and the region runs from the end of
 the last dropped step's last such launch to the end of the trace's last such
 launch.  Without ``--step-kernel`` the whole trace is the region.
+``--kernel NAME --first I --count N`` prints instead the duration statistics
+of dispatches I .. I+N-1 (start order) of one kernel, for a benchmark whose
+sections issue a known number of launches each.  ``--counters`` reads a
+``rocprofv3 --pmc`` ``*_counter_collection.csv`` instead and prints the average
+reading per dispatch of every kernel and counter.
 
 Figures: ``span`` = last end - first start inside the region; ``busy`` = the
 length of the union of all kernel intervals (kernels on different streams
@@ -132,14 +137,60 @@ def summarize(rows, steps: int | None) -> str:
     return "\n".join(lines)
 
 
+def kernel_slice(rows, kernel: str, first: int, count: int) -> str:
+    """Duration statistics of dispatches [first, first + count) (0-based, in
+    start order) of the kernel whose name contains ``kernel``."""
+    mine = [(start, end) for name, start, end in rows if kernel in name]
+    chosen = mine[first : first + count if count else None]
+    if not chosen:
+        return f"{kernel}: {len(mine)} dispatches in the trace, none in the slice"
+    durations = sorted((end - start) / 1e3 for start, end in chosen)
+    span = chosen[-1][1] - chosen[0][0]
+    return (
+        f"{kernel}: dispatches {first}..{first + len(chosen) - 1} of {len(mine)}: avg {sum(durations) / len(durations):.2f} us, "
+        f"median {durations[len(durations) // 2]:.2f}, min {durations[0]:.2f}, max {durations[-1]:.2f}; "
+        f"first start to last end {span / 1e3:.1f} us = {span / 1e3 / len(chosen):.2f} us per dispatch"
+    )
+
+
+def counters_summary(path: str) -> str:
+    """Per kernel and counter of a ``rocprofv3 --pmc`` CSV
+    (``*_counter_collection.csv``): dispatches and the average reading per
+    dispatch (a counter's rows of one dispatch, one per sampled instance, are
+    added first)."""
+    per_dispatch: dict[tuple[str, str, str], float] = defaultdict(float)
+    with open(path, newline="") as fh:
+        for row in csv.DictReader(fh):
+            key = (short_name(row["Kernel_Name"]) + f" (grid {row['Grid_Size']})", row["Counter_Name"], row["Dispatch_Id"])
+            per_dispatch[key] += float(row["Counter_Value"])
+    totals: dict[tuple[str, str], list[float]] = defaultdict(list)
+    for (kernel, counter, _), value in per_dispatch.items():
+        totals[(kernel, counter)].append(value)
+    lines = [f"{'kernel (grid size in threads)':<72} {'counter':<28} {'dispatches':>10} {'average':>16}"]
+    for (kernel, counter), values in sorted(totals.items()):
+        lines.append(f"{kernel[:72]:<72} {counter:<28} {len(values):>10} {sum(values) / len(values):>16.1f}")
+    return "\n".join(lines)
+
+
 def main(argv=None) -> None:
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("trace", help="rocprofv3 *_kernel_trace.csv")
     ap.add_argument("--step-kernel", help="substring of a kernel name that runs --per-step times per step")
     ap.add_argument("--per-step", type=int, default=1)
     ap.add_argument("--skip-steps", type=int, default=0)
+    ap.add_argument("--kernel", help="instead of the region summary: statistics of a slice of this kernel's dispatches")
+    ap.add_argument("--first", type=int, default=0, help="with --kernel: index of the slice's first dispatch")
+    ap.add_argument("--count", type=int, default=0, help="with --kernel: dispatches in the slice (0 = to the end)")
+    ap.add_argument("--counters", action="store_true", help="the file is a --pmc counter_collection.csv: average readings")
     args = ap.parse_args(argv)
-    rows, steps = select_region(read_trace(args.trace), args.step_kernel, args.per_step, args.skip_steps)
+    if args.counters:
+        sys.stdout.write(counters_summary(args.trace) + "\n")
+        return
+    trace = read_trace(args.trace)
+    if args.kernel:
+        sys.stdout.write(kernel_slice(trace, args.kernel, args.first, args.count) + "\n")
+        return
+    rows, steps = select_region(trace, args.step_kernel, args.per_step, args.skip_steps)
     sys.stdout.write(summarize(rows, steps) + "\n")
 
 

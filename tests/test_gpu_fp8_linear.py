@@ -163,3 +163,62 @@ def test_contraction_longer_than_one_window_of_weight_scales(device):
         xq.to(device), xs.to(device), wq.to(device), ws.t().contiguous().to(device), in_dim=n
     )
     assert torch.equal(got_t, got)
+
+
+def test_projections_that_share_an_activation_quantize_it_once(device):
+    """q, k and v read the same activation: the second and third forward (and
+    weight-gradient) products take the first one's quantization.  Same bits as
+    with the sharing switched off; a changed activation (in place, or another
+    tensor at another address) is quantized again."""
+    from unittest.mock import patch
+
+    from flex_shard_amd.blockwise_fp8.fp8_blockwise_linear import shared_activation_quantizer as shared
+
+    gen = torch.Generator().manual_seed(8)
+    x = torch.randn(256, 384, generator=gen).bfloat16().to(device)
+    grad = (torch.randn(256, 256, generator=gen) * 0.01).bfloat16().to(device)
+    weights = []
+    for _ in range(3):
+        wq, ws = eager.quantize_blockwise((torch.randn(256, 384, generator=gen) * 0.02).bfloat16(), 128)
+        weights.append(BlockwiseFp8Weight(wq.to(device), ws.to(device), 128, orig_dtype=torch.bfloat16))
+    gemms = Fp8BlockwiseGemms(block_size=128)
+
+    def run():
+        outs = [gemms.forward(x, w) for w in weights]
+        grads = [gemms.backward(grad, x, w, True, True) for w in weights]
+        return outs, grads
+
+    shared.clear()
+    calls = {"rows": 0, "tokens": 0}
+    real_rows, real_tokens = hip_ops.act_quant_1x128, hip_ops.act_quant_128x1_transposed
+
+    def count_rows(t, **kw):
+        calls["rows"] += 1
+        return real_rows(t, **kw)
+
+    def count_tokens(t, **kw):
+        calls["tokens"] += 1
+        return real_tokens(t, **kw)
+
+    with patch.object(hip_ops, "act_quant_1x128", count_rows), patch.object(hip_ops, "act_quant_128x1_transposed", count_tokens):
+        outs, grads = run()
+        assert calls == {"rows": 1, "tokens": 1}  # x once per form (the output gradient goes through act_quant_both)
+        x.mul_(2.0)  # in place: the version counter moves
+        outs2, _ = run()
+        assert calls == {"rows": 2, "tokens": 2}
+        moved = x.clone()
+        gemms.forward(moved, weights[0])
+        assert calls["rows"] == 3
+    shared.enabled = False
+    try:
+        plain_outs, plain_grads = run()
+    finally:
+        shared.enabled = True
+        shared.clear()
+    for a, b in zip(outs2, plain_outs):
+        assert torch.equal(a, b)
+    assert not torch.equal(outs[0], outs2[0])
+    x.div_(2.0)
+    again_outs, again_grads = run()
+    for (gx, gw), (px, pw) in zip(again_grads, grads):
+        assert torch.equal(gx, px) and torch.equal(gw, pw)
