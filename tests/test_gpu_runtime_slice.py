@@ -409,3 +409,96 @@ def test_microbatches_without_sync_accumulate_in_fp32_and_the_upcast_is_deferred
     for shard, w0 in zip(runtime.sharded_params, wants[0]):
         assert torch.equal(shard.grad.view(w0.shape), w0)
     torch.cuda.synchronize()
+
+
+def test_two_fp8_buckets_with_prefetch_on_alternating_unshard_streams(device):
+    """Two FP8 buckets (one per layer) under hooks that prefetch the bucket used
+    next, in the forward and in the backward: the prefetched unshards are begun
+    on the context's two unshard streams in turn, while the other layer
+    computes, and taken by the next unshard.  Rank 0 of 2 (the other rank's
+    rows and contributions deposited), three steps with an update of the
+    shards in between; everything against the kernels called directly."""
+    gen = torch.Generator().manual_seed(11)
+    model = _mlp(device, gen)
+    full = [p.detach().clone() for p in model.parameters()]
+    convert_to_flex_shard_float8_blockwise_linear(model)
+    context = BucketCommContext.create(device)
+    assert len(context.unshard_streams) == 2
+    world = 2
+    runtimes, groups, others = [], [], []
+    for index, layer in enumerate(model):
+        fqn = f"{index}.weight"
+        named = [(fqn, nn.Parameter(full[index].clone()))]
+        placement = Fp8BucketedBlockShard(world_size=world, weight_factory=make_blockwise_fp8_weight)
+        group = LocalReduceGroup(world, 0)
+        mesh1 = FakeMesh(world, 1)
+        infos1 = make_param_infos(named, placement, mesh1)
+        for info in infos1:
+            info.reduce_dtype = torch.float32
+        others.append((placement, named, infos1, mesh1))
+        runtime = BucketRuntime.shard_module_params(model, [fqn], placement, FakeMesh(world, 0, group), context)
+        runtimes.append(runtime)
+        groups.append(group)
+    used_streams = []
+    for index, (layer, runtime) in enumerate(zip(model, runtimes)):
+        runtime.install_hooks(
+            layer,
+            forward_prefetch=runtimes[index + 1] if index + 1 < len(runtimes) else None,
+            backward_prefetch=runtimes[index - 1] if index > 0 else None,
+        )
+        inner = runtime.begin_unshard
+
+        def recording(*args, _inner=inner, **kwargs):
+            handle = _inner(*args, **kwargs)
+            used_streams.append(handle._side_stream.cuda_stream if handle._side_stream is not None else None)
+            return handle
+
+        runtime.begin_unshard = recording
+    prefetched = {"forward": 0, "backward": 0}
+    for name, runtime in (("forward", runtimes[1]), ("backward", runtimes[0])):
+        inner = runtime.prefetch
+
+        def counting(_inner=inner, _name=name):
+            prefetched[_name] += 1
+            return _inner()
+
+        runtime.prefetch = counting
+
+    x = torch.randn(96, 256, generator=gen).bfloat16().to(device).requires_grad_()
+    grad_out = (torch.randn(96, 256, generator=gen) * 0.01).bfloat16().to(device)
+    scale = 1.0
+    for step in range(3):
+        if step:
+            scale *= 0.5
+            with torch.no_grad():
+                for runtime in runtimes:
+                    for p in runtime.sharded_params:
+                        p.mul_(0.5)
+                        p.grad = None
+                x.grad = None
+        weights = [w * scale for w in full]
+        want_out, want_gx, want_gw = _direct(weights, x.detach(), grad_out)
+        # what rank 1 sends: its payload of the current weights, and a gradient contribution
+        contributions = []
+        for index, (placement, named, infos1, mesh1) in enumerate(others):
+            named[0][1].data.copy_(weights[index])
+            shards1 = [local_rows(p, i) for (_, p), i in zip(named, infos1)]
+            groups[index].gather_rows[1] = placement.prepare_unshard_bucket(shards1, infos1, mesh1, None).buffers[0].clone()
+            other_grad = torch.randn(full[index].shape, generator=gen).to(device)
+            groups[index].deposit(1, placement.prepare_reduce_grad([other_grad], infos1, mesh1, None).buffers[0])
+            contributions.append(other_grad)
+        out = model(x)
+        assert all(not r.is_unsharded for r in runtimes)
+        out.backward(grad_out)
+        context.wait_and_clear_reduce_grad_states()
+        assert torch.equal(out.detach(), want_out) and torch.equal(x.grad, want_gx)
+        for runtime, gw, other_grad in zip(runtimes, want_gw, contributions):
+            (info,) = runtime.infos
+            want = local_rows(nn.Parameter((gw.float() * 0.5 + other_grad * 0.5).bfloat16()), info)
+            assert torch.equal(runtime.sharded_params[0].grad, want)
+    assert prefetched == {"forward": 3, "backward": 3}
+    side = [s for s in used_streams if s is not None]
+    assert len(side) == len(used_streams) == 12  # 2 buckets x (forward + backward) x 3 steps, all on side streams
+    assert set(side) == {s.cuda_stream for s in context.unshard_streams}
+    assert all(a != b for a, b in zip(side, side[1:]))  # the two streams take turns
+    torch.cuda.synchronize()
