@@ -754,7 +754,7 @@ def main() -> None:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB -> 256 MiB segment copy, the known-size kernel that the "
                     "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
-    ap.add_argument("--only", choices=("muon", "fp8_linear", "runtime_layer_step"),
+    ap.add_argument("--only", choices=("muon", "fp8_linear", "runtime_layer_step", "unpack", "gradients"),
                     help="profiling aid: run only this secondary section (for counter runs, which slow "
                     "every kernel down) and print its figures instead of the benchmark line")
     args = ap.parse_args()
@@ -771,6 +771,17 @@ def main() -> None:
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
+    if args.calibrate_copy:
+        calibrate_copy(device)
+    if args.only in ("unpack", "gradients"):
+        if args.only == "unpack":
+            placement, mesh, infos, work = build_quant_workload(device, 1)
+            del work
+            out = {"unpack_gathered_layout": bench_unpack(device, placement, infos)}
+        else:
+            out = {"gradient_path": bench_gradients(device)}
+        print(json.dumps(out))
+        return
     if args.only == "muon":
         print(json.dumps({"muon_newton_schulz": bench_muon(device)}))
         return
@@ -781,8 +792,6 @@ def main() -> None:
         print(json.dumps({"fp8_linear_forward_8192_tokens": bench_fp8_linear(device),
                           "fp8_linear_backward_8192_tokens": bench_fp8_linear_backward(device)}))
         return
-    if args.calibrate_copy:
-        calibrate_copy(device)
     q = bench_quant_pack(device, args.steps, args.warmup, args.layers, extras=True)
     placement, infos, work, metadata, mesh = q.pop("work")
     check_against_oracle(placement, infos, work, metadata, mesh)

@@ -547,6 +547,8 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         steady = by_first_address.get(tensors[live[0]].data_ptr() if live else 0)
         if steady is None or steady.layout is not infos[0].bucket_layout or len(tensors) != steady.ntensors:
             return None, None, None
+        if live and tensors[live[0]].get_device() != steady.device_index:  # an address means something on one device only
+            return None, None, None
         # (the loop of _shard_signature, with the identity check of the infos folded in)
         steady_infos = steady.infos
         signature, versions = [], []
@@ -765,7 +767,13 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
             if group is not None:
                 live, by_first_address = group
                 steady = by_first_address.get(tensors[live[0]].data_ptr() if live else 0)
-                if steady is not None and steady.layout is layout and len(tensors) == steady.ntensors:
+                if (
+                    steady is not None
+                    and steady.layout is layout
+                    and len(tensors) == steady.ntensors
+                    # an address means something on one device only (-1: not on a GPU)
+                    and (not live or tensors[live[0]].get_device() == steady.device_index)
+                ):
                     versions = []
                     for index, want in zip(live, steady.signature):
                         info, t = infos[index], tensors[index]
