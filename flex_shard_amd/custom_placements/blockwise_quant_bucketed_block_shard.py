@@ -129,10 +129,12 @@ GATHER_RING_SLOTS = 3
 class _QuantUnshardState:
     """The placement's private state of one prepared unshard."""
 
-    __slots__ = ("infos", "pg", "debug_fqn", "metadata")
+    __slots__ = ("infos", "pg", "debug_fqn", "metadata", "copied_out")
 
     def __init__(self, infos: list, pg: Any, debug_fqn: str | None, metadata: quant_plan.QuantBucketMetadata) -> None:
         self.infos, self.pg, self.debug_fqn, self.metadata = infos, pg, debug_fqn, metadata
+        #: the persistent buffers were refilled behind the exchange, in ``run_prepared_unshard``
+        self.copied_out = False
 
 
 # A forward pack that a backward re-gather may take once is remembered as a
@@ -250,6 +252,9 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
     qdata_dtype: torch.dtype
     scale_dtype: torch.dtype
     num_scale_tensors: int = 1
+    #: refill persistent buffers in ``run_prepared_unshard`` (behind a synchronous
+    #: exchange, on its stream) rather than in ``finish_prepared_unshard``
+    refill_behind_exchange: bool = True
 
     _BlockRowParam = quant_plan.BlockRowParam
     _BlockRowUnit = quant_plan.BlockRowUnit
@@ -834,11 +839,29 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         return state
 
     def run_prepared_unshard(self, prepared: PlacementPreparedUnshard, *, async_op: bool = False) -> Any | None:
-        """One uint8 all-gather of the equally sized payload rows."""
+        """One uint8 all-gather of the equally sized payload rows.  A refill of
+        persistent buffers (their storage is allocated before the unshard
+        begins: ``refills_persistent_buffers_in_finish`` is False) is written
+        here, right behind a synchronous exchange and on its stream, so a
+        prefetched bucket arrives unpacked and the consumer stream's finish is
+        views only; the gathered rows are then dead when run returns.  A first
+        unshard, an asynchronous exchange and a traced graph leave the
+        copy-out to finish."""
         state = self._unshard_state(prepared)
         local, gathered = prepared.buffers
         with record_comm("FlexShard::all_gather", state.debug_fqn):
-            return all_gather_rows(gathered, local, state.pg, async_op=async_op)
+            work = all_gather_rows(gathered, local, state.pg, async_op=async_op)
+        if (
+            self.refill_behind_exchange
+            and work is None
+            and prepared.persistent_buffers is not None
+            and not torch.compiler.is_compiling()
+        ):
+            rows = gathered.view(len(state.metadata.rank_qdata_numels), local.numel())
+            self._check_rank_rows(state, rows)
+            with record_copy_out():
+                state.copied_out = self._copy_out_rank_rows_fused(state.metadata, rows, prepared.persistent_buffers[0])
+        return work
 
     def finish_prepared_unshard(self, prepared: PlacementPreparedUnshard) -> PlacementUnshardResult:
         state = self._unshard_state(prepared)
@@ -900,6 +923,10 @@ class BlockwiseQuantBucketedBlockShard(BucketedBlockShard):
         self, prepared: PlacementPreparedUnshard, rank_rows: torch.Tensor, state: "_QuantUnshardState"
     ) -> PlacementUnshardResult:
         compact = self._compact_buffer(prepared, state.metadata, rank_rows.device)
+        if state.copied_out and prepared.persistent_buffers is not None:
+            return PlacementUnshardResult(
+                full_params=self._full_params_from_compact(state, compact), persistent_buffers=[compact]
+            )
         with record_copy_out():
             # Rank cuts partition one globally ordered stream of block rows, so
             # joining each rank's valid region restores parameter order.
