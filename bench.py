@@ -502,6 +502,74 @@ def bench_muon(device, reps=4):
             "newton_schulz_only_frac_of_bf16_mfma_peak": flops / ns_per / 1e9 / BF16_MFMA_PEAK_TFLOPS}
 
 
+def bench_side_stream_copies(device, gemms: int = 12, copies: int = 6, nbytes: int = 220 << 20):
+    """What a copy on a side stream costs the MFMA kernels on the main stream:
+    twelve FP8 forward GEMMs (8192 tokens, gate/up [14336, 4096]) alone, beside
+    six 220 MB segment copies, and beside six torch ``copy_`` kernels of the
+    same bytes.  Each figure is the best of three runs (the first launch of a
+    kernel in a process loads its code object, milliseconds that are not the
+    kernels' own)."""
+    from flex_shard_amd import hip_ops
+    from flex_shard_amd.custom_placements._copy_kernels import SegmentCopyDescriptor, copy_segments
+    from flex_shard_amd.testing import seeded_normal
+
+    tokens, n, k = 8192, 14336, 4096
+    x = seeded_normal((tokens, k), 1.0, 4000, device)
+    w = seeded_normal((n, k), 0.02, 4100, device)
+    wq, ws = hip_ops.act_quant_1x128(w)
+    ws = ws.t().contiguous()[: n // 128].contiguous()
+    xq, xs = hip_ops.act_quant_1x128(x)
+    y = torch.empty((tokens, n), dtype=torch.bfloat16, device=device)
+    src = torch.randint(0, 255, (nbytes // 4,), dtype=torch.int32, device=device)
+    dst = torch.empty_like(src)
+    desc = SegmentCopyDescriptor.create(src_offsets=[0], numels=[src.numel()], dst_offsets=[0], device=device)
+    side = torch.cuda.Stream(device)
+    side_work = {
+        "segment_copies": lambda: copy_segments(src, dst, desc),
+        "torch_copies": lambda: dst.copy_(src),
+    }
+
+    def run(kind):
+        for _ in range(3):
+            hip_ops.fp8_gemm_1x128_128x128(xq, xs, wq, ws, out=y)
+        torch.cuda.synchronize()
+        start, end, side_end = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+        start.record()
+        if kind:
+            side.wait_event(start)
+            with torch.cuda.stream(side):
+                for _ in range(copies):
+                    side_work[kind]()
+                side_end.record()
+        for _ in range(gemms):
+            hip_ops.fp8_gemm_1x128_128x128(xq, xs, wq, ws, out=y)
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end), (start.elapsed_time(side_end) if kind else 0.0)
+
+    def alone(kind):
+        side_work[kind]()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(copies):
+            side_work[kind]()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end)
+
+    out = {"gemms": gemms, "copies": copies, "copy_MB": nbytes / 1e6,
+           "gemms_alone_ms": min(run(None)[0] for _ in range(3))}
+    for kind in side_work:
+        main_ms, side_ms = min(run(kind) for _ in range(3))
+        out[kind] = {
+            "copies_alone_ms": alone(kind),
+            "gemms_beside_copies_ms": main_ms,
+            "copies_done_at_ms": side_ms,
+        }
+    return out
+
+
 def bench_fp8_linear(device, tokens: int = 8192, reps: int = 10):
     """Forward of the blockwise FP8 linear on the layer's projections: 8192
     tokens against q/o [4096, 4096], gate/up [14336, 4096] and down
@@ -754,7 +822,8 @@ def main() -> None:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB -> 256 MiB segment copy, the known-size kernel that the "
                     "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
-    ap.add_argument("--only", choices=("muon", "fp8_linear", "runtime_layer_step", "unpack", "gradients"),
+    ap.add_argument("--only", choices=("muon", "fp8_linear", "runtime_layer_step", "unpack", "gradients",
+                                       "side_stream_copies"),
                     help="profiling aid: run only this secondary section (for counter runs, which slow "
                     "every kernel down) and print its figures instead of the benchmark line")
     args = ap.parse_args()
@@ -787,6 +856,9 @@ def main() -> None:
         return
     if args.only == "runtime_layer_step":
         print(json.dumps({"runtime_layer_step": bench_runtime_layer_step(device)}))
+        return
+    if args.only == "side_stream_copies":
+        print(json.dumps({"side_stream_copies": bench_side_stream_copies(device)}))
         return
     if args.only == "fp8_linear":
         print(json.dumps({"fp8_linear_forward_8192_tokens": bench_fp8_linear(device),
@@ -896,6 +968,11 @@ def main() -> None:
         }
         torch.cuda.empty_cache()
         secondary["runtime_layer_step"] = bench_runtime_layer_step(device)
+        torch.cuda.empty_cache()
+        secondary["side_stream_copies"] = {
+            k: ({kk: round(vv, 3) for kk, vv in v.items()} if isinstance(v, dict) else round(v, 3) if isinstance(v, float) else v)
+            for k, v in bench_side_stream_copies(device).items()
+        }
         result["secondary"] = secondary
     print(json.dumps(result))
 

@@ -1,6 +1,7 @@
 """GPU parity of the gradient path (copy-in, fp32 accumulation, fixed-order
 reduce + copy-out) and of the Muon / Newton-Schulz kernels."""
 
+import numpy as np
 import pytest
 import torch
 import torch.nn as nn
@@ -143,6 +144,55 @@ def test_casting_pack_for_any_length_and_alignment(device, src_dtype, dst_dtype)
         want[do : do + n] = t[so : so + n].cpu().to(dst_dtype)
     want[zero_at : zero_at + zero_len] = 0
     assert torch.equal(out.cpu(), want)
+
+
+
+@pytest.mark.parametrize(
+    "src_dtype,dst_dtype",
+    [(torch.bfloat16, torch.float32), (torch.float32, torch.bfloat16), (torch.float32, torch.float32),
+     (torch.bfloat16, torch.bfloat16)],
+)
+@pytest.mark.parametrize("nsegments,longest", [(200, 150_000), (5000, 12_000)])
+def test_pack_shares_slices_of_uneven_segments(device, src_dtype, dst_dtype, nsegments, longest):
+    """A large gather: segments of very different lengths from several inputs,
+    zero-fill segments among them, several thousand segments in one launch,
+    aligned and unaligned offsets."""
+    rng = np.random.default_rng(nsegments + 1)
+    ninputs = 5
+    numels = rng.integers(0, longest, nsegments)
+    numels[nsegments // 3] = longest
+    aligned = rng.random(nsegments) < 0.7  # most segments on 8-element boundaries on both sides
+    numels = np.where(aligned, numels // 8 * 8, numels).tolist()
+    tensor_index = rng.integers(-1, ninputs, nsegments).tolist()
+    src_cursor = [0] * ninputs
+    src_offs, dst_offs, d_cur = [], [], 0
+    for k, (n, t) in enumerate(zip(numels, tensor_index)):
+        if not aligned[k]:
+            d_cur += int(rng.integers(1, 8))
+        if t >= 0:
+            if not aligned[k]:
+                src_cursor[t] += int(rng.integers(1, 8))
+            src_offs.append(src_cursor[t])
+            src_cursor[t] += n
+            src_cursor[t] = -(-src_cursor[t] // 8) * 8
+        else:
+            src_offs.append(0)
+        dst_offs.append(d_cur)
+        d_cur = -(-(d_cur + n) // 8) * 8
+    gen = torch.Generator().manual_seed(5)
+    inputs_host = [torch.randn(max(c, 8), generator=gen).to(src_dtype) for c in src_cursor]
+    inputs = [t.to(device) for t in inputs_host]
+    out = torch.full((d_cur + 8,), 7.0, dtype=dst_dtype, device=device)
+    table = lambda values: torch.tensor(values, dtype=torch.int64, device=device)
+    hip_ops.pack_segments(
+        table([t.data_ptr() for t in inputs]), table(tensor_index), table(src_offs), table(numels), table(dst_offs),
+        longest, src_dtype, out,
+    )
+    want = torch.full((d_cur + 8,), 7.0, dtype=dst_dtype)
+    for t, s, n, d in zip(tensor_index, src_offs, numels, dst_offs):
+        want[d : d + n] = 0 if t < 0 else inputs_host[t][s : s + n].to(dst_dtype)
+    view = torch.int32 if dst_dtype == torch.float32 else torch.int16
+    assert torch.equal(out.cpu().view(view), want.view(view))
 
 
 def test_copy_in_through_a_bucket_while_compiling(device):

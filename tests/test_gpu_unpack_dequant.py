@@ -1,6 +1,7 @@
 """GPU parity of the unpack side: rank-row compaction (segment copy), the fused
 compaction + dequantization kernel, and the dequantizer, against the oracle."""
 
+import numpy as np
 import pytest
 import torch
 import torch.nn as nn
@@ -217,6 +218,44 @@ def test_segment_copy_splits_long_segments(device, golden):
         ref[10:1007] = 0
         ref[1500:4833] = 0
         assert torch.equal(dst, ref)
+
+
+
+@pytest.mark.parametrize("nsegments,longest", [(300, 200_000), (6000, 9_000), (9, 3_000_000)])
+def test_segment_copy_shares_slices_of_uneven_segments(device, nsegments, longest):
+    """Large launches over segments of very different lengths: a few hundred
+    segments, several thousand short ones, and a few long ones, in any address
+    order, at every unit size and relative alignment; then the zero kernel
+    over the same destinations.  Bytes outside the segments stay."""
+    rng = np.random.default_rng(nsegments)
+    numels = rng.integers(0, longest, nsegments).tolist()
+    numels[nsegments // 2] = longest  # the longest sizes the launch
+    numels[0] = 0
+    gaps = rng.integers(0, 9, nsegments).tolist()
+    src_offs, dst_offs, s_cur, d_cur = [], [], 0, 3
+    for n, gap in zip(numels, gaps):
+        src_offs.append(s_cur)
+        dst_offs.append(d_cur)
+        s_cur += n + (gap % 3)
+        d_cur += n + gap
+    order = rng.permutation(nsegments).tolist()  # segments need not be sorted by address
+    pick = lambda values: [values[i] for i in order]
+    for dtype in (torch.uint8, torch.int16, torch.int64):
+        src_host = torch.from_numpy(rng.integers(0, 120, s_cur + 1).astype(np.int64)).to(dtype)
+        dst_host = torch.full((d_cur + 5,), 7, dtype=dtype)
+        desc = SegmentCopyDescriptor.create(
+            src_offsets=pick(src_offs), numels=pick(numels), dst_offsets=pick(dst_offs), device=device
+        )
+        dst = dst_host.to(device)
+        copy_segments(src_host.to(device), dst, desc)
+        want = dst_host.clone()
+        for s, n, d in zip(src_offs, numels, dst_offs):
+            want[d : d + n] = src_host[s : s + n]
+        assert torch.equal(dst.cpu(), want)
+        zero_segments(dst, desc)
+        for n, d in zip(numels, dst_offs):
+            want[d : d + n] = 0
+        assert torch.equal(dst.cpu(), want)
 
 
 # ---------------------------------------------------------------- dequantize
