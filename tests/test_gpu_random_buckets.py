@@ -1,0 +1,229 @@
+"""Seeded random buckets through the whole FP8 unshard path on the GPU
+(quantize + pack on every rank, rank rows gathered contiguous or strided at an
+odd byte offset, unpack with and without dequantization) against the CPU
+oracle: payload bytes, FP8 bytes, scale bits and dequantized bf16 bits."""
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from flex_shard_amd import Fp8BucketedBlockShard
+from flex_shard_amd.testing import (
+    FakeMesh,
+    gather_rank_rows,
+    local_rows,
+    make_param_infos,
+    prepare_unshard_on_each_rank,
+)
+from oracle import cport
+from oracle import layout as olayout
+
+pytestmark = pytest.mark.gpu
+
+
+class _RecordingFactory:
+    def __init__(self):
+        self.calls = []
+
+    def __call__(self, fp8_data, recip_scale, block_size, *, orig_dtype, requires_grad):
+        self.calls.append((fp8_data, recip_scale))
+        return fp8_data
+
+
+def _bits(t):
+    return t.contiguous().view(torch.int32)
+
+
+def _random_bucket(rng, block):
+    """1-6 parameters: matrices around multiples of the tile size (whole and
+    partial tiles in both directions, single rows, widths below one tile), some
+    stacked, with outliers, zero tiles, a subnormal tile and huge values."""
+    shapes = []
+    for _ in range(int(rng.integers(1, 7))):
+        rows = int(rng.integers(0, 4)) * block + int(rng.integers(0, block + 1))
+        cols = int(rng.integers(0, 4)) * block + int(rng.integers(0, block + 1))
+        rows, cols = max(rows, 1), max(cols, 1)
+        if rng.random() < 0.25:
+            shapes.append((int(rng.integers(2, 4)), rows, cols))
+        else:
+            shapes.append((rows, cols))
+    params = []
+    for shape in shapes:
+        w = torch.from_numpy(rng.standard_normal(shape).astype(np.float32)) * float(10.0 ** rng.integers(-4, 3))
+        flat = w.view(-1, shape[-1])
+        r, c = flat.shape
+        for _ in range(int(rng.integers(0, 3))):  # zero tiles
+            r0, c0 = int(rng.integers(0, r)) // block * block, int(rng.integers(0, c)) // block * block
+            flat[r0 : r0 + block, c0 : c0 + block] = 0
+        for _ in range(int(rng.integers(0, 3))):  # outliers
+            flat[int(rng.integers(0, r)), int(rng.integers(0, c))] = float(rng.choice([448.0, -3.0e4, 1.0e30, 7.5e-3]))
+        if rng.random() < 0.3:  # a tile whose amax is below the floor
+            r0, c0 = int(rng.integers(0, r)) // block * block, int(rng.integers(0, c)) // block * block
+            flat[r0 : r0 + block, c0 : c0 + block] = 1.0e-20
+        params.append(w)
+    return shapes, params
+
+
+@pytest.mark.parametrize("seed", range(160))
+def test_random_bucket_round_trip_matches_oracle(device, seed):
+    rng = np.random.default_rng(1000 + seed)
+    block = int(rng.choice([2, 4, 8, 16, 32, 128]))
+    world = int(rng.choice([1, 2, 3, 4, 5, 8]))
+    fp32_master = bool(rng.random() < 0.3)
+    shapes, params = _random_bucket(rng, block)
+    dtype = torch.float32 if fp32_master else torch.bfloat16
+    named = [(f"w{i}", nn.Parameter(p.to(dtype).to(device), requires_grad=False)) for i, p in enumerate(params)]
+    factory = _RecordingFactory()
+    pl = Fp8BucketedBlockShard(world_size=world, weight_factory=factory, block_size=block)
+
+    prepared = []
+    for rank in range(world):
+        mesh = FakeMesh(world, rank)
+        infos = make_param_infos(named, pl, mesh)
+        for info in infos:
+            info.param_dtype = torch.bfloat16  # an fp32 master is quantized as its bf16 rounding
+        shards = [local_rows(p, i) for (_, p), i in zip(named, infos, strict=True)]
+        prepared.append(pl.prepare_unshard_bucket(shards, infos, mesh, None))
+
+    # every rank's payload: the naive pack of whole-matrix quantization, pads zero
+    matrix_shapes = [olayout.matrix_shape(s) for s in shapes]
+    lay = olayout.quant_layout(matrix_shapes, block, world)
+    quantized = [cport.quantize_blockwise(p.view(-1, p.shape[-1]), block, cast_to_bf16=True) for p in params]
+    qs, ss = [q for q, _ in quantized], [s for _, s in quantized]
+    for rank in range(world):
+        want = olayout.pack_rank_payload(lay, rank, qs, ss, block)
+        assert torch.equal(prepared[rank].buffers[0].cpu(), want), f"payload of rank {rank}"
+
+    # gathered rows, contiguous or strided from an odd byte; unpack on a random rank
+    rows = gather_rank_rows(prepared)
+    if rng.random() < 0.5:
+        shift = int(rng.choice([1, 3, 5, 7]))
+        parent = torch.full((world, rows.shape[1] + 9), 0xEE, dtype=torch.uint8, device=device)
+        parent[:, shift : shift + rows.shape[1]] = rows
+        rows = parent[:, shift : shift + rows.shape[1]]
+    on_rank = int(rng.integers(0, world))
+    result, dequant = pl.finish_prepared_unshard_with_dequant(prepared[on_rank], rows)
+    assert len(factory.calls) == len(shapes) == len(dequant)
+    for (fp8, recip), deq, shape, (oq, osc) in zip(factory.calls, dequant, shapes, quantized, strict=True):
+        assert tuple(fp8.shape) == tuple(shape)
+        assert torch.equal(fp8.reshape(-1, shape[-1]).view(torch.uint8).cpu(), oq)
+        assert torch.equal(_bits(recip.cpu()).view(-1), _bits(osc).view(-1))
+        want = cport.dequant_blockwise(oq, osc, block)
+        assert deq.dtype == torch.bfloat16 and tuple(deq.shape) == tuple(shape)
+        got = deq.reshape(-1, shape[-1]).cpu()
+        nan = want.isnan()
+        assert torch.equal(got.isnan(), nan)
+        assert torch.equal(got.view(torch.int16)[~nan], want.view(torch.int16)[~nan])
+    factory.calls.clear()
+    plain = pl._finish_unshard_from_rank_rows(prepared[on_rank], rows)
+    for weight, (oq, _), shape in zip(plain.full_params, quantized, shapes, strict=True):
+        assert torch.equal(weight.reshape(-1, shape[-1]).view(torch.uint8).cpu(), oq)
+
+
+# ------------------------------------------------------------ dense unshard
+def _dense_shapes(rng, nblocks):
+    """1-5 parameters whose sharded dimension divides into ``nblocks`` blocks,
+    vectors among them."""
+    shapes = []
+    for _ in range(int(rng.integers(1, 6))):
+        rows = nblocks * int(rng.integers(1, 6))
+        if rng.random() < 0.25:
+            shapes.append((rows,))
+        else:
+            shapes.append((rows, int(rng.integers(1, 40))))
+    return shapes
+
+
+def _dense_case(rng, worlds, most_blocks):
+    """Random uneven blocks per rank and parameter shapes that the planner
+    accepts (it refuses a bucket in which some rank's range is only padding)."""
+    from flex_shard_amd import BucketedBlockShard
+
+    for _ in range(50):
+        world = int(rng.choice(worlds))
+        blocks = [int(rng.integers(0, most_blocks + 1)) for _ in range(world)]
+        if sum(blocks) == 0:
+            blocks[int(rng.integers(0, world))] = 1
+        shapes = _dense_shapes(rng, sum(blocks))
+        pl = BucketedBlockShard(dims=(0,), blocks_per_rank=tuple(blocks))
+        named = [(f"p{i}", nn.Parameter(torch.empty(s, device="meta"))) for i, s in enumerate(shapes)]
+        try:
+            for rank in range(world):
+                make_param_infos(named, pl, FakeMesh(world, rank))
+        except ValueError as exc:
+            assert "only padding" in str(exc)
+            continue
+        return world, blocks, shapes
+    raise AssertionError("no accepted bucket in 50 draws")
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_dense_unshard_restores_every_parameter(device, seed):
+    """BucketedBlockShard with random uneven blocks per rank (empty ranks
+    among them): prepare on every rank, local exchange, run + finish on every
+    rank; the full parameters are the originals in the unsharded dtype."""
+    from tests.test_gpu_dense_unshard import _unshard_every_rank
+
+    rng = np.random.default_rng(5000 + seed)
+    world, blocks, shapes = _dense_case(rng, [2, 3, 4, 5], 3)
+    master, unsharded = [(torch.float32, torch.bfloat16), (torch.float32, None), (torch.bfloat16, None)][int(rng.integers(0, 3))]
+    gen = torch.Generator().manual_seed(seed)
+    named = [(f"p{i}", nn.Parameter(torch.randn(s, generator=gen).to(master).to(device))) for i, s in enumerate(shapes)]
+    want_dtype = unsharded or master
+    _, _, results = _unshard_every_rank(named, tuple(blocks), device, unsharded)
+    for result in results:
+        for (_, param), full in zip(named, result.full_params, strict=True):
+            assert full.dtype == want_dtype and full.shape == param.shape
+            assert torch.equal(full, param.detach().to(want_dtype))
+
+
+# ------------------------------------------------------------ gradient path
+@pytest.mark.parametrize("seed", range(40))
+def test_random_gradient_bucket_copy_in_and_reduce(device, seed):
+    """Random dense buckets: every rank's one-pass copy-in equals the oracle's
+    reduce-scatter input rows, and the fixed-order reduction on a random rank
+    equals the oracle's left fold of the rank contributions, for SUM, AVG and a
+    custom divide factor, with fp32 or bf16 gradients reduced in fp32."""
+    import torch.distributed as dist
+
+    from flex_shard_amd import BucketedBlockShard, GradientReduction, LocalReduceGroup
+
+    rng = np.random.default_rng(9000 + seed)
+    world, blocks, shapes = _dense_case(rng, [2, 3, 4, 8], 2)
+    grad_dtype = torch.bfloat16 if rng.random() < 0.5 else torch.float32
+    rank = int(rng.integers(0, world))
+    reduction, post = [(GradientReduction(op=dist.ReduceOp.SUM), 1.0), (GradientReduction(), float(world)),
+                       (GradientReduction(divide_factor=16.0), 16.0)][int(rng.integers(0, 3))]
+    pl = BucketedBlockShard(dims=(0,), blocks_per_rank=tuple(blocks))
+    group = LocalReduceGroup(world, rank)
+    named = [(f"w{i}", nn.Parameter(torch.empty(s, device="meta", dtype=torch.bfloat16))) for i, s in enumerate(shapes)]
+    infos = make_param_infos(named, pl, FakeMesh(world, rank, group))
+    for info in infos:
+        info.reduce_dtype = torch.float32
+    layout = infos[0].bucket_layout
+    per_rank, mine = [], None
+    for r in range(world):
+        gen = torch.Generator().manual_seed(seed * 100 + r)
+        grads = [torch.randn(s, generator=gen).to(grad_dtype).to(device) for s in shapes]
+        per_rank.append(grads)
+        prepared = pl.prepare_reduce_grad(grads, infos, FakeMesh(world, rank, group), None)
+        want_rows = olayout.reduce_scatter_input(
+            [g.cpu() for g in grads], [layout.param_layouts[i.fqn].param_offset for i in infos],
+            layout.global_numel, layout.rank_offsets, layout.rank_numels, torch.float32,
+        )
+        assert torch.equal(prepared.buffers[0].view(want_rows.shape).cpu(), want_rows), f"copy-in of rank {r}"
+        group.deposit(r, prepared.buffers[0])
+        if r == rank:
+            mine = prepared
+    result = pl.reduce_prepared_grad(mine, reduction)
+    for i, (info, shard) in enumerate(zip(infos, result.sharded_grads, strict=True)):
+        total = None
+        for r in range(world):  # the left fold in rank order, each term scaled as the reduction scales it
+            term = per_rank[r][i].cpu().float()
+            if post != 1.0:
+                term = term * (1.0 / post)
+            total = term.clone() if total is None else total + term
+        lo = layout.param_layouts[info.fqn].local_global_offset - layout.param_layouts[info.fqn].param_offset
+        want = total.reshape(-1)[lo : lo + info.local_numel].view(info.local_shape)
+        assert shard.dtype == torch.float32 and torch.equal(shard.cpu(), want), (rank, i)
