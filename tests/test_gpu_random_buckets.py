@@ -227,3 +227,50 @@ def test_random_gradient_bucket_copy_in_and_reduce(device, seed):
         lo = layout.param_layouts[info.fqn].local_global_offset - layout.param_layouts[info.fqn].param_offset
         want = total.reshape(-1)[lo : lo + info.local_numel].view(info.local_shape)
         assert shard.dtype == torch.float32 and torch.equal(shard.cpu(), want), (rank, i)
+
+
+# ------------------------------------------------------------ FP8 products
+def _small_int_fp8(shape, gen, high):
+    return torch.randint(-high, high + 1, shape, generator=gen).to(torch.float32).to(torch.float8_e4m3fn)
+
+
+@pytest.mark.parametrize("seed", range(36))
+def test_random_shapes_of_the_three_fp8_products_are_integer_exact(device, seed):
+    """Random m, n (any size) and k (multiples of 128), small-integer operands
+    and power-of-two scales: forward, input-gradient and weight-gradient
+    products are the one bf16 rounding of the exact result, whatever the tile
+    tails and the number of tiles per round."""
+    from flex_shard_amd import hip_ops
+    from oracle import eager
+
+    rng = np.random.default_rng(7000 + seed)
+    m = int(rng.integers(1, 900))
+    n = int(rng.integers(1, 900)) if rng.random() < 0.8 else int(rng.integers(1, 40)) * 128
+    k = int(rng.integers(1, 9)) * 128
+    gen = torch.Generator().manual_seed(seed)
+    kb, nb = k // 128, -(-n // 128)
+    pow2 = lambda shape: torch.exp2(torch.randint(-2, 3, shape, generator=gen).float())
+    # forward: x [m, k] with scales [k/128, m], weight [n, k] with scales [n/128, k/128]
+    xq, wq = _small_int_fp8((m, k), gen, 1), _small_int_fp8((n, k), gen, 1)
+    xs, ws = pow2((kb, m)), pow2((nb, kb))
+    want = eager.fp8_gemm_1x128_128x128(xq, xs, wq, ws, out_dtype=torch.float32)
+    got = hip_ops.fp8_gemm_1x128_128x128(xq.to(device), xs.to(device), wq.to(device), ws.to(device))
+    assert torch.equal(got.cpu(), want.bfloat16()), ("forward", m, n, k)
+    # input gradient: contraction over the weight's rows (k of them here), its scales read across
+    in_dim = -(-n // 16) * 16  # the byte transpose takes widths that are multiples of 16
+    gq, gs = _small_int_fp8((m, k), gen, 1), pow2((kb, m))
+    w_rows = _small_int_fp8((k, in_dim), gen, 1)  # weight [out = k, in]
+    w_scales = pow2((kb, -(-in_dim // 128)))
+    wt = hip_ops.fp8_transpose(w_rows.to(device))  # [in, out]
+    got = hip_ops.fp8_gemm_1x128_128x128_dgrad(gq.to(device), gs.to(device), wt, w_scales.to(device), in_dim)
+    want = eager.fp8_gemm_1x128_128x128(
+        gq, gs, w_rows.view(torch.uint8).t().contiguous().view(torch.float8_e4m3fn), w_scales.t().contiguous(),
+        out_dtype=torch.float32,
+    )
+    assert torch.equal(got.cpu(), want.bfloat16()), ("input gradient", m, in_dim, k)
+    # weight gradient: both operands with one scale per column and run of 128 along k
+    aq, bq = _small_int_fp8((m, k), gen, 4), _small_int_fp8((n, k), gen, 4)
+    a_s, b_s = pow2((kb, m)), pow2((kb, n))
+    want = eager.fp8_gemm_1x128_128x1(aq, a_s, bq, b_s, out_dtype=torch.float32)
+    got = hip_ops.fp8_gemm_1x128_128x1(aq.to(device), a_s.to(device), bq.to(device), b_s.to(device))
+    assert torch.equal(got.cpu(), want.bfloat16()), ("weight gradient", m, n, k)
