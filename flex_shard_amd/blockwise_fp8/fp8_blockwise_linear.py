@@ -73,6 +73,20 @@ class _SharedActivationQuantizer:
         self._entries[form] = (key, x, result)
         return result
 
+    def quantize_both(self, x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+        """Both forms of ``x`` from one pass over it (``hip_ops.act_quant_both``),
+        kept and handed out like the single forms."""
+        if not self.enabled or torch.compiler.is_compiling():
+            return hip_ops.act_quant_both(x)
+        key = (x.data_ptr(), x._version, x.shape, x.stride(), x.dtype, hip_ops.stream_ptr(x.device))
+        rows, runs = self._entries.get("rows"), self._entries.get("token_runs")
+        if rows is not None and runs is not None and rows[0] == key and runs[0] == key:
+            return (*rows[2], *runs[2])
+        result = hip_ops.act_quant_both(x)
+        self._entries["rows"] = (key, x, result[:2])
+        self._entries["token_runs"] = (key, x, result[2:])
+        return result
+
     def clear(self) -> None:
         self._entries.clear()
 
@@ -91,6 +105,19 @@ class Fp8BlockwiseGemms:
     def forward(self, x_2d: torch.Tensor, weight: BlockwiseFp8Weight) -> torch.Tensor:
         """``x_2d @ weight_matrix.T`` with shape ``(tokens, rows)``; a stacked
         ``[*stack, out, in]`` weight multiplies as its flattened matrix."""
+        return self._forward(x_2d, weight, False)[0]
+
+    def forward_with_token_runs(
+        self, x_2d: torch.Tensor, weight: BlockwiseFp8Weight
+    ) -> tuple[torch.Tensor, tuple[torch.Tensor, torch.Tensor]]:
+        """:meth:`forward`, and the activation quantized in runs of 128 tokens,
+        transposed, with its scales: what :meth:`backward` needs of ``x_2d`` for
+        the weight gradient (pass it as ``x_token_runs``).  The one pass over
+        the activation that quantizes it for the product writes this form too,
+        so the backward neither keeps nor re-reads the bf16 activation."""
+        return self._forward(x_2d, weight, True)
+
+    def _forward(self, x_2d: torch.Tensor, weight: BlockwiseFp8Weight, with_token_runs: bool):
         self._check(weight)
         if x_2d.ndim != 2:
             raise ValueError(f"expected a 2D activation, got {tuple(x_2d.shape)}")
@@ -98,19 +125,19 @@ class Fp8BlockwiseGemms:
         logical_out_dim, in_dim = weight_matrix.shape
         if x_2d.shape[1] != in_dim:
             raise ValueError(f"input last dim {x_2d.shape[1]} does not match weight input dim {in_dim}")
-        if x_2d.dtype != torch.bfloat16:
-            x_2d = x_2d.to(torch.bfloat16)
-        if x_2d.stride(1) != 1 or x_2d.stride(0) % 8 or x_2d.data_ptr() % 16:
-            x_2d = x_2d.contiguous()
-        if in_dim % 8:
-            x_2d = _pad_last_dim_to(x_2d, -(-in_dim // 8) * 8)
+        x_2d = _as_quantizer_input(x_2d)
         # The quantizer pads the activation to whole 128-element runs itself;
         # only a weight whose rows are not whole runs has to be copied.
-        x_fp8, x_scale = shared_activation_quantizer.quantize("rows", x_2d, hip_ops.act_quant_1x128)
+        token_runs = None
+        if with_token_runs:
+            x_fp8, x_scale, *token_runs = shared_activation_quantizer.quantize_both(x_2d)
+            token_runs = tuple(token_runs)
+        else:
+            x_fp8, x_scale = shared_activation_quantizer.quantize("rows", x_2d, hip_ops.act_quant_1x128)
         padded_in_dim = x_fp8.shape[1]
         if weight_matrix.shape[1] != padded_in_dim or weight_matrix.stride(1) != 1 or weight_matrix.stride(0) % 16:
             weight_matrix = _pad_last_dim_to(weight_matrix.view(torch.uint8), padded_in_dim).view(torch.float8_e4m3fn)
-        return hip_ops.fp8_gemm_1x128_128x128(x_fp8, x_scale, weight_matrix, weight.recip_scale)
+        return hip_ops.fp8_gemm_1x128_128x128(x_fp8, x_scale, weight_matrix, weight.recip_scale), token_runs
 
     def _check(self, weight: BlockwiseFp8Weight) -> None:
         if self.block_size != weight.block_size:
@@ -127,19 +154,33 @@ class Fp8BlockwiseGemms:
     def backward(
         self,
         grad_output_2d: torch.Tensor,
-        x_2d: torch.Tensor,
+        x_2d: torch.Tensor | None,
         weight: BlockwiseFp8Weight,
         needs_x_grad: bool,
         needs_weight_grad: bool,
+        *,
+        x_token_runs: tuple[torch.Tensor, torch.Tensor] | None = None,
     ) -> tuple[torch.Tensor | None, torch.Tensor | None]:
         """``(grad_x_2d, grad_weight)``; ``grad_weight`` is contiguous, has the
-        weight's shape and its original dtype."""
+        weight's shape and its original dtype.  With ``x_token_runs`` (from
+        :meth:`forward_with_token_runs`) ``x_2d`` may be None."""
         self._check(weight)
         weight_matrix = weight.fp8_data.flatten(0, -2)
         out_dim, in_dim = weight_matrix.shape
         if grad_output_2d.ndim != 2 or grad_output_2d.shape[1] != out_dim:
             raise ValueError(f"grad_output {tuple(grad_output_2d.shape)} does not match weight output dim {out_dim}")
-        if x_2d.ndim != 2 or x_2d.shape != (grad_output_2d.shape[0], in_dim):
+        tokens = grad_output_2d.shape[0]
+        if x_token_runs is not None:
+            runs_fp8, runs_scale = x_token_runs
+            want = (-(-in_dim // 8) * 8, -(-tokens // 128) * 128)
+            if tuple(runs_fp8.shape) != want or tuple(runs_scale.shape) != (want[1] // 128, want[0]):
+                raise ValueError(
+                    f"x_token_runs {tuple(runs_fp8.shape)} / {tuple(runs_scale.shape)} do not match {tokens} tokens "
+                    f"and weight input dim {in_dim}"
+                )
+        elif x_2d is None:
+            raise ValueError("backward needs the activation or its token-run form")
+        if x_2d is not None and (x_2d.ndim != 2 or x_2d.shape != (tokens, in_dim)):
             raise ValueError(
                 f"activation {tuple(x_2d.shape)} does not match grad_output {tuple(grad_output_2d.shape)} "
                 f"and weight input dim {in_dim}"
@@ -167,9 +208,12 @@ class Fp8BlockwiseGemms:
             # runs of 128 tokens for both operands; the quantizer pads the token count itself
             if grad_t_fp8 is None:
                 grad_t_fp8, grad_t_scale = hip_ops.act_quant_128x1_transposed(grad_output_2d)
-            x_t_fp8, x_t_scale = shared_activation_quantizer.quantize(
-                "token_runs", _as_quantizer_input(x_2d), hip_ops.act_quant_128x1_transposed
-            )
+            if x_token_runs is not None:
+                x_t_fp8, x_t_scale = x_token_runs
+            else:
+                x_t_fp8, x_t_scale = shared_activation_quantizer.quantize(
+                    "token_runs", _as_quantizer_input(x_2d), hip_ops.act_quant_128x1_transposed
+                )
             grad_weight = hip_ops.fp8_gemm_1x128_128x1(grad_t_fp8, grad_t_scale, x_t_fp8, x_t_scale)
             grad_weight = grad_weight[:out_dim, :in_dim].to(weight.dtype).contiguous().view(weight.shape)
         return grad_x, grad_weight
@@ -196,25 +240,44 @@ class _PrequantizedLinearFunction(torch.autograd.Function):
         x_2d = x.reshape(-1, x_shape[-1])
         if x_2d.shape[-1] != weight.shape[-1]:
             raise ValueError(f"input last dim {x_2d.shape[-1]} does not match weight input dim {weight.shape[-1]}")
-        out = gemms.forward(x_2d, weight).reshape(*x_shape[:-1], *weight.shape[:-1])
+        # With a weight gradient to come, the pass that quantizes x for the
+        # product also writes the form the weight gradient contracts over, and
+        # that (1 byte per element) is kept instead of x.
+        keeps_token_runs = (
+            ctx.needs_input_grad[1] and hasattr(gemms, "forward_with_token_runs") and not torch.compiler.is_compiling()
+        )
+        if keeps_token_runs:
+            out, token_runs = gemms.forward_with_token_runs(x_2d, weight)
+            ctx.save_for_backward(weight, *token_runs)
+        else:
+            out = gemms.forward(x_2d, weight)
+            ctx.save_for_backward(weight, x)
+        out = out.reshape(*x_shape[:-1], *weight.shape[:-1])
         if bias is not None:
             out = out + bias
-        ctx.save_for_backward(x, weight)
+        ctx.keeps_token_runs = keeps_token_runs
+        ctx.x_shape = x_shape
         ctx.gemms = gemms
         ctx.has_bias = bias is not None
         return out
 
     @staticmethod
     def backward(ctx: Any, grad_output: torch.Tensor):
-        x, weight = ctx.saved_tensors
+        weight, *kept = ctx.saved_tensors
         out_dim = math.prod(weight.shape[:-1])
         grad_output_2d = grad_output.reshape(-1, out_dim).contiguous()
         needs_x_grad, needs_weight_grad, needs_bias_grad = ctx.needs_input_grad[:3]
-        grad_x, grad_weight = ctx.gemms.backward(
-            grad_output_2d, x.reshape(-1, x.shape[-1]), weight, needs_x_grad, needs_weight_grad
-        )
+        if ctx.keeps_token_runs:
+            grad_x, grad_weight = ctx.gemms.backward(
+                grad_output_2d, None, weight, needs_x_grad, needs_weight_grad, x_token_runs=tuple(kept)
+            )
+        else:
+            (x,) = kept
+            grad_x, grad_weight = ctx.gemms.backward(
+                grad_output_2d, x.reshape(-1, x.shape[-1]), weight, needs_x_grad, needs_weight_grad
+            )
         if grad_x is not None:
-            grad_x = grad_x.reshape(x.shape)
+            grad_x = grad_x.reshape(ctx.x_shape)
         grad_bias = None
         if ctx.has_bias and needs_bias_grad:
             grad_bias = grad_output_2d.sum(dim=0).view(weight.shape[:-1])

@@ -246,6 +246,52 @@ def test_autograd_through_the_prequantized_linear(device):
     assert torch.equal(module(x.to(device)).detach(), plain)
 
 
+
+@pytest.mark.parametrize("tokens,in_dim", [(96, 128), (77, 100), (300, 392)])
+def test_weight_gradient_from_the_forward_pass_token_runs(device, tokens, in_dim):
+    """With a weight gradient to come the forward quantizes the activation in
+    both forms at once and keeps the token-run form instead of the activation:
+    the gradients are bit for bit those of a backward that is handed the
+    activation, for ragged token counts and widths too; without a weight
+    gradient, and with a GEMM object that has only the reference's two methods,
+    the activation is kept as before."""
+    gen = torch.Generator().manual_seed(tokens + in_dim)
+    w, x, g, wq, ws, _ = _case(gen, tokens, (256,), in_dim, device)
+    gemms = Fp8BlockwiseGemms(block_size=128)
+
+    def run(requires_grad, gemms_object):
+        weight = BlockwiseFp8Weight(wq.to(device), ws.to(device), 128, orig_dtype=torch.bfloat16, requires_grad=requires_grad)
+        x_dev = x.to(device).clone().requires_grad_()
+        out = prequantized_linear(x_dev, weight, None, gemms_object)
+        saved = [t for t in out.grad_fn.saved_tensors if t is not None]
+        out.backward(g.to(device))
+        return out.detach(), x_dev.grad, weight.grad, saved
+
+    want_x, want_w = gemms.backward(g.to(device), x.to(device), BlockwiseFp8Weight(wq.to(device), ws.to(device), 128, orig_dtype=torch.bfloat16), True, True)
+    out, grad_x, grad_w, saved = run(True, gemms)
+    assert torch.equal(grad_x, want_x) and torch.equal(grad_w, want_w)
+    assert not any(t.dtype == torch.bfloat16 and t.shape == x.shape for t in saved)  # x itself is not kept
+    padded_in, padded_tokens = -(-in_dim // 8) * 8, -(-tokens // 128) * 128
+    assert any(t.dtype == E4M3 and tuple(t.shape) == (padded_in, padded_tokens) for t in saved)
+    out2, grad_x2, grad_w2, saved2 = run(False, gemms)
+    assert torch.equal(out2, out) and torch.equal(grad_x2, want_x) and grad_w2 is None
+    assert any(t.shape == x.shape and t.dtype == torch.bfloat16 for t in saved2)
+
+    class ReferenceInterfaceOnly:
+        block_size = 128
+        forward = staticmethod(gemms.forward)
+        backward = staticmethod(gemms.backward)
+
+    out3, grad_x3, grad_w3, saved3 = run(True, ReferenceInterfaceOnly())
+    assert torch.equal(out3, out) and torch.equal(grad_x3, want_x) and torch.equal(grad_w3, want_w)
+    assert any(t.shape == x.shape and t.dtype == torch.bfloat16 for t in saved3)
+    with pytest.raises(ValueError, match="x_token_runs"):
+        gemms.backward(g.to(device), None, BlockwiseFp8Weight(wq.to(device), ws.to(device), 128, orig_dtype=torch.bfloat16),
+                       True, True, x_token_runs=(torch.empty(8, 128, dtype=E4M3, device=device), torch.empty(1, 8, device=device)))
+    with pytest.raises(ValueError, match="token-run form"):
+        gemms.backward(g.to(device), None, BlockwiseFp8Weight(wq.to(device), ws.to(device), 128, orig_dtype=torch.bfloat16), True, True)
+
+
 def test_llama_sized_gradients_on_sampled_entries(device):
     """At the size the measurements quote (8192 tokens, a [4096, 14336]
     weight gradient and its input gradient) a sample of output entries is
