@@ -17,9 +17,9 @@ LIB_PATH = os.path.join(_PKG_DIR, "libflexshard_hip.so")
 FSH_OK = 0
 FSH_MAX_QUANT_CHUNKS = 24
 
-SRC_BF16, SRC_F32, SRC_F32_AS_BF16 = 0, 1, 2
+SRC_BF16, SRC_F32, SRC_F32_AS_BF16, SRC_F16, SRC_F32_AS_F16 = 0, 1, 2, 3, 4
 EPS_INPUT_DTYPE, EPS_FP32 = 0, 1
-DT_BF16, DT_F32 = 0, 1
+DT_BF16, DT_F32, DT_F16 = 0, 1, 2
 REDUCE_SUM, REDUCE_PREMUL, REDUCE_POSTMUL, REDUCE_POSTDIV = 0, 1, 2, 3
 
 

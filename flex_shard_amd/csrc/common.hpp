@@ -60,6 +60,29 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   return (f != f) ? 0x7FC0u : r;
 }
 
+// float -> fp16 bits, round to nearest even over the whole range, subnormal
+// results included, in integer arithmetic plus one fp32 add: the hardware
+// conversion rounded exact ties of subnormal results away from zero (e.g.
+// 690.5 x 2^-24 to 691) where torch's cast gives the even neighbour.
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+  uint32_t u = f32_as_u32(f);
+  const uint32_t sign = (u >> 16) & 0x8000u;
+  u &= 0x7FFFFFFFu;
+  uint32_t h;
+  if (u >= 0x47800000u) {  // 65536 and above, infinity, NaN
+    h = u > 0x7F800000u ? 0x7E00u : 0x7C00u;
+  } else if (u < 0x38800000u) {  // below 2^-14: the sum's low mantissa bits are the subnormal's
+    h = f32_as_u32(u32_as_f32(u) + 0.5f) - 0x3F000000u;
+  } else {  // rebias the exponent, add half an ulp (to even), carry into the exponent up to infinity
+    h = (u + 0xC8000FFFu + ((u >> 13) & 1u)) >> 13;
+  }
+  return sign | h;
+}
+// The fp16 value nearest to f, as a float.
+__device__ __forceinline__ float f32_round_to_f16(float f) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(f32_to_f16_bits(f))));
+}
+
 // Integer max across the 64 lanes of a wavefront, result in every lane.
 // Data-parallel-primitive moves: two quad permutes, two mirrors inside each
 // row of 16 lanes, then two row broadcasts leave the total in lane 63.

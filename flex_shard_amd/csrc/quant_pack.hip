@@ -50,7 +50,7 @@ struct QuantParams {
   int64_t total_tiles;
   int64_t zero_begin[2];
   int64_t zero_len[2];
-  float eps[3];  // indexed by src_kind
+  float eps[5];  // indexed by src_kind
   int32_t nchunks;
   int32_t block;
 };
@@ -201,8 +201,10 @@ __device__ __forceinline__ float load_as_quant_dtype(const QuantChunkDev& ch, in
   const int64_t idx = row * ch.src_row_stride + col;
   if (ch.src_kind == FSH_SRC_BF16)
     return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(ch.src)[idx]);
+  if (ch.src_kind == FSH_SRC_F16) return static_cast<float>(reinterpret_cast<const _Float16*>(ch.src)[idx]);
   const float f = reinterpret_cast<const float*>(ch.src)[idx];
   if (ch.src_kind == FSH_SRC_F32_AS_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(f));
+  if (ch.src_kind == FSH_SRC_F32_AS_F16) return f32_round_to_f16(f);
   return f;
 }
 
@@ -543,6 +545,10 @@ static int quantize_pack_impl(const fsh_quant_chunk* chunks, int32_t nchunks, vo
   prm.eps[FSH_SRC_BF16] = eps_bf16;
   prm.eps[FSH_SRC_F32] = eps32;
   prm.eps[FSH_SRC_F32_AS_BF16] = eps_bf16;
+  // 1e-12 is below fp16's smallest subnormal (6e-8): in the input dtype the
+  // floor is 0, and an all-zero tile gets scale inf, reciprocal 0 and NaN
+  // bytes, as the reference's arithmetic gives.
+  prm.eps[FSH_SRC_F16] = prm.eps[FSH_SRC_F32_AS_F16] = eps_mode == FSH_EPS_FP32 ? eps32 : 0.0f;
 
   int64_t tiles = 0;
   bool all_bf16_fast = true;
@@ -551,7 +557,7 @@ static int quantize_pack_impl(const fsh_quant_chunk* chunks, int32_t nchunks, vo
     if (in.src_dev == nullptr || in.rows <= 0 || in.in_dim <= 0 || in.src_row_stride < in.in_dim)
       return fail(FSH_EINVAL, "fsh_quantize_pack: chunk %d has bad shape (rows %lld, in_dim %lld, stride %lld)", i,
                   (long long)in.rows, (long long)in.in_dim, (long long)in.src_row_stride);
-    if (in.src_kind < 0 || in.src_kind > FSH_SRC_F32_AS_BF16)
+    if (in.src_kind < 0 || in.src_kind > FSH_SRC_F32_AS_F16)
       return fail(FSH_EINVAL, "fsh_quantize_pack: chunk %d has unknown src_kind %d", i, in.src_kind);
     const int64_t tiles_r = ceil_div(in.rows, block), tiles_c = ceil_div(in.in_dim, block);
     if (in.qdata_offset < 0 || in.qdata_offset + in.rows * in.in_dim > payload_nbytes)
@@ -561,7 +567,8 @@ static int quantize_pack_impl(const fsh_quant_chunk* chunks, int32_t nchunks, vo
         in.scale_offset + 4 * tiles_r * tiles_c > payload_nbytes)
       return fail(FSH_EINVAL, "fsh_quantize_pack: chunk %d scales at %lld misaligned or outside payload", i,
                   (long long)in.scale_offset);
-    const int64_t elem = in.src_kind == FSH_SRC_BF16 ? 2 : 4;
+    const int64_t elem = (in.src_kind == FSH_SRC_BF16 || in.src_kind == FSH_SRC_F16) ? 2 : 4;
+    const bool half_kind = in.src_kind == FSH_SRC_F16 || in.src_kind == FSH_SRC_F32_AS_F16;
     if (!aligned(in.src_dev, elem)) return fail(FSH_EINVAL, "fsh_quantize_pack: chunk %d source misaligned", i);
     QuantChunkDev& out = prm.chunks[i];
     out.src = static_cast<const uint8_t*>(in.src_dev);
@@ -573,7 +580,7 @@ static int quantize_pack_impl(const fsh_quant_chunk* chunks, int32_t nchunks, vo
     out.tile_begin = tiles;
     out.tiles_c = static_cast<int32_t>(tiles_c);
     out.src_kind = in.src_kind;
-    out.fast = block == 128 && aligned(in.src_dev, 16) && (in.src_row_stride * elem) % 16 == 0 &&
+    out.fast = !half_kind && block == 128 && aligned(in.src_dev, 16) && (in.src_row_stride * elem) % 16 == 0 &&
                in.in_dim % 8 == 0 && in.qdata_offset % 8 == 0;
     all_bf16_fast = all_bf16_fast && out.fast && in.src_kind == FSH_SRC_BF16 && in.rows < (1LL << 30) &&
                     in.in_dim < (1LL << 30);

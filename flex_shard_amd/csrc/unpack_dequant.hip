@@ -46,7 +46,7 @@ __device__ __forceinline__ void dequant4(uint32_t w, float s, float* out) {
   out[3] = hi.y * s;
 }
 
-template <int DQ>  // FSH_DT_BF16 or FSH_DT_F32
+template <int DQ>  // FSH_DT_BF16, FSH_DT_F32 or FSH_DT_F16
 __global__ __launch_bounds__(kThreads) void unpack_dequant_kernel(
     const uint8_t* __restrict__ rows, const fsh_unpack_chunk* __restrict__ chunks,
     const int64_t* __restrict__ tile_starts, int nchunks, uint8_t* __restrict__ compact,
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kThreads) void unpack_dequant_kernel(
   const int64_t t = bid - tile_starts[lo];
   const int64_t tr = t / tiles_c, tc = t - tr * tiles_c;
   const int tid = threadIdx.x;
-  constexpr int kElem = DQ == FSH_DT_BF16 ? 2 : 4;
+  constexpr int kElem = DQ == FSH_DT_F32 ? 4 : 2;
 
   const float scale = load_f32_any(rows + ch.src_scale_offset + 4 * (tr * tiles_c + tc));
   if (compact != nullptr && tid == 0)
@@ -127,6 +127,13 @@ __global__ __launch_bounds__(kThreads) void unpack_dequant_kernel(
           o.z = f32_to_bf16_bits(f[4]) | (f32_to_bf16_bits(f[5]) << 16);
           o.w = f32_to_bf16_bits(f[6]) | (f32_to_bf16_bits(f[7]) << 16);
           store_stream_u32x4(dq + idx * 2, o);
+        } else if (DQ == FSH_DT_F16) {
+          u32x4 o;
+          o.x = f32_to_f16_bits(f[0]) | (f32_to_f16_bits(f[1]) << 16);
+          o.y = f32_to_f16_bits(f[2]) | (f32_to_f16_bits(f[3]) << 16);
+          o.z = f32_to_f16_bits(f[4]) | (f32_to_f16_bits(f[5]) << 16);
+          o.w = f32_to_f16_bits(f[6]) | (f32_to_f16_bits(f[7]) << 16);
+          store_stream_u32x4(dq + idx * 2, o);
         } else {
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
@@ -152,6 +159,8 @@ __global__ __launch_bounds__(kThreads) void unpack_dequant_kernel(
       const float f = __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(b), 0) * scale;
       if (DQ == FSH_DT_BF16)
         reinterpret_cast<uint16_t*>(dq)[idx] = static_cast<uint16_t>(f32_to_bf16_bits(f));
+      else if (DQ == FSH_DT_F16)
+        reinterpret_cast<uint16_t*>(dq)[idx] = static_cast<uint16_t>(f32_to_f16_bits(f));
       else
         reinterpret_cast<float*>(dq)[idx] = f;
     }
@@ -171,9 +180,9 @@ FSH_API int fsh_unpack_dequant(const void* rows_dev, const fsh_unpack_chunk* chu
   if (nchunks == 0 || total_tiles == 0) return FSH_OK;
   if (!rows_dev || !chunks_dev || !tile_starts_dev) return fail(FSH_EINVAL, "fsh_unpack_dequant: null pointer");
   if (!compact_dev && !dequant_dev) return fail(FSH_EINVAL, "fsh_unpack_dequant: nothing to write");
-  if (dequant_dtype != FSH_DT_BF16 && dequant_dtype != FSH_DT_F32)
+  if (dequant_dtype != FSH_DT_BF16 && dequant_dtype != FSH_DT_F32 && dequant_dtype != FSH_DT_F16)
     return fail(FSH_EINVAL, "fsh_unpack_dequant: unsupported dequant dtype %d", dequant_dtype);
-  if (dequant_dev && !aligned(dequant_dev, dequant_dtype == FSH_DT_BF16 ? 2 : 4))
+  if (dequant_dev && !aligned(dequant_dev, dequant_dtype == FSH_DT_F32 ? 4 : 2))
     return fail(FSH_EINVAL, "fsh_unpack_dequant: dequant buffer misaligned for its dtype");
   if (total_tiles > 0x7FFFFFFFLL)
     return fail(FSH_ENOTSUP, "fsh_unpack_dequant: %lld tiles exceed the grid limit", (long long)total_tiles);
@@ -181,6 +190,10 @@ FSH_API int fsh_unpack_dequant(const void* rows_dev, const fsh_unpack_chunk* chu
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dequant_dtype == FSH_DT_BF16)
     hipLaunchKernelGGL((unpack_dequant_kernel<FSH_DT_BF16>), g, b, 0, s, static_cast<const uint8_t*>(rows_dev),
+                       chunks_dev, tile_starts_dev, nchunks, static_cast<uint8_t*>(compact_dev),
+                       static_cast<uint8_t*>(dequant_dev), block);
+  else if (dequant_dtype == FSH_DT_F16)
+    hipLaunchKernelGGL((unpack_dequant_kernel<FSH_DT_F16>), g, b, 0, s, static_cast<const uint8_t*>(rows_dev),
                        chunks_dev, tile_starts_dev, nchunks, static_cast<uint8_t*>(compact_dev),
                        static_cast<uint8_t*>(dequant_dev), block);
   else

@@ -65,9 +65,11 @@ def _quantize_dense_weight_to_blockwise_fp8(
     _require_gpu_rows(weight, "Blockwise FP8 quantization")
     if weight.stride(-1) != 1:
         weight = weight.contiguous()
-    kind = {torch.bfloat16: hip_ops.SRC_BF16, torch.float32: hip_ops.SRC_F32}.get(weight.dtype)
+    kind = {torch.bfloat16: hip_ops.SRC_BF16, torch.float32: hip_ops.SRC_F32, torch.float16: hip_ops.SRC_F16}.get(
+        weight.dtype
+    )
     if kind is None:
-        raise NotImplementedError(f"the HIP quantizer reads bf16 or fp32 weights, not {weight.dtype}")
+        raise NotImplementedError(f"the HIP quantizer reads bf16, fp16 or fp32 weights, not {weight.dtype}")
     tiles_r, tiles_c = _scale_shape(weight.shape, block_size)
     data_nbytes = out_dim * in_dim
     scale_start = quant_plan.align_up(data_nbytes, quant_plan.VEC_ALIGN_BYTES)
@@ -171,9 +173,11 @@ class Fp8BucketedBlockShard(BlockwiseQuantBucketedBlockShard):
             (torch.bfloat16, torch.bfloat16): hip_ops.SRC_BF16,
             (torch.float32, torch.float32): hip_ops.SRC_F32,
             (torch.float32, torch.bfloat16): hip_ops.SRC_F32_AS_BF16,
+            (torch.float16, torch.float16): hip_ops.SRC_F16,
+            (torch.float32, torch.float16): hip_ops.SRC_F32_AS_F16,
         }
-        if quant_dtype not in (torch.bfloat16, torch.float32):
-            raise NotImplementedError(f"the HIP quantizer quantizes bf16 or fp32 values, not {quant_dtype}")
+        if quant_dtype not in (torch.bfloat16, torch.float32, torch.float16):
+            raise NotImplementedError(f"the HIP quantizer quantizes bf16, fp16 or fp32 values, not {quant_dtype}")
         return table.get((tensor_dtype, quant_dtype))
 
     def _make_quantize_pack_launch(self, specs, payload_nbytes, zero_ranges, device) -> hip_ops.QuantPackPlan:

@@ -16,6 +16,7 @@ import torch
 from . import _native
 from ._native import (
     DT_BF16,
+    DT_F16,
     DT_F32,
     EPS_FP32,
     EPS_INPUT_DTYPE,
@@ -24,13 +25,15 @@ from ._native import (
     REDUCE_PREMUL,
     REDUCE_SUM,
     SRC_BF16,
+    SRC_F16,
     SRC_F32,
     SRC_F32_AS_BF16,
+    SRC_F32_AS_F16,
 )
 
 __all__ = [
-    "DT_BF16", "DT_F32", "EPS_FP32", "EPS_INPUT_DTYPE", "REDUCE_POSTDIV", "REDUCE_POSTMUL",
-    "REDUCE_PREMUL", "REDUCE_SUM", "SRC_BF16", "SRC_F32", "SRC_F32_AS_BF16",
+    "DT_BF16", "DT_F16", "DT_F32", "EPS_FP32", "EPS_INPUT_DTYPE", "REDUCE_POSTDIV", "REDUCE_POSTMUL",
+    "REDUCE_PREMUL", "REDUCE_SUM", "SRC_BF16", "SRC_F16", "SRC_F32", "SRC_F32_AS_BF16", "SRC_F32_AS_F16",
     "MuonStepPlan", "QuantChunkSpec", "QuantPackPlan", "accumulate_grad", "act_quant_128x1_transposed", "act_quant_1x128", "act_quant_both",
     "copy_segments", "fp8_gemm_1x128_128x1", "fp8_gemm_1x128_128x128", "fp8_gemm_1x128_128x128_dgrad",
     "fp8_transpose", "gemm_nt", "gemm_nt_group", "muon_apply", "muon_prepare", "newton_schulz_multi",
@@ -116,7 +119,7 @@ class QuantPackPlan:
                 raise ValueError(
                     f"chunk must be a non-empty 2-D view with unit column stride, got {tuple(t.shape)} / {t.stride()}"
                 )
-            expected = torch.bfloat16 if spec.src_kind == SRC_BF16 else torch.float32
+            expected = {SRC_BF16: torch.bfloat16, SRC_F16: torch.float16}.get(spec.src_kind, torch.float32)
             if t.dtype != expected:
                 raise ValueError(f"chunk dtype {t.dtype} does not match src_kind {spec.src_kind}")
             slot.src_dev = t.data_ptr()
@@ -262,7 +265,7 @@ def unpack_dequant(
     if dequant is not None:
         if not dequant.is_contiguous():
             raise ValueError("dequant must be contiguous")
-        dq_dtype = _dt(dequant.dtype)
+        dq_dtype = DT_F16 if dequant.dtype == torch.float16 else _dt(dequant.dtype)
     status = _native.lib().fsh_unpack_dequant(
         rows.data_ptr(), chunk_table.data_ptr(), tile_starts.data_ptr(), nchunks, total_tiles,
         compact.data_ptr() if compact is not None else None,

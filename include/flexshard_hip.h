@@ -55,6 +55,8 @@ const char* fsh_last_error(void);
 #define FSH_SRC_BF16 0        /* bf16 shard, quantized as is                  */
 #define FSH_SRC_F32 1         /* fp32 shard, quantized as fp32                */
 #define FSH_SRC_F32_AS_BF16 2 /* fp32 master shard, rounded to bf16 first     */
+#define FSH_SRC_F16 3         /* fp16 shard, quantized as is (element path)   */
+#define FSH_SRC_F32_AS_F16 4  /* fp32 master shard, rounded to fp16 first     */
 
 /* Floor applied to a tile's amax. */
 #define FSH_EPS_INPUT_DTYPE 0 /* 1e-12 rounded to the quantization dtype      */
@@ -127,6 +129,7 @@ int fsh_zero_segments(void* dst_dev, const int64_t* numels_dev, const int64_t* d
 
 #define FSH_DT_BF16 0
 #define FSH_DT_F32 1
+#define FSH_DT_F16 2 /* fsh_unpack_dequant's dequantized output only */
 /* out[dst_off[s]+i] = cast(inputs[tensor_idx[s]][src_off[s]+i]), i < numel[s];
  * offsets in elements; input_ptrs_dev holds the inputs' device addresses.  A
  * negative tensor index makes the segment a zero fill, so one launch can
@@ -159,7 +162,7 @@ typedef struct fsh_unpack_chunk {
  * of ceil(rows/block)*ceil(in_dim/block); tile_starts_dev[i] = first tile
  * index of chunk i (nchunks+1 entries, exclusive prefix sum).
  * compact_dev may be NULL (no compaction), dequant_dev may be NULL (no
- * dequantization).  dequant dtype is FSH_DT_BF16 or FSH_DT_F32.
+ * dequantization).  dequant dtype is FSH_DT_BF16, FSH_DT_F32 or FSH_DT_F16.
  */
 int fsh_unpack_dequant(const void* rows_dev, const fsh_unpack_chunk* chunks_dev,
                        const int64_t* tile_starts_dev, int32_t nchunks, int64_t total_tiles,

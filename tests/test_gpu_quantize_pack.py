@@ -173,6 +173,52 @@ def test_fp32_master_is_quantized_as_bf16(device, golden):
     assert torch.equal(payload[256 * 256 :].view(torch.int32), _bits(osc).view(-1))
 
 
+
+@pytest.mark.parametrize("shape,block", [((6, 4), 4), ((12, 6), 4), ((130, 129), 128), ((256, 384), 128), ((64, 64), 16), ((1, 3), 4)])
+def test_fp16_shards_quantize_like_their_fp32_values(device, shape, block):
+    """An fp16 weight (and an fp32 master quantized as fp16) against the eager
+    restatement of the reference on fp16 input.  fp16 to fp32 is exact and no
+    nonzero fp16 amax lies below the 1e-12 floor, so for every tile with a
+    nonzero amax the result also equals the (pinned) C quantization of the
+    upcast values.  In fp16 the floor itself rounds to zero: an all-zero tile
+    gets scale inf, stored reciprocal 0 and NaN bytes (0 x inf), as the
+    reference's arithmetic gives; the sign of that NaN depends on the platform
+    and is not compared.  With the fp32 floor the zero tile is finite."""
+    gen = torch.Generator().manual_seed(shape[0] * 31 + shape[1])
+    w = (torch.randn(shape, generator=gen) * 0.05).half()
+    w[0, 0] = 6.1e-5  # subnormal and tiny values keep their exact magnitude
+    w[-1, -1] = 65504.0
+    oq, osc = eager.quantize_blockwise(w, block)
+    q, s = _quant_gpu(w.to(device), block)
+    assert torch.equal(q, oq.view(torch.uint8)) and torch.equal(_bits(s), _bits(osc))
+    cq, csc = cport.quantize_blockwise(w.float(), block)
+    assert torch.equal(q, cq) and torch.equal(_bits(s), _bits(csc))
+    # an fp32 master whose parameter dtype is fp16 quantizes its fp16 rounding
+    master = w.float() * (1 + 2.0**-13)
+    pl = Fp8BucketedBlockShard(world_size=1, weight_factory=_factory, block_size=block)
+    param = nn.Parameter(master.to(device))
+    (info,) = make_param_infos([("w", param)], pl, FakeMesh(1))
+    info.param_dtype = torch.float16
+    prepared = pl.prepare_unshard_bucket([param.detach()], [info], FakeMesh(1), None)
+    md = prepared.placement_state.metadata
+    payload = prepared.buffers[0].cpu()
+    rq, rs = eager.quantize_blockwise(master.half(), block)
+    assert torch.equal(payload[: md.rank_qdata_numels[0]], rq.view(torch.uint8).reshape(-1))
+    assert torch.equal(payload[md.rank_scale_byte_offsets[0] : md.rank_packed_nbytes[0]].view(torch.int32), _bits(rs).view(-1))
+    # zero tile
+    z = w.clone()
+    z[:block, :block] = 0
+    q, s = _quant_gpu(z.to(device), block)
+    oq, osc = eager.quantize_blockwise(z, block)
+    tile = torch.zeros(shape, dtype=torch.bool)
+    tile[:block, :block] = True
+    assert s[0, 0].item() == 0.0 and osc[0, 0].item() == 0.0
+    assert ((q[tile] & 0x7F) == 0x7F).all() and ((oq.view(torch.uint8)[tile] & 0x7F) == 0x7F).all()
+    assert torch.equal(q[~tile], oq.view(torch.uint8)[~tile])
+    q, s = _quant_gpu(z.to(device), block, eps_mode=hip_ops.EPS_FP32)
+    assert (q[tile] == 0).all() and _bits(s)[0, 0].item() == 0x2720D7C5
+
+
 def test_strided_and_offset_sources(device):
     """Shards that are row-strided views (unit column stride) or start at an
     odd element are read in place; results equal the contiguous copy."""

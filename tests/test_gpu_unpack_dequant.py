@@ -18,6 +18,7 @@ from flex_shard_amd.testing import (
     seeded_bucket,
 )
 from oracle import cport
+from oracle import eager as eager_oracle
 from oracle import layout as olayout
 
 pytestmark = pytest.mark.gpu
@@ -291,8 +292,48 @@ def test_dequant_is_bit_exact_with_oracle(device, shape, block):
         want = cport.dequant_blockwise(data, scale, block, dtype)
         view = torch.int32 if dtype == torch.float32 else torch.int16
         assert torch.equal(got.view(view), want.view(view))
+    # fp16 output: torch's own cast of the fp32 product (these scales put most products among the fp16
+    # subnormals, exact ties included, and the larger ones past fp16's range)
+    for factor in (1.0, 64.0, 3.0e4):
+        got = blockwise_dequant_weight(data.to(device).view(E4M3), (scale * factor).to(device), block, torch.float16).cpu()
+        want = eager_oracle.dequant_blockwise(data.view(E4M3), scale * factor, block, torch.float16)
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
     nan = torch.full((4, 4), 0x7F, dtype=torch.uint8)
     assert blockwise_dequant_weight(nan.to(device).view(E4M3), torch.ones(1, 1, device=device), 4).isnan().all()
+    assert blockwise_dequant_weight(nan.to(device).view(E4M3), torch.ones(1, 1, device=device), 4, torch.float16).isnan().all()
+
+
+
+def test_fp16_bucket_round_trip_and_fp16_dequantization(device):
+    """fp16 parameters through pack, gather and unpack on 4 ranks: the factory
+    gets the oracle's bytes and scales with orig_dtype fp16, and the fused
+    dequantization writes fp16 equal to torch's one rounding of the fp32
+    product, from aligned rows and from strided rows at an odd offset."""
+    shapes, block, world = [(512, 256), (130, 136), (3, 64, 128)], 128, 4
+    factory = RecordingFactory()
+    pl = Fp8BucketedBlockShard(world_size=world, weight_factory=factory, block_size=block)
+    gen = torch.Generator().manual_seed(8)
+    named = [(f"w{i}", nn.Parameter((torch.randn(s, generator=gen) * 0.02).half().to(device), requires_grad=False))
+             for i, s in enumerate(shapes)]
+    prepared = prepare_unshard_on_each_rank(pl, named, world)
+    rows = gather_rank_rows(prepared)
+    parent = torch.zeros((world, rows.shape[1] + 5), dtype=torch.uint8, device=device)
+    parent[:, 3 : 3 + rows.shape[1]] = rows
+    for rank_rows in (rows, parent[:, 3 : 3 + rows.shape[1]]):
+        factory.calls.clear()
+        _, dequant = pl.finish_prepared_unshard_with_dequant(prepared[1], rank_rows, dequant_dtype=torch.float16)
+        for (_, p), call, deq in zip(named, factory.calls, dequant, strict=True):
+            flat = p.detach().cpu().flatten(0, -2)
+            oq, osc = eager_oracle.quantize_blockwise(flat, block)
+            assert call[3] == torch.float16
+            assert torch.equal(call[0].flatten(0, -2).view(torch.uint8).cpu(), oq.view(torch.uint8))
+            assert torch.equal(_bits(call[1].cpu()), _bits(osc))
+            want = eager_oracle.dequant_blockwise(oq, osc, block, torch.float16)
+            assert deq.dtype == torch.float16 and deq.shape == p.shape
+            assert torch.equal(deq.flatten(0, -2).cpu().view(torch.int16), want.view(torch.int16))
+    fp8 = factory.calls[0][0]
+    got = blockwise_dequant_weight(fp8.flatten(0, -2), factory.calls[0][1], block, torch.float16)
+    assert torch.equal(got.view(torch.int16), dequant[0].flatten(0, -2).view(torch.int16))
 
 
 def test_fused_unpack_with_dequant_matches_oracle(device):
