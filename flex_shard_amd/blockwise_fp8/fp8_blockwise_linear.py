@@ -101,6 +101,9 @@ class Fp8BlockwiseGemms:
 
     block_size: int
     out_dtype: torch.dtype = torch.bfloat16
+    #: ``backward`` reads a gradient whose rows are strided (a slice of a wider
+    #: matrix) in place; the autograd function then hands it over as it is
+    accepts_strided_rows = True
 
     def forward(self, x_2d: torch.Tensor, weight: BlockwiseFp8Weight) -> torch.Tensor:
         """``x_2d @ weight_matrix.T`` with shape ``(tokens, rows)``; a stacked
@@ -265,7 +268,9 @@ class _PrequantizedLinearFunction(torch.autograd.Function):
     def backward(ctx: Any, grad_output: torch.Tensor):
         weight, *kept = ctx.saved_tensors
         out_dim = math.prod(weight.shape[:-1])
-        grad_output_2d = grad_output.reshape(-1, out_dim).contiguous()
+        grad_output_2d = grad_output.reshape(-1, out_dim)
+        if not getattr(ctx.gemms, "accepts_strided_rows", False):
+            grad_output_2d = grad_output_2d.contiguous()
         needs_x_grad, needs_weight_grad, needs_bias_grad = ctx.needs_input_grad[:3]
         if ctx.keeps_token_runs:
             grad_x, grad_weight = ctx.gemms.backward(

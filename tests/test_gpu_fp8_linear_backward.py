@@ -292,6 +292,28 @@ def test_weight_gradient_from_the_forward_pass_token_runs(device, tokens, in_dim
         gemms.backward(g.to(device), None, BlockwiseFp8Weight(wq.to(device), ws.to(device), 128, orig_dtype=torch.bfloat16), True, True)
 
 
+
+def test_strided_output_gradient_is_read_in_place(device):
+    """The gradient of an output that was concatenated with another tensor is
+    a column slice of a wider matrix (row stride 2 x its width): the backward
+    reads it as it lies and gives the bits of the contiguous copy."""
+    gen = torch.Generator().manual_seed(21)
+    w, x, g, wq, ws, _ = _case(gen, 200, (256,), 384, device)
+    weight = BlockwiseFp8Weight(wq.to(device), ws.to(device), 128, orig_dtype=torch.bfloat16, requires_grad=True)
+    x_dev = x.to(device).requires_grad_()
+    out = prequantized_linear(x_dev, weight)
+    other = torch.zeros_like(out).requires_grad_()
+    wide_grad = torch.randn(200, 512, generator=gen).bfloat16().to(device) * 0.01
+    seen = []
+    out.register_hook(lambda grad: seen.append((grad.stride(), grad.is_contiguous())))
+    torch.cat([other, out], dim=-1).backward(wide_grad)
+    assert seen == [((512, 1), False)]
+    want_x, want_w = Fp8BlockwiseGemms(block_size=128).backward(
+        wide_grad[:, 256:].contiguous(), x.to(device), weight.detach(), True, True
+    )
+    assert torch.equal(x_dev.grad, want_x) and torch.equal(weight.grad, want_w)
+
+
 def test_llama_sized_gradients_on_sampled_entries(device):
     """At the size the measurements quote (8192 tokens, a [4096, 14336]
     weight gradient and its input gradient) a sample of output entries is
