@@ -115,6 +115,8 @@ class MuonGroup(Structure):
         ("workspace_nbytes", c_int64),
         ("neg_adjusted_lr", c_float),
         ("direction_scale", c_float),
+        ("master_dtype", c_int32),
+        ("reserved", c_int32),
     ]
 
 
@@ -186,6 +188,8 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     ),
     "fsh_muon_prepare": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_float, c_float, c_int32, c_void_p]),
     "fsh_muon_apply": (c_int, [c_void_p, c_void_p, c_int64, c_float, c_float, c_float, c_void_p]),
+    "fsh_muon_prepare_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_float, c_float, c_int32, c_void_p]),
+    "fsh_muon_apply_f32": (c_int, [c_void_p, c_void_p, c_int64, c_float, c_float, c_float, c_void_p]),
     "fsh_muon_step": (
         c_int,
         [POINTER(MuonGroup), c_int32, c_float, c_float, c_int32, c_float, c_float, c_float, c_float, c_int32, c_float,

@@ -173,6 +173,63 @@ __global__ __launch_bounds__(kThreads) void muon_apply_kernel(uint16_t* __restri
         muon_apply_one(bf16_bits_to_f32(param[i]), bf16_bits_to_f32(dir[i]), decay, neg_lr, dir_scale));
 }
 
+// fp32 master state: m = lerp(m, g, 1-mu) stays fp32; out = bf16 of the
+// Nesterov blend (or of m), the input of the orthogonalization.
+__global__ __launch_bounds__(kThreads) void muon_prepare_f32_kernel(float* __restrict__ mom,
+                                                                   const float* __restrict__ grad,
+                                                                   uint16_t* __restrict__ out, int64_t n,
+                                                                   float one_minus_mu, float mu, int nesterov,
+                                                                   int vec_ok) {
+  const int64_t tid = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t nthreads = static_cast<int64_t>(gridDim.x) * kThreads;
+  int64_t done = 0;
+  if (vec_ok) {
+    const int64_t groups = n / 8;
+    for (int64_t gi = tid; gi < groups; gi += nthreads) {
+      float m[8], g[8];
+      load8_f32(mom + gi * 8, m);
+      load8_f32(grad + gi * 8, g);
+      uint32_t ob[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) muon_prepare_one_f32(m[j], g[j], one_minus_mu, mu, nesterov, &m[j], &ob[j]);
+      store8_f32(mom + gi * 8, m);
+      store_stream_u32x4(out + gi * 8, pack8(ob));
+    }
+    done = groups * 8;
+  }
+  for (int64_t i = done + tid; i < n; i += nthreads) {
+    float m;
+    uint32_t ob;
+    muon_prepare_one_f32(mom[i], grad[i], one_minus_mu, mu, nesterov, &m, &ob);
+    mom[i] = m;
+    out[i] = static_cast<uint16_t>(ob);
+  }
+}
+
+// p = p * decay; p = p + neg_lr * d', d' = scale == 1 ? d : d * scale, all fp32; d is bf16.
+__global__ __launch_bounds__(kThreads) void muon_apply_f32_kernel(float* __restrict__ param,
+                                                                 const uint16_t* __restrict__ dir, int64_t n,
+                                                                 float decay, float neg_lr, float dir_scale,
+                                                                 int vec_ok) {
+  const int64_t tid = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t nthreads = static_cast<int64_t>(gridDim.x) * kThreads;
+  int64_t done = 0;
+  if (vec_ok) {
+    const int64_t groups = n / 8;
+    for (int64_t gi = tid; gi < groups; gi += nthreads) {
+      float pv[8], dv[8];
+      load8_f32(param + gi * 8, pv);
+      unpack8(load_stream_u32x4(dir + gi * 8), dv);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) pv[j] = muon_apply_one_f32(pv[j], dv[j], decay, neg_lr, dir_scale);
+      store8_f32(param + gi * 8, pv);
+    }
+    done = groups * 8;
+  }
+  for (int64_t i = done + tid; i < n; i += nthreads)
+    param[i] = muon_apply_one_f32(param[i], bf16_bits_to_f32(dir[i]), decay, neg_lr, dir_scale);
+}
+
 }  // namespace
 }  // namespace fsh
 
@@ -266,4 +323,34 @@ FSH_API int fsh_muon_apply(void* param_dev, const void* direction_dev, int64_t n
                      static_cast<const uint16_t*>(direction_dev), numel, decay_factor, neg_adjusted_lr,
                      direction_scale, vec_ok);
   return check_launch("fsh_muon_apply");
+}
+
+FSH_API int fsh_muon_prepare_f32(float* momentum_dev, const float* grad_dev, void* out_dev, int64_t numel,
+                                 float lerp_weight, float nesterov_weight, int32_t nesterov, void* stream) {
+  using namespace fsh;
+  if (numel < 0) return fail(FSH_EINVAL, "fsh_muon_prepare_f32: negative numel");
+  if (numel == 0) return FSH_OK;
+  if (!momentum_dev || !grad_dev || !out_dev) return fail(FSH_EINVAL, "fsh_muon_prepare_f32: null pointer");
+  if (!aligned(momentum_dev, 4) || !aligned(grad_dev, 4) || !aligned(out_dev, 2))
+    return fail(FSH_EINVAL, "fsh_muon_prepare_f32: pointers misaligned for their dtypes");
+  const int vec_ok = aligned(momentum_dev, 16) && aligned(grad_dev, 16) && aligned(out_dev, 16);
+  hipLaunchKernelGGL(muon_prepare_f32_kernel, dim3(grid_for(ceil_div(numel, 8))), dim3(kThreads), 0,
+                     static_cast<hipStream_t>(stream), momentum_dev, grad_dev, static_cast<uint16_t*>(out_dev), numel,
+                     lerp_weight, nesterov_weight, nesterov, vec_ok);
+  return check_launch("fsh_muon_prepare_f32");
+}
+
+FSH_API int fsh_muon_apply_f32(float* param_dev, const void* direction_dev, int64_t numel, float decay_factor,
+                               float neg_adjusted_lr, float direction_scale, void* stream) {
+  using namespace fsh;
+  if (numel < 0) return fail(FSH_EINVAL, "fsh_muon_apply_f32: negative numel");
+  if (numel == 0) return FSH_OK;
+  if (!param_dev || !direction_dev) return fail(FSH_EINVAL, "fsh_muon_apply_f32: null pointer");
+  if (!aligned(param_dev, 4) || !aligned(direction_dev, 2))
+    return fail(FSH_EINVAL, "fsh_muon_apply_f32: pointers misaligned for their dtypes");
+  const int vec_ok = aligned(param_dev, 16) && aligned(direction_dev, 16);
+  hipLaunchKernelGGL(muon_apply_f32_kernel, dim3(grid_for(ceil_div(numel, 8))), dim3(kThreads), 0,
+                     static_cast<hipStream_t>(stream), param_dev, static_cast<const uint16_t*>(direction_dev), numel,
+                     decay_factor, neg_adjusted_lr, direction_scale, vec_ok);
+  return check_launch("fsh_muon_apply_f32");
 }

@@ -1084,6 +1084,55 @@ __global__ __launch_bounds__(kNormThreads) void muon_prepare_sumsq_kernel(const 
   store_block_partial(s, lds, &q.partial[b * kNormBlocksPerMatrix + blockIdx.x]);
 }
 
+// The same for fp32 master state: momentum buffers and gradients are fp32,
+//   m = lerp(m, g, 1 - mu) (fp32);  u = bf16(nesterov ? lerp(g, m, mu) : m).
+__global__ __launch_bounds__(kNormThreads) void muon_prepare_sumsq_f32_kernel(const MuonPrepareBatch q) {
+  __shared__ float lds[kNormThreads / 64];
+  const int64_t b = blockIdx.y;
+  float* mom = reinterpret_cast<float*>(q.momentum_ptrs[b]);
+  const float* grad = reinterpret_cast<const float*>(q.grad_ptrs[b]);
+  uint16_t* out = q.out + b * q.numel;
+  const int64_t groups = q.numel / 8;
+  const int64_t per = ceil_div(groups, (int64_t)kNormBlocksPerMatrix);
+  const int64_t begin = blockIdx.x * per;
+  const int64_t end = (begin + per) < groups ? (begin + per) : groups;
+  float s = 0.0f;
+  constexpr int kUnroll = 2;  // 2 x (32 + 32) bytes of loads per thread before the first store
+  int64_t g = begin + threadIdx.x;
+  for (; g + (kUnroll - 1) * kNormThreads < end; g += kUnroll * kNormThreads) {
+    float mv[kUnroll][8], gv[kUnroll][8];
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+      load8_f32(mom + (g + k * kNormThreads) * 8, mv[k]);
+      load8_f32(grad + (g + k * kNormThreads) * 8, gv[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+      uint32_t ob[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        muon_prepare_one_f32(mv[k][j], gv[k][j], q.one_minus_mu, q.mu, q.nesterov, &mv[k][j], &ob[j]);
+      store8_f32(mom + (g + k * kNormThreads) * 8, mv[k]);
+      const u32x4 u = pack8(ob);
+      store_stream_u32x4(out + (g + k * kNormThreads) * 8, u);
+      s = add_squares8(s, u);
+    }
+  }
+  for (; g < end; g += kNormThreads) {
+    float mv[8], gv[8];
+    load8_f32(mom + g * 8, mv);
+    load8_f32(grad + g * 8, gv);
+    uint32_t ob[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) muon_prepare_one_f32(mv[j], gv[j], q.one_minus_mu, q.mu, q.nesterov, &mv[j], &ob[j]);
+    store8_f32(mom + g * 8, mv);
+    const u32x4 u = pack8(ob);
+    store_stream_u32x4(out + g * 8, u);
+    s = add_squares8(s, u);
+  }
+  store_block_partial(s, lds, &q.partial[b * kNormBlocksPerMatrix + blockIdx.x]);
+}
+
 // The update of Muon for the same batch: parameter b (a separate allocation)
 // takes the direction in slot b of the batch buffer,
 //   p = bf16(p * decay);  p = bf16(p + neg_lr * d)   (d first scaled and rounded if scale != 1).
@@ -1123,6 +1172,40 @@ __global__ __launch_bounds__(kNormThreads) void muon_apply_batch_kernel(const Mu
 #pragma unroll
         for (int j = 0; j < 8; ++j) pb[j] = muon_apply_one(pv[j], dv[j], q.decay, q.neg_lr, q.dir_scale);
         store_stream_u32x4(param + g * 8, pack8(pb));
+      }
+    }
+  }
+}
+
+// The update on fp32 parameters: p = p * decay; p = p + neg_lr * d, d the bf16
+// direction (times scale in fp32 if scale != 1).
+__global__ __launch_bounds__(kNormThreads) void muon_apply_batch_f32_kernel(const MuonApplyBatch q) {
+  const int64_t b = blockIdx.y;
+  float* param = reinterpret_cast<float*>(q.param_ptrs[b]);
+  const uint16_t* dir = q.direction + b * q.numel;
+  const int64_t groups = q.numel / 8;
+  constexpr int kUnroll = 2;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kNormThreads * kUnroll;
+  for (int64_t g0 = static_cast<int64_t>(blockIdx.x) * kNormThreads * kUnroll + threadIdx.x; g0 < groups; g0 += stride) {
+    float pv[kUnroll][8];
+    u32x4 draw[kUnroll];
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+      const int64_t g = g0 + k * kNormThreads;
+      if (g < groups) {
+        load8_f32(param + g * 8, pv[k]);
+        draw[k] = load_stream_u32x4(dir + g * 8);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+      const int64_t g = g0 + k * kNormThreads;
+      if (g < groups) {
+        float dv[8];
+        unpack8(draw[k], dv);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pv[k][j] = muon_apply_one_f32(pv[k][j], dv[j], q.decay, q.neg_lr, q.dir_scale);
+        store8_f32(param + g * 8, pv[k]);
       }
     }
   }
@@ -1437,6 +1520,9 @@ FSH_API int fsh_muon_step(const fsh_muon_group* groups, int32_t count, float ler
       return fail(FSH_EINVAL, "fsh_muon_step: group %d has a null pointer", i);
     if (!aligned(g.batch_dev, 16) || !aligned(g.workspace_dev, 256))
       return fail(FSH_EINVAL, "fsh_muon_step: group %d: batch buffer must be 16-byte and workspace 256-byte aligned", i);
+    if (g.master_dtype != FSH_DT_BF16 && g.master_dtype != FSH_DT_F32)
+      return fail(FSH_EINVAL, "fsh_muon_step: group %d: master_dtype %d is neither FSH_DT_BF16 nor FSH_DT_F32", i,
+                  g.master_dtype);
     if (g.workspace_nbytes < fsh_newton_schulz_workspace_bytes(g.batch, g.rows, g.cols))
       return fail(FSH_EINVAL, "fsh_muon_step: group %d: workspace of %lld bytes, need %lld", i,
                   (long long)g.workspace_nbytes, (long long)fsh_newton_schulz_workspace_bytes(g.batch, g.rows, g.cols));
@@ -1459,8 +1545,12 @@ FSH_API int fsh_muon_step(const fsh_muon_group* groups, int32_t count, float ler
     q.one_minus_mu = lerp_weight;
     q.mu = nesterov_weight;
     q.nesterov = nesterov;
-    hipLaunchKernelGGL(muon_prepare_sumsq_kernel, dim3(kNormBlocksPerMatrix, static_cast<uint32_t>(g.batch)),
-                       dim3(kNormThreads), 0, stream, q);
+    if (g.master_dtype == FSH_DT_F32)
+      hipLaunchKernelGGL(muon_prepare_sumsq_f32_kernel, dim3(kNormBlocksPerMatrix, static_cast<uint32_t>(g.batch)),
+                         dim3(kNormThreads), 0, stream, q);
+    else
+      hipLaunchKernelGGL(muon_prepare_sumsq_kernel, dim3(kNormBlocksPerMatrix, static_cast<uint32_t>(g.batch)),
+                         dim3(kNormThreads), 0, stream, q);
     if (int rc = check_launch("muon_prepare_sumsq_kernel")) return rc;
   }
   NsState st[FSH_MAX_NS_PROBLEMS];
@@ -1472,7 +1562,9 @@ FSH_API int fsh_muon_step(const fsh_muon_group* groups, int32_t count, float ler
   // separate launch applies them.
   GemmUpdate updates[FSH_MAX_NS_PROBLEMS];
   for (int i = 0; i < count; ++i) {
-    const bool fused = steps > 0 && takes_large_tile_kernel(ns_product(st[i], 2, a, b, c, true));
+    // (the epilogue writes bf16 parameters; fp32 masters take the separate launch)
+    const bool fused = steps > 0 && groups[i].master_dtype == FSH_DT_BF16 &&
+                       takes_large_tile_kernel(ns_product(st[i], 2, a, b, c, true));
     updates[i].ptrs = fused ? groups[i].param_ptrs_dev : nullptr;
     updates[i].decay = decay_factor;
     updates[i].neg_lr = groups[i].neg_adjusted_lr;
@@ -1491,10 +1583,12 @@ FSH_API int fsh_muon_step(const fsh_muon_group* groups, int32_t count, float ler
     q.dir_scale = g.direction_scale;
     const int64_t groups8 = q.numel / 8;
     const int64_t blocks = ceil_div(groups8, (int64_t)kNormThreads * 4);  // four 16-byte groups per thread
-    hipLaunchKernelGGL(muon_apply_batch_kernel,
-                       dim3(static_cast<uint32_t>(blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks)),
-                            static_cast<uint32_t>(g.batch)),
-                       dim3(kNormThreads), 0, stream, q);
+    const dim3 grid(static_cast<uint32_t>(blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks)),
+                    static_cast<uint32_t>(g.batch));
+    if (g.master_dtype == FSH_DT_F32)
+      hipLaunchKernelGGL(muon_apply_batch_f32_kernel, grid, dim3(kNormThreads), 0, stream, q);
+    else
+      hipLaunchKernelGGL(muon_apply_batch_kernel, grid, dim3(kNormThreads), 0, stream, q);
     if (int rc = check_launch("muon_apply_batch_kernel")) return rc;
   }
   return FSH_OK;

@@ -50,7 +50,19 @@ def _require_bf16_gpu(*tensors: torch.Tensor) -> None:
         if t.device.type != "cuda":
             raise RuntimeError("Muon kernels run on the GPU; this package has no CPU compute path.")
         if t.dtype != torch.bfloat16:
-            raise NotImplementedError(f"the Muon kernels operate on bf16 tensors, got {t.dtype}")
+            raise NotImplementedError(f"the Newton-Schulz kernels operate on bf16 tensors, got {t.dtype}")
+        if not t.is_contiguous():
+            raise ValueError("the Muon kernels need contiguous tensors")
+
+
+def _require_master_gpu(*tensors: torch.Tensor) -> None:
+    """Parameters, gradients and momentum buffers: bf16 or fp32 (the
+    reference's optimizer math is dtype-generic; its own tests run fp32)."""
+    for t in tensors:
+        if t.device.type != "cuda":
+            raise RuntimeError("Muon kernels run on the GPU; this package has no CPU compute path.")
+        if t.dtype not in (torch.bfloat16, torch.float32):
+            raise NotImplementedError(f"the Muon kernels update bf16 or fp32 tensors, got {t.dtype}")
         if not t.is_contiguous():
             raise ValueError("the Muon kernels need contiguous tensors")
 
@@ -60,8 +72,13 @@ def _prepare_muon_input(
 ) -> torch.Tensor:
     """``momentum_buffer.lerp_(gradient, 1 - momentum)`` and then either
     ``lerp(gradient, momentum_buffer, momentum)`` (Nesterov) or a copy of the
-    buffer into ``out``; one fused launch."""
-    _require_bf16_gpu(gradient, momentum_buffer, out)
+    buffer into ``out``; one fused launch.  Gradient and momentum buffer are
+    both bf16 or both fp32; ``out`` is the bf16 tensor the orthogonalization
+    reads (the reference casts its input to bf16 as its first step)."""
+    _require_master_gpu(gradient, momentum_buffer)
+    _require_bf16_gpu(out)
+    if gradient.dtype != momentum_buffer.dtype:
+        raise ValueError(f"gradient {gradient.dtype} and momentum buffer {momentum_buffer.dtype} differ in dtype")
     hip_ops.muon_prepare(momentum_buffer, gradient, out, momentum=momentum, nesterov=nesterov)
     return out
 
@@ -127,15 +144,18 @@ def _apply_muon_update(
     compute_matrix_shape: Sequence[int],
 ) -> torch.Tensor:
     """``parameter *= 1 - lr*weight_decay; parameter += -adjusted_lr * direction``
-    with a bf16 rounding after each, in one launch."""
-    _require_bf16_gpu(parameter, direction)
+    in one launch: with a bf16 rounding after each on a bf16 parameter, in
+    fp32 on an fp32 one.  ``direction`` is the bf16 orthogonalized matrix."""
+    _require_master_gpu(parameter)
+    _require_bf16_gpu(direction)
     adjusted = _adjust_muon_learning_rate(lr, adjust_lr_fn, compute_matrix_shape)
     hip_ops.muon_apply(parameter, direction, decay_factor=1 - lr * weight_decay, neg_adjusted_lr=-adjusted)
     return parameter
 
 
 class OwnedMuon:
-    """Muon over whole bf16 matrices owned by this rank.
+    """Muon over whole bf16 or fp32 matrices owned by this rank (momentum
+    buffers in the parameter's dtype, gradients too).
 
     Defaults follow the reference (dist_muon/optimizer.py:205-222): lr 1e-3,
     weight decay 0.1, momentum 0.95, Nesterov, 5 Newton-Schulz steps with the
@@ -162,13 +182,13 @@ class OwnedMuon:
         for p in self.params:
             if p.ndim != 2:
                 raise ValueError(f"Muon updates whole matrices; got a parameter of shape {tuple(p.shape)}")
-        _require_bf16_gpu(*self.params)
+        _require_master_gpu(*self.params)
         self.lr, self.weight_decay, self.momentum, self.nesterov = lr, weight_decay, momentum, nesterov
         self.ns_coefficients, self.ns_steps, self.eps, self.adjust_lr_fn = ns_coefficients, ns_steps, eps, adjust_lr_fn
         self.momentum_buffers = [torch.zeros_like(p) for p in self.params]
         # Matrices of one shape are orthogonalized as one batch; the step's
         # launch tables (address tables, batch buffers, workspaces) are built once.
-        self._groups: dict[tuple[int, int], list[int]] = {}
+        self._groups: dict[tuple[int, int, torch.dtype], list[int]] = {}  # (rows, cols, dtype) -> parameter indices
         # Matrices whose rows or columns are not multiples of 8 (the batched
         # step's 16-byte rows) take the per-matrix kernels, padded inside
         # the orthogonalization.
@@ -177,14 +197,14 @@ class OwnedMuon:
             if p.shape[0] % 8 or p.shape[1] % 8:
                 self._odd.append(index)
             else:
-                self._groups.setdefault(tuple(p.shape), []).append(index)
+                self._groups.setdefault((*p.shape, p.dtype), []).append(index)
         self._plan = None
         if self._groups:
             self._plan = hip_ops.MuonStepPlan(
                 [
                     # whole parameters are their own learning-rate reference shape: direction scale 1
-                    (shape, len(members), -_adjust_muon_learning_rate(lr, adjust_lr_fn, shape), 1.0)
-                    for shape, members in self._groups.items()
+                    (key[:2], len(members), -_adjust_muon_learning_rate(lr, adjust_lr_fn, key[:2]), 1.0, key[2])
+                    for key, members in self._groups.items()
                 ],
                 self.params[0].device,
             )
@@ -202,9 +222,11 @@ class OwnedMuon:
         if missing:
             raise RuntimeError(f"Muon parameters {missing} have no gradient; no parameter was updated")
         for p, g in zip(self.params, grads):
-            if g.shape != p.shape:
-                raise ValueError(f"gradient shape {tuple(g.shape)} does not match parameter {tuple(p.shape)}")
-        _require_bf16_gpu(*grads)
+            if g.shape != p.shape or g.dtype != p.dtype:
+                raise ValueError(
+                    f"gradient {tuple(g.shape)} {g.dtype} does not match parameter {tuple(p.shape)} {p.dtype}"
+                )
+        _require_master_gpu(*grads)
         # One C call: per shape group a momentum launch over all its matrices
         # (which also leaves the sums of squares the normalization needs),
         # Newton-Schulz with every product issued for all groups together, and
@@ -213,7 +235,8 @@ class OwnedMuon:
         for index in self._odd:
             p, g = self.params[index], grads[index]
             direction = _prepare_muon_input(
-                g, self.momentum_buffers[index], momentum=self.momentum, nesterov=self.nesterov, out=torch.empty_like(p)
+                g, self.momentum_buffers[index], momentum=self.momentum, nesterov=self.nesterov,
+                out=torch.empty(p.shape, dtype=torch.bfloat16, device=p.device),
             )
             _compute_muon_direction(direction, ns_coefficients=self.ns_coefficients, ns_steps=self.ns_steps, eps=self.eps)
             _apply_muon_update(
@@ -233,5 +256,5 @@ class OwnedMuon:
             # lr and adjust_lr_fn are read on every step, like the weight decay
             # beside them: a scheduler that changes opt.lr moves both halves of
             # the update together.
-            neg_adjusted_lrs=[-_adjust_muon_learning_rate(self.lr, self.adjust_lr_fn, shape) for shape in self._groups],
+            neg_adjusted_lrs=[-_adjust_muon_learning_rate(self.lr, self.adjust_lr_fn, key[:2]) for key in self._groups],
         )

@@ -687,33 +687,49 @@ def fp8_gemm_1x128_128x1(
     return out
 
 
+def _muon_master_dtype(who: str, masters: Sequence[torch.Tensor], bf16: Sequence[torch.Tensor]) -> torch.dtype:
+    """The dtype of the master tensors of a Muon elementwise step (all bf16 or
+    all fp32, contiguous, of equal numel with the bf16 operands)."""
+    dtype, numel = masters[0].dtype, masters[0].numel()
+    if dtype not in (torch.bfloat16, torch.float32):
+        raise NotImplementedError(f"{who} takes bf16 or fp32 master tensors, got {dtype}")
+    for t in masters:
+        if t.dtype != dtype or not t.is_contiguous() or t.numel() != numel:
+            raise ValueError(f"{who} needs contiguous tensors of one dtype and equal numel")
+    for t in bf16:
+        if t.dtype != torch.bfloat16 or not t.is_contiguous() or t.numel() != numel:
+            raise ValueError(f"{who} needs a contiguous bf16 Newton-Schulz operand of the same numel")
+    return dtype
+
+
 def muon_prepare(
     momentum_buffer: torch.Tensor, grad: torch.Tensor, out: torch.Tensor, *, momentum: float, nesterov: bool
 ) -> None:
+    """Momentum update and the input of the orthogonalization.  ``momentum_buffer``
+    and ``grad`` are both bf16 or both fp32; ``out`` is bf16."""
     _require_gpu(momentum_buffer, grad, out)
-    for t in (momentum_buffer, grad, out):
-        if t.dtype != torch.bfloat16 or not t.is_contiguous() or t.numel() != grad.numel():
-            raise ValueError("muon_prepare needs contiguous bf16 tensors of equal numel")
-    status = _native.lib().fsh_muon_prepare(
+    dtype = _muon_master_dtype("muon_prepare", (momentum_buffer, grad), (out,))
+    entry = "fsh_muon_prepare" if dtype == torch.bfloat16 else "fsh_muon_prepare_f32"
+    status = getattr(_native.lib(), entry)(
         momentum_buffer.data_ptr(), grad.data_ptr(), out.data_ptr(), grad.numel(), 1 - momentum, momentum,
         int(nesterov), stream_ptr(grad.device),
     )
-    _native.check(status, "fsh_muon_prepare")
+    _native.check(status, entry)
 
 
 def muon_apply(
     param: torch.Tensor, direction: torch.Tensor, *, decay_factor: float, neg_adjusted_lr: float,
     direction_scale: float = 1.0,
 ) -> None:
+    """Decayed update of a bf16 or fp32 ``param`` by the bf16 ``direction``."""
     _require_gpu(param, direction)
-    for t in (param, direction):
-        if t.dtype != torch.bfloat16 or not t.is_contiguous() or t.numel() != param.numel():
-            raise ValueError("muon_apply needs contiguous bf16 tensors of equal numel")
-    status = _native.lib().fsh_muon_apply(
+    dtype = _muon_master_dtype("muon_apply", (param,), (direction,))
+    entry = "fsh_muon_apply" if dtype == torch.bfloat16 else "fsh_muon_apply_f32"
+    status = getattr(_native.lib(), entry)(
         param.data_ptr(), direction.data_ptr(), param.numel(), decay_factor, neg_adjusted_lr, direction_scale,
         stream_ptr(param.device),
     )
-    _native.check(status, "fsh_muon_apply")
+    _native.check(status, entry)
 
 
 class MuonStepPlan:
@@ -724,9 +740,10 @@ class MuonStepPlan:
     re-uploaded only when a tensor moved (gradients usually do, parameters and
     momentum buffers usually do not)."""
 
-    def __init__(self, groups: Sequence[tuple[tuple[int, int], int, float, float]], device: torch.device) -> None:
-        """``groups``: per shape group (shape, matrix count, neg_adjusted_lr,
-        direction_scale)."""
+    def __init__(self, groups: Sequence[tuple], device: torch.device) -> None:
+        """``groups``: per group (shape, matrix count, neg_adjusted_lr,
+        direction_scale[, master dtype]); the master dtype (of parameters,
+        gradients and momentum buffers) is bf16 when left out, or fp32."""
         if not groups:
             raise ValueError("a Muon step needs at least one group")
         if len(groups) > _native.MAX_NS_PROBLEMS:
@@ -736,10 +753,14 @@ class MuonStepPlan:
         self._device = device
         self._table = (_native.MuonGroup * len(groups))()
         self._shapes: list[tuple[int, int]] = []
+        self._dtypes: list[torch.dtype] = []
         self._address_tables: list[list[tuple[torch.Tensor, list[int]]]] = []
         self.batches: list[torch.Tensor] = []
         self.workspaces: list[torch.Tensor] = []
-        for slot, (shape, n, neg_lr, scale) in zip(self._table, groups):
+        for slot, (shape, n, neg_lr, scale, *rest) in zip(self._table, groups):
+            master = rest[0] if rest else torch.bfloat16
+            if master not in (torch.bfloat16, torch.float32):
+                raise NotImplementedError(f"Muon master tensors are bf16 or fp32, got {master}")
             if len(shape) != 2 or shape[0] % 8 or shape[1] % 8 or n <= 0:
                 raise NotImplementedError(f"whole matrices with rows and cols multiples of 8, got {n} x {tuple(shape)}")
             batch = torch.empty((n, *shape), dtype=torch.bfloat16, device=device)
@@ -748,21 +769,23 @@ class MuonStepPlan:
             self.batches.append(batch)
             self.workspaces.append(workspace)
             self._shapes.append(tuple(shape))
+            self._dtypes.append(master)
+            slot.master_dtype = DT_BF16 if master == torch.bfloat16 else DT_F32
             self._address_tables.append(tables)
             slot.param_ptrs_dev, slot.momentum_ptrs_dev, slot.grad_ptrs_dev = (t.data_ptr() for t, _ in tables)
             slot.batch_dev, slot.batch, slot.rows, slot.cols = batch.data_ptr(), n, shape[0], shape[1]
             slot.workspace_dev, slot.workspace_nbytes = workspace.data_ptr(), workspace.numel()
             slot.neg_adjusted_lr, slot.direction_scale = neg_lr, scale
 
-    def _refresh(self, table: torch.Tensor, current: list[int], tensors: Sequence[torch.Tensor], shape) -> None:
+    def _refresh(self, table: torch.Tensor, current: list[int], tensors: Sequence[torch.Tensor], shape, dtype) -> None:
         if len(tensors) != len(current):
             raise ValueError(f"expected {len(current)} matrices of shape {shape}, got {len(tensors)}")
         addresses = []
         for t in tensors:
             if t.device != self._device:
                 raise ValueError(f"all matrices of a Muon step must live on {self._device}, got {t.device}")
-            if t.dtype != torch.bfloat16 or not t.is_contiguous() or tuple(t.shape) != shape:
-                raise ValueError(f"the Muon step kernels need contiguous bf16 matrices of shape {shape}")
+            if t.dtype != dtype or not t.is_contiguous() or tuple(t.shape) != shape:
+                raise ValueError(f"the Muon step kernels need contiguous {dtype} matrices of shape {shape}")
             if t.data_ptr() % 16:
                 raise ValueError("the Muon step kernels need 16-byte aligned matrices")
             addresses.append(t.data_ptr())
@@ -796,9 +819,9 @@ class MuonStepPlan:
         for name, lists in (("parameter", params), ("momentum", momenta), ("gradient", grads)):
             if len(lists) != len(self._shapes):
                 raise ValueError(f"expected {name} lists for {len(self._shapes)} groups, got {len(lists)}")
-        for tables, shape, p, m, g in zip(self._address_tables, self._shapes, params, momenta, grads):
+        for tables, shape, dtype, p, m, g in zip(self._address_tables, self._shapes, self._dtypes, params, momenta, grads):
             for (table, current), tensors in zip(tables, (p, m, g)):
-                self._refresh(table, current, tensors, shape)
+                self._refresh(table, current, tensors, shape, dtype)
         a, b, c = coefficients
         status = _native.lib().fsh_muon_step(
             self._table, len(self._shapes), lerp_weight, nesterov_weight, 1 if nesterov else 0, decay_factor, a, b, c,

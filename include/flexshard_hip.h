@@ -289,6 +289,16 @@ int fsh_muon_prepare(void* momentum_dev, const void* grad_dev, void* out_dev, in
                      int32_t nesterov, void* stream);
 int fsh_muon_apply(void* param_dev, const void* direction_dev, int64_t numel, float decay_factor,
                    float neg_adjusted_lr, float direction_scale, void* stream);
+/* The same two steps of the same reference lines on fp32 master state (fp32
+ * gradient, momentum buffer and parameter, as the reference's own optimizer
+ * tests use): the momentum and the parameter are updated in fp32 with no
+ * intermediate rounding; `out` is the bf16 input of the orthogonalization
+ * (the cast of dist_muon/optimizer.py:2131), `direction` its bf16 result,
+ * scaled in fp32 when direction_scale != 1 (:2093-2096 on an fp32 buffer). */
+int fsh_muon_prepare_f32(float* momentum_dev, const float* grad_dev, void* out_bf16_dev, int64_t numel,
+                         float lerp_weight, float nesterov_weight, int32_t nesterov, void* stream);
+int fsh_muon_apply_f32(float* param_dev, const void* direction_bf16_dev, int64_t numel, float decay_factor,
+                       float neg_adjusted_lr, float direction_scale, void* stream);
 
 /* ------------------------------------------------------------------------
  * 8. Forward product of a linear layer with a prequantized weight.
@@ -394,7 +404,11 @@ int fsh_fp8_gemm_1x128_128x1(const void* aq_dev, const float* as_dev, const void
  * written); other groups get one update launch.
  * The parameters, gradients and momentum buffers of a group are separate
  * allocations, named by device tables of their addresses; each must be a
- * contiguous bf16 [rows, cols] matrix at a 16-byte aligned address.
+ * contiguous [rows, cols] matrix of the group's master_dtype at a 16-byte
+ * aligned address.  With fp32 masters the momentum buffers and parameters
+ * are updated in fp32 (fsh_muon_prepare_f32 / fsh_muon_apply_f32, same bits),
+ * only the Newton-Schulz input is rounded to bf16, and the update is always a
+ * separate launch.
  * batch_dev is scratch of batch*rows*cols bf16: it holds the momentum
  * output and, for groups updated by a separate launch, the orthogonalized
  * direction afterwards (its contents after the call are otherwise unspecified).
@@ -415,6 +429,8 @@ typedef struct fsh_muon_group {
   int64_t workspace_nbytes;
   float neg_adjusted_lr;            /* -lr * shape factor of dist_muon/optimizer.py:2031-2046  */
   float direction_scale;            /* 1, or ratio / reference_ratio of :2082-2097             */
+  int32_t master_dtype;             /* FSH_DT_BF16 or FSH_DT_F32: parameters, gradients, momentum */
+  int32_t reserved;
 } fsh_muon_group;
 int fsh_muon_step(const fsh_muon_group* groups, int32_t count, float lerp_weight /* 1 - mu */,
                   float nesterov_weight /* mu */, int32_t nesterov, float decay_factor /* 1 - lr*wd */, float a,

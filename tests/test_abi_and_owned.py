@@ -38,13 +38,15 @@ def test_library_exports_every_declared_symbol():
     assert sorted(_native.SIGNATURES) == declared
     lib = _native.lib()
     assert lib.fsh_version() >= 1
-    assert lib.fsh_last_error() == b""
+    assert isinstance(lib.fsh_last_error(), bytes)  # empty until a call of this thread has failed
 
 
 def test_struct_sizes_match_the_header():
     assert ctypes.sizeof(_native.QuantChunk) == 56
     assert ctypes.sizeof(_native.UnpackChunk) == 56
     assert ctypes.sizeof(_native.GemmDesc) == 5 * 8 + 14 * 8 + 2 * 4 + 2 * 4 + 2 * 4
+    assert ctypes.sizeof(_native.MuonGroup) == 9 * 8 + 2 * 4 + 2 * 4
+    assert ctypes.sizeof(_native.NsProblem) == 6 * 8
 
 
 def test_host_side_argument_checks_need_no_gpu():

@@ -18,6 +18,7 @@ from flex_shard_amd.custom_placements.utils import gradient_reduce_plan, reduce_
 from flex_shard_amd.dist_muon import (
     OwnedMuon,
     _apply_muon_update,
+    _compute_muon_direction,
     _estimate_muon_compute_cost,
     _prepare_muon_input,
     _zeropower_via_newtonschulz,
@@ -765,6 +766,93 @@ def test_owned_muon_step_matches_torch_optim_muon(device, golden):
     assert all(torch.equal(a, b) for a, b in zip(mine, before))
 
 
+
+def test_muon_elementwise_kernels_on_fp32_masters(device):
+    """fp32 gradient, momentum buffer and parameter (the dtype of the
+    reference's own optimizer tests): the momentum and the parameter are
+    updated in fp32, bit for bit the interpolation and the decayed update
+    written as separate fp32 multiplies and adds, and within an fp32 ulp of the
+    operands of torch.lerp / mul_ / add_ (which may fuse a multiply-add); the
+    orthogonalization's bf16 input is the one rounding of the fp32 blend."""
+    gen = torch.Generator().manual_seed(16)
+    n = 100003
+    grad = torch.randn(n, generator=gen)
+    mom = torch.randn(n, generator=gen) * 0.1
+
+    def lerp(start, end, w):  # torch.lerp's two branches, every operation rounded on its own
+        diff = end - start
+        w32 = torch.tensor(w, dtype=torch.float32)  # the weight and 1 - weight are fp32 values
+        return start + w32 * diff if w < 0.5 else end - diff * (1 - w32)
+
+    for nesterov in (True, False):
+        m_gpu, out = mom.to(device), torch.empty(n, dtype=torch.bfloat16, device=device)
+        _prepare_muon_input(grad.to(device), m_gpu, momentum=0.95, nesterov=nesterov, out=out)
+        w_small = torch.tensor(1 - 0.95, dtype=torch.float32)
+        m_ref = mom + w_small * (grad - mom)
+        u_ref = lerp(grad, m_ref, 0.95) if nesterov else m_ref
+        assert torch.equal(m_gpu.cpu(), m_ref)
+        assert torch.equal(out.cpu(), u_ref.bfloat16())
+        m_torch = mom.clone().lerp_(grad, 1 - 0.95)
+        assert torch.allclose(m_gpu.cpu(), m_torch, rtol=1e-6, atol=1e-6)  # a fused multiply-add moves an fp32 ulp of the operands
+        o_torch = (torch.lerp(grad, m_torch, 0.95) if nesterov else m_torch).bfloat16()
+        assert (out.cpu() != o_torch).float().mean() < 1e-3
+    p = torch.randn(n, generator=gen) * 0.02
+    d = torch.randn(n, generator=gen).bfloat16()
+    alpha = -eager.adjusted_lr(1e-3, None, (7168, 2048))
+    for scale in (1.0, 0.5303300858899106):
+        p_gpu = p.to(device)
+        hip_ops.muon_apply(p_gpu, d.to(device), decay_factor=1 - 1e-3 * 0.1, neg_adjusted_lr=alpha, direction_scale=scale)
+        f32 = lambda v: torch.tensor(v, dtype=torch.float32)
+        dd = d.float() if scale == 1.0 else d.float() * f32(scale)
+        want = p * f32(1 - 1e-3 * 0.1) + f32(alpha) * dd
+        assert torch.equal(p_gpu.cpu(), want)
+        p_torch = p.clone().mul_(1 - 1e-3 * 0.1).add_(dd, alpha=alpha)
+        assert torch.allclose(p_gpu.cpu(), p_torch, rtol=1e-6, atol=1e-6)
+    with pytest.raises(ValueError, match="differ in dtype"):
+        _prepare_muon_input(grad.to(device), mom.bfloat16().to(device), momentum=0.95, nesterov=True,
+                            out=torch.empty(n, dtype=torch.bfloat16, device=device))
+
+
+def test_owned_muon_on_fp32_masters_matches_torch_optim_muon(device, golden):
+    """Three steps on fp32 whole matrices (two shapes for the batched step,
+    one whose sides are not multiples of 8 for the per-matrix path, and a bf16
+    parameter beside them) against torch.optim.Muon on the host; the batched
+    step gives the bits of the per-matrix kernels."""
+    tol = golden["muon_tolerance"]["atol"]
+    gen = torch.Generator().manual_seed(17)
+    shapes = [(256, 128), (128, 128), (256, 128), (100, 36), (128, 128)]
+    dtypes = [torch.float32, torch.float32, torch.float32, torch.float32, torch.bfloat16]
+    start = [(torch.randn(s, generator=gen) * 0.02).to(dt) for s, dt in zip(shapes, dtypes)]
+    mine = [p.clone().to(device) for p in start]
+    by_hand = [p.clone().to(device) for p in start]
+    hand_momentum = [torch.zeros_like(p) for p in by_hand]
+    theirs = [nn.Parameter(p.clone()) for p in start]
+    opt_mine = OwnedMuon(mine)
+    assert all(m.dtype == p.dtype for m, p in zip(opt_mine.momentum_buffers, mine))
+    opt_theirs = torch.optim.Muon(theirs, lr=1e-3, weight_decay=0.1, momentum=0.95, nesterov=True)
+    for _ in range(3):
+        grads = [torch.randn(s, generator=gen).to(dt) for s, dt in zip(shapes, dtypes)]
+        opt_mine.step([g.to(device) for g in grads])
+        for p, m, g in zip(by_hand, hand_momentum, grads):
+            direction = _prepare_muon_input(g.to(device), m, momentum=0.95, nesterov=True,
+                                            out=torch.empty(p.shape, dtype=torch.bfloat16, device=device))
+            _compute_muon_direction(direction)
+            _apply_muon_update(p, direction, lr=1e-3, weight_decay=0.1, adjust_lr_fn=None, compute_matrix_shape=p.shape)
+        for p, g in zip(theirs, grads):
+            p.grad = g.clone()
+        opt_theirs.step()
+    for a, h, b in zip(mine, by_hand, theirs):
+        assert torch.equal(a, h)
+        assert (a.cpu().float() - b.detach().float()).abs().max().item() <= tol
+        assert torch.allclose(a.cpu().float(), b.detach().float(), atol=1e-3)
+    for m, h in zip(opt_mine.momentum_buffers, hand_momentum):
+        assert torch.equal(m, h)
+    with pytest.raises(ValueError, match="does not match parameter"):
+        opt_mine.step([torch.zeros_like(p).bfloat16() if p.dtype == torch.float32 else torch.zeros_like(p) for p in mine])
+    with pytest.raises(NotImplementedError, match="bf16 or fp32"):
+        OwnedMuon([torch.zeros(8, 8, dtype=torch.float16, device=device)])
+
+
 # ------------------------------------------- config 5 at the benchmarked size
 CONFIG5_SHAPES = [(7168, 2048)] * 24 + [(2048, 2048)] * 24
 
@@ -818,17 +906,17 @@ def test_owned_muon_step_config5_matches_reference_step(device, golden):
     # The step applies the update from the last product's epilogue and never
     # stores the direction; the same kernels give it here for the comparison.
     batches = {
-        shape: torch.stack([
+        key[:2]: torch.stack([
             _prepare_muon_input(grads[i], torch.zeros_like(grads[i]), momentum=0.95, nesterov=True,
                                 out=torch.empty_like(grads[i]))
             for i in members
         ])
-        for shape, members in opt._groups.items()
+        for key, members in opt._groups.items()
     }
     hip_ops.newton_schulz_multi([(b, None) for b in batches.values()], COEFFS, 5, 1e-7)
     for i in checked:
         shape = CONFIG5_SHAPES[i]
-        slot = opt._groups[shape].index(i)
+        slot = opt._groups[(*shape, torch.bfloat16)].index(i)
         direction = batches[shape][slot].cpu()
         momentum = torch.zeros(shape, dtype=torch.bfloat16)
         g = grads[i].cpu()
