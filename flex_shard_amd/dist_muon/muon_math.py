@@ -155,7 +155,8 @@ def _apply_muon_update(
 
 class OwnedMuon:
     """Muon over whole bf16 or fp32 matrices owned by this rank (momentum
-    buffers in the parameter's dtype, gradients too).
+    buffers in the parameter's dtype, gradients too); a parameter with leading
+    dimensions is a batch of matrices.
 
     Defaults follow the reference (dist_muon/optimizer.py:205-222): lr 1e-3,
     weight decay 0.1, momentum 0.95, Nesterov, 5 Newton-Schulz steps with the
@@ -180,24 +181,30 @@ class OwnedMuon:
         if not self.params:
             raise ValueError("OwnedMuon needs at least one parameter")
         for p in self.params:
-            if p.ndim != 2:
-                raise ValueError(f"Muon updates whole matrices; got a parameter of shape {tuple(p.shape)}")
+            if p.ndim < 2:
+                raise ValueError(f"Muon updates matrices; got a parameter of shape {tuple(p.shape)}")
         _require_master_gpu(*self.params)
         self.lr, self.weight_decay, self.momentum, self.nesterov = lr, weight_decay, momentum, nesterov
         self.ns_coefficients, self.ns_steps, self.eps, self.adjust_lr_fn = ns_coefficients, ns_steps, eps, adjust_lr_fn
         self.momentum_buffers = [torch.zeros_like(p) for p in self.params]
-        # Matrices of one shape are orthogonalized as one batch; the step's
+        # A parameter with leading dimensions ([experts, rows, cols]) is a
+        # batch of independent matrices (the reference views it as one,
+        # dist_muon/optimizer.py:2082-2091): the step works on 2-D views.
+        self._matrix_counts = [math.prod(p.shape[:-2]) for p in self.params]
+        self._matrices = self._as_matrices(self.params)
+        self._momentum_matrices = self._as_matrices(self.momentum_buffers)
+        # Matrices of one shape and dtype are orthogonalized as one batch; the step's
         # launch tables (address tables, batch buffers, workspaces) are built once.
-        self._groups: dict[tuple[int, int, torch.dtype], list[int]] = {}  # (rows, cols, dtype) -> parameter indices
+        self._groups: dict[tuple[int, int, torch.dtype], list[int]] = {}  # (rows, cols, dtype) -> matrix indices
         # Matrices whose rows or columns are not multiples of 8 (the batched
         # step's 16-byte rows) take the per-matrix kernels, padded inside
         # the orthogonalization.
         self._odd: list[int] = []
-        for index, p in enumerate(self.params):
-            if p.shape[0] % 8 or p.shape[1] % 8:
+        for index, m in enumerate(self._matrices):
+            if m.shape[0] % 8 or m.shape[1] % 8:
                 self._odd.append(index)
             else:
-                self._groups.setdefault((*p.shape, p.dtype), []).append(index)
+                self._groups.setdefault((*m.shape, m.dtype), []).append(index)
         self._plan = None
         if self._groups:
             self._plan = hip_ops.MuonStepPlan(
@@ -210,6 +217,14 @@ class OwnedMuon:
             )
             self._batch = dict(zip(self._groups, self._plan.batches))
             self._workspace = dict(zip(self._groups, self._plan.workspaces))
+
+    @staticmethod
+    def _as_matrices(tensors: Sequence[torch.Tensor]) -> list[torch.Tensor]:
+        """The 2-D matrices of the tensors, in order, as views."""
+        matrices = []
+        for t in tensors:
+            matrices.extend(t.view(-1, *t.shape[-2:]).unbind(0) if t.ndim > 2 else (t,))
+        return matrices
 
     def flops_per_step(self) -> int:
         return 2 * sum(_estimate_muon_compute_cost(tuple(p.shape), self.ns_steps) for p in self.params)
@@ -232,10 +247,11 @@ class OwnedMuon:
         # Newton-Schulz with every product issued for all groups together, and
         # an update launch per group.  Same bits as _prepare_muon_input ->
         # _compute_muon_direction -> _apply_muon_update per matrix.
+        grad_matrices = self._as_matrices(grads)
         for index in self._odd:
-            p, g = self.params[index], grads[index]
+            p, g = self._matrices[index], grad_matrices[index]
             direction = _prepare_muon_input(
-                g, self.momentum_buffers[index], momentum=self.momentum, nesterov=self.nesterov,
+                g, self._momentum_matrices[index], momentum=self.momentum, nesterov=self.nesterov,
                 out=torch.empty(p.shape, dtype=torch.bfloat16, device=p.device),
             )
             _compute_muon_direction(direction, ns_coefficients=self.ns_coefficients, ns_steps=self.ns_steps, eps=self.eps)
@@ -247,9 +263,9 @@ class OwnedMuon:
             return
         members = list(self._groups.values())
         self._plan.step(
-            [[self.params[i] for i in group] for group in members],
-            [[self.momentum_buffers[i] for i in group] for group in members],
-            [[grads[i] for i in group] for group in members],
+            [[self._matrices[i] for i in group] for group in members],
+            [[self._momentum_matrices[i] for i in group] for group in members],
+            [[grad_matrices[i] for i in group] for group in members],
             lerp_weight=1 - self.momentum, nesterov_weight=self.momentum, nesterov=self.nesterov,
             decay_factor=1 - self.lr * self.weight_decay, coefficients=self.ns_coefficients, steps=self.ns_steps,
             eps=self.eps,

@@ -853,6 +853,40 @@ def test_owned_muon_on_fp32_masters_matches_torch_optim_muon(device, golden):
         OwnedMuon([torch.zeros(8, 8, dtype=torch.float16, device=device)])
 
 
+
+def test_owned_muon_takes_stacked_parameters_as_batches_of_matrices(device, golden):
+    """A parameter with leading dimensions ([experts, rows, cols]) is updated
+    as its matrices would be on their own (dist_muon/optimizer.py:2082-2091
+    views it as a batch): same bits as an optimizer over the unbound
+    matrices, for the batched step and for the per-matrix path of shapes that
+    are not multiples of 8, and within the reference's bar of its step in
+    eager torch on the host."""
+    tol = golden["muon_tolerance"]["atol"]
+    gen = torch.Generator().manual_seed(19)
+    shapes = [(3, 64, 128), (2, 100, 36), (128, 64), (2, 2, 64, 128)]
+    dtypes = [torch.float32, torch.bfloat16, torch.bfloat16, torch.bfloat16]
+    start = [(torch.randn(s, generator=gen) * 0.02).to(dt) for s, dt in zip(shapes, dtypes)]
+    stacked = [p.clone().to(device) for p in start]
+    separate = [m.clone() for p in start for m in p.to(device).reshape(-1, *p.shape[-2:]).unbind(0)]
+    host = [m.clone() for p in start for m in p.reshape(-1, *p.shape[-2:]).unbind(0)]
+    host_momentum = [torch.zeros_like(m) for m in host]
+    opt_stacked, opt_separate = OwnedMuon(stacked, adjust_lr_fn="match_rms_adamw"), OwnedMuon(separate, adjust_lr_fn="match_rms_adamw")
+    assert opt_stacked.flops_per_step() == opt_separate.flops_per_step()
+    for _ in range(2):
+        grads = [torch.randn(s, generator=gen).to(dt) for s, dt in zip(shapes, dtypes)]
+        opt_stacked.step([g.to(device) for g in grads])
+        flat = [m.contiguous() for g in grads for m in g.reshape(-1, *g.shape[-2:]).unbind(0)]
+        opt_separate.step([g.to(device) for g in flat])
+        for p, g, m in zip(host, flat, host_momentum):
+            eager.muon_step(p, g, m, adjust_lr_fn="match_rms_adamw")
+    ours = [m for p in stacked for m in p.reshape(-1, *p.shape[-2:]).unbind(0)]
+    for a, b, c in zip(ours, separate, host, strict=True):
+        assert torch.equal(a, b)
+        assert (a.cpu().float() - c.float()).abs().max().item() <= tol
+    with pytest.raises(ValueError, match="Muon updates matrices"):
+        OwnedMuon([torch.zeros(64, device=device, dtype=torch.bfloat16)])
+
+
 # ------------------------------------------- config 5 at the benchmarked size
 CONFIG5_SHAPES = [(7168, 2048)] * 24 + [(2048, 2048)] * 24
 
