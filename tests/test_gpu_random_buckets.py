@@ -274,3 +274,64 @@ def test_random_shapes_of_the_three_fp8_products_are_integer_exact(device, seed)
     want = eager.fp8_gemm_1x128_128x1(aq, a_s, bq, b_s, out_dtype=torch.float32)
     got = hip_ops.fp8_gemm_1x128_128x1(aq.to(device), a_s.to(device), bq.to(device), b_s.to(device))
     assert torch.equal(got.cpu(), want.bfloat16()), ("weight gradient", m, n, k)
+
+
+# ------------------------------------------------------------ mixed bucket
+@pytest.mark.parametrize("seed", range(30))
+def test_random_mixed_bucket_unshard_and_gradients(device, seed):
+    """Random mixed buckets (Shard(0) vectors and matrices of random sizes in
+    random order around one or two blockwise FP8 matrices, so the FP8 payload
+    starts at odd offsets inside the rank rows): on every rank the Shard(0)
+    members come back as they were and the FP8 members as the oracle's
+    whole-matrix quantization; with every rank contributing the parameters
+    themselves as gradients, each rank's reduced gradient is the rank-order
+    fold of `world` copies of its own shard times 1 / world."""
+    from flex_shard_amd import GradientReduction
+    from oracle import eager
+    from tests.test_gpu_mixed_bucket import _bucket, _unshard_as
+
+    rng = np.random.default_rng(3000 + seed)
+    world = int(rng.choice([2, 3, 4]))
+    block = int(rng.choice([4, 8, 16]))
+    shapes = []
+    for index in range(int(rng.integers(1, 4))):
+        rows = world * int(rng.integers(1, 5))  # Shard(0) splits dim 0 evenly here
+        shape = (rows,) if rng.random() < 0.5 else (rows, int(rng.integers(1, 9)))
+        shapes.append((f"dense{index}", shape, "shard0"))
+    for index in range(int(rng.integers(1, 3))):
+        rows = int(rng.integers(1, 4)) * block + int(rng.integers(0, block))
+        cols = int(rng.integers(1, 4)) * block + int(rng.integers(0, block))
+        shapes.append((f"fp8_{index}", (max(rows, 1), max(cols, 1)), "fp8"))
+    shapes = [shapes[i] for i in rng.permutation(len(shapes))]
+    mixed, raw, member, factory, named, ranks = _bucket(device, world, block, shapes)
+    originals = {fqn: p.detach().clone() for fqn, p in named}
+    kinds = {fqn: kind for fqn, _, kind in shapes}
+    for rank in range(world):
+        factory.calls.clear()
+        _, result = _unshard_as(mixed, ranks, rank)
+        calls = iter(factory.calls)
+        for (fqn, _), full in zip(named, result.full_params, strict=True):
+            if kinds[fqn] == "shard0":
+                assert torch.equal(full, originals[fqn]), (rank, fqn)
+            else:
+                fp8, scale, orig_dtype, _ = next(calls)
+                want_q, want_s = eager.quantize_blockwise(originals[fqn].cpu(), block)
+                assert full is fp8 and orig_dtype == torch.bfloat16
+                assert torch.equal(fp8.view(torch.uint8).cpu(), want_q.view(torch.uint8)), (rank, fqn)
+                assert torch.equal(scale.cpu().view(torch.int32), want_s.view(torch.int32)), (rank, fqn)
+    reduce_inputs = []
+    for mesh, group, infos, _ in ranks:
+        grads = [originals[info.fqn].float() for info in infos]
+        reduce_inputs.append(mixed.prepare_reduce_grad(grads, infos, mesh, None))
+    for rank, (mesh, group, infos, shards) in enumerate(ranks):
+        for other, p in enumerate(reduce_inputs):
+            if other != rank:
+                group.deposit(other, p.buffers[0])
+        reduced = mixed.reduce_prepared_grad(reduce_inputs[rank], GradientReduction())
+        for grad, shard in zip(reduced.sharded_grads, shards, strict=True):
+            # the average of `world` equal contributions, folded in rank order as the reduction folds them
+            term = shard.float() * torch.tensor(1.0 / world, dtype=torch.float32)
+            want = term.clone()
+            for _ in range(world - 1):
+                want = want + term
+            assert grad.dtype == torch.float32 and torch.equal(grad, want), rank
