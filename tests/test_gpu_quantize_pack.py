@@ -262,6 +262,26 @@ def test_many_chunks_split_into_several_launches(device):
     assert torch.equal(prepared.buffers[0].cpu(), olayout.pack_rank_payload(lay, 0, list(qs), list(ss), 8))
 
 
+
+@pytest.mark.parametrize("nparams,world", [(7, 1), (8, 1), (12, 1), (24, 1), (25, 1), (40, 1), (30, 3)])
+def test_vector_kernel_with_many_chunks(device, nparams, world):
+    """bf16 shards on 128x128 tiles take the vector kernel, whose chunk lookup
+    comes in an 8-entry and a 24-entry form and which is launched once per 24
+    chunks: 7, 8, 12, 24, 25 and 40 parameters on one rank, and 30 over three
+    ranks, whole and partial tiles, against the oracle's naive pack."""
+    gen = torch.Generator().manual_seed(nparams * 10 + world)
+    shapes = [((128, 256), (256, 128), (130, 136), (384, 128), (64, 200))[i % 5] for i in range(nparams)]
+    params = [(torch.randn(s, generator=gen) * 0.02).bfloat16() for s in shapes]
+    named = [(f"w{i}", nn.Parameter(p.to(device), requires_grad=False)) for i, p in enumerate(params)]
+    pl = Fp8BucketedBlockShard(world_size=world, weight_factory=_factory)
+    prepared = prepare_unshard_on_each_rank(pl, named, world)
+    lay = olayout.quant_layout(shapes, 128, world)
+    qs, ss = zip(*[cport.quantize_blockwise(p, 128) for p in params])
+    for rank in range(world):
+        want = olayout.pack_rank_payload(lay, rank, list(qs), list(ss), 128)
+        assert torch.equal(prepared[rank].buffers[0].cpu(), want), f"rank {rank}"
+
+
 def test_payload_cache_forward_backward(device):
     """Forward always repacks; a backward graph task may take the cached
     payload back once; compiling bypasses the cache."""

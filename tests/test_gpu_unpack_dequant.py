@@ -304,6 +304,34 @@ def test_dequant_is_bit_exact_with_oracle(device, shape, block):
 
 
 
+
+@pytest.mark.parametrize("block,shapes", [
+    (128, [(256, 128), (130, 136), (384, 256), (128, 128)] * 18),
+    (4, [(16, 8), (9, 12), (8, 8), (5, 3), (12, 4)] * 15),
+])
+def test_fused_unpack_with_more_than_64_chunks(device, block, shapes):
+    """The tile-to-chunk lookup resolves up to 64 chunks with one ballot and
+    bisects beyond that: 72 and 75 parameters over 8 ranks (a chunk per
+    parameter and rank that holds rows of it: more than 64), compact bytes,
+    scales and dequantized values against the oracle."""
+    world = 8
+    factory = RecordingFactory()
+    pl = Fp8BucketedBlockShard(world_size=world, weight_factory=factory, block_size=block)
+    gen = torch.Generator().manual_seed(len(shapes) + block)
+    named = [(f"w{i}", nn.Parameter((torch.randn(s, generator=gen) * 0.02).bfloat16().to(device), requires_grad=False))
+             for i, s in enumerate(shapes)]
+    prepared = prepare_unshard_on_each_rank(pl, named, world)
+    rows = gather_rank_rows(prepared)
+    table, starts, total_tiles, _ = pl._unpack_table(pl._unshard_state(prepared[3]), rows.stride(0), rows.device)
+    assert table.shape[0] > 64
+    _, dequant = pl.finish_prepared_unshard_with_dequant(prepared[3], rows)
+    for (_, p), call, deq in zip(named, factory.calls, dequant, strict=True):
+        oq, osc = cport.quantize_blockwise(p.detach().cpu(), block)
+        assert torch.equal(call[0].view(torch.uint8).cpu(), oq) and torch.equal(_bits(call[1].cpu()), _bits(osc))
+        want = cport.dequant_blockwise(oq, osc, block)
+        assert torch.equal(deq.cpu().view(torch.int16), want.view(torch.int16))
+
+
 def test_fp16_bucket_round_trip_and_fp16_dequantization(device):
     """fp16 parameters through pack, gather and unpack on 4 ranks: the factory
     gets the oracle's bytes and scales with orig_dtype fp16, and the fused
