@@ -282,6 +282,36 @@ def test_vector_kernel_with_many_chunks(device, nparams, world):
         assert torch.equal(prepared[rank].buffers[0].cpu(), want), f"rank {rank}"
 
 
+
+@pytest.mark.parametrize("block", [128, 16])
+def test_large_pads_of_short_and_empty_ranks_are_zeroed(device, block):
+    """One wide single-block-row matrix next to a small one on 3 ranks: the
+    ranks that get little or nothing pad their payload up to the longest
+    rank's row, hundreds of KB of zeros written by several pad workgroups,
+    whatever the buffers held before."""
+    shapes = [(block, 300_000), (2 * block, block)]
+    gen = torch.Generator().manual_seed(block)
+    params = [(torch.randn(s, generator=gen) * 0.02).bfloat16() for s in shapes]
+    named = [(f"w{i}", nn.Parameter(p.to(device), requires_grad=False)) for i, p in enumerate(params)]
+    pl = Fp8BucketedBlockShard(world_size=3, weight_factory=_factory, block_size=block)
+    for _ in range(2):  # the second round takes recycled buffers that held the first round's payloads
+        junk = torch.full((64 << 20,), 0xAB, dtype=torch.uint8, device=device)
+        del junk
+        prepared = prepare_unshard_on_each_rank(pl, named, 3)
+        lay = olayout.quant_layout(shapes, block, 3)
+        qs, ss = zip(*[cport.quantize_blockwise(p, block) for p in params])
+        sizes = []
+        for rank in range(3):
+            want = olayout.pack_rank_payload(lay, rank, list(qs), list(ss), block)
+            got = prepared[rank].buffers[0].cpu()
+            assert torch.equal(got, want), f"rank {rank}"
+            sizes.append(int((want != 0).sum()))
+        assert min(sizes) < max(sizes) // 100  # some rank's row is nearly all padding
+        for p in prepared:
+            p.buffers[0].fill_(0xCD)  # poison what goes back to the recycled buffers
+        del prepared
+
+
 def test_payload_cache_forward_backward(device):
     """Forward always repacks; a backward graph task may take the cached
     payload back once; compiling bypasses the cache."""
