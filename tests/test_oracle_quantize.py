@@ -250,3 +250,28 @@ def test_quantize_dequantize_round_trip_error_bound():
     tiles = w.float().view(4, 16, 4, 16).abs().amax(dim=(1, 3))
     bound = tiles.repeat_interleave(16, 0).repeat_interleave(16, 1) / 16
     assert ((back - w.float()).abs() <= bound).all()
+
+
+@pytest.mark.parametrize("shape,block", [((12, 6), 4), ((130, 129), 128), ((64, 64), 16)])
+def test_eager_restatement_on_fp16_input(shape, block):
+    """What the reference's arithmetic gives on fp16: fp16 to fp32 is exact and
+    no nonzero fp16 amax lies under the 1e-12 floor, so every tile with a
+    nonzero amax equals the C quantization of the upcast values (pinned above);
+    the floor itself rounds to 0 in fp16, so an all-zero tile gets scale inf,
+    stored reciprocal 0 and NaN bytes (0 x inf)."""
+    gen = torch.Generator().manual_seed(shape[0] + block)
+    w = (torch.randn(shape, generator=gen) * 0.05).half()
+    w[0, 0], w[-1, -1] = 6.1e-5, 65504.0
+    q, s = eager.quantize_blockwise(w, block)
+    cq, cs = cport.quantize_blockwise(w.float(), block)
+    assert torch.equal(q.view(torch.uint8), cq) and torch.equal(s.view(torch.int32), cs.view(torch.int32))
+    assert torch.tensor(1e-12).half().item() == 0.0
+    w[:block, :block] = 0
+    q, s = eager.quantize_blockwise(w, block)
+    cq, cs = cport.quantize_blockwise(w.float(), block)
+    tile = torch.zeros(shape, dtype=torch.bool)
+    tile[:block, :block] = True
+    assert s[0, 0].item() == 0.0 and ((q.view(torch.uint8)[tile] & 0x7F) == 0x7F).all()
+    assert torch.equal(q.view(torch.uint8)[~tile], cq[~tile])
+    assert torch.equal(s.view(torch.int32).view(-1)[1:], cs.view(torch.int32).view(-1)[1:])
+    assert cs[0, 0].view(torch.int32).item() == 0x2720D7C5 and (cq[tile] == 0).all()  # the fp32 floor keeps the tile finite
