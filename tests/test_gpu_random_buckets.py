@@ -335,3 +335,97 @@ def test_random_mixed_bucket_unshard_and_gradients(device, seed):
             for _ in range(world - 1):
                 want = want + term
             assert grad.dtype == torch.float32 and torch.equal(grad, want), rank
+
+
+# ------------------------------------------------------------ runtime slice
+@pytest.mark.parametrize("seed", range(12))
+def test_random_layer_stacks_under_the_runtime_hooks(device, seed):
+    """2-4 FP8 linear layers of random widths, one bucket each, under the
+    runtime's hooks with or without prefetch of the next bucket, on one or two
+    unshard streams, 1-3 microbatches of which only the last syncs, for two
+    steps with an update of the shards in between: outputs, input gradients
+    and the reduced shard gradients equal the same kernels called directly on
+    one stream, bit for bit (a missing wait or a buffer reused too early would
+    show here)."""
+    from flex_shard_amd import LocalReduceGroup
+    from flex_shard_amd.blockwise_fp8 import (
+        BlockwiseFp8Weight,
+        Fp8BlockwiseGemms,
+        convert_to_flex_shard_float8_blockwise_linear,
+        make_blockwise_fp8_weight,
+    )
+    from flex_shard_amd.custom_placements.fp8_bucketed_block_shard import _quantize_dense_weight_to_blockwise_fp8
+    from flex_shard_amd.flex_shard import BucketCommContext, BucketRuntime
+
+    rng = np.random.default_rng(11000 + seed)
+    nlayers = int(rng.integers(2, 5))
+    widths = [int(rng.integers(1, 4)) * 128 for _ in range(nlayers + 1)]
+    tokens = int(rng.integers(1, 4)) * 64
+    prefetch = bool(rng.random() < 0.7)
+    streams = int(rng.integers(1, 3))
+    microbatches = int(rng.integers(1, 4))
+    gen = torch.Generator().manual_seed(seed)
+    model = nn.Sequential(*[nn.Linear(widths[i], widths[i + 1], bias=False) for i in range(nlayers)])
+    with torch.no_grad():
+        for p in model.parameters():
+            p.copy_(torch.randn(p.shape, generator=gen) * 0.05)
+    model = model.to(device=device, dtype=torch.bfloat16)
+    full = [p.detach().clone() for p in model.parameters()]
+    convert_to_flex_shard_float8_blockwise_linear(model)
+    context = BucketCommContext.create(device, unshard_streams=streams)
+    runtimes = []
+    for index in range(nlayers):
+        placement = Fp8BucketedBlockShard(world_size=1, weight_factory=make_blockwise_fp8_weight)
+        mesh = FakeMesh(1, 0, LocalReduceGroup(1, 0))
+        runtimes.append(BucketRuntime.shard_module_params(model, [f"{index}.weight"], placement, mesh, context))
+    for index, (layer, runtime) in enumerate(zip(model, runtimes)):
+        runtime.install_hooks(
+            layer,
+            forward_prefetch=runtimes[index + 1] if prefetch and index + 1 < nlayers else None,
+            backward_prefetch=runtimes[index - 1] if prefetch and index > 0 else None,
+        )
+
+    def direct(weights, x, grad_out):
+        gemms = Fp8BlockwiseGemms(128)
+        quantized = []
+        for w in weights:
+            q, s = _quantize_dense_weight_to_blockwise_fp8(w, 128, torch.float8_e4m3fn)
+            quantized.append(BlockwiseFp8Weight(q, s, 128))
+        acts = [x]
+        for w in quantized:
+            acts.append(gemms.forward(acts[-1], w))
+        grads, g = [None] * len(weights), grad_out
+        for i in reversed(range(len(weights))):
+            g, grads[i] = gemms.backward(g, acts[i], quantized[i], True, True)
+        return acts[-1], g, grads
+
+    scale = 1.0
+    for step in range(2):
+        if step:
+            scale = 0.5
+            with torch.no_grad():
+                for runtime in runtimes:
+                    for p in runtime.sharded_params:
+                        p.mul_(0.5)
+                        p.grad = None
+        weights = [w * scale for w in full]
+        xs = [torch.randn(tokens, widths[0], generator=gen).bfloat16().to(device).requires_grad_() for _ in range(microbatches)]
+        gos = [(torch.randn(tokens, widths[-1], generator=gen) * 0.01).bfloat16().to(device) for _ in range(microbatches)]
+        wants = [direct(weights, x.detach(), go) for x, go in zip(xs, gos)]
+        for k, (x, go) in enumerate(zip(xs, gos)):
+            last = k == microbatches - 1
+            for runtime in runtimes:
+                runtime.set_requires_gradient_sync(last)
+            out = model(x)
+            out.backward(go)
+            assert torch.equal(out.detach(), wants[k][0]), (step, k)
+            assert torch.equal(x.grad, wants[k][1]), (step, k)
+        context.wait_and_clear_reduce_grad_states()
+        for index, runtime in enumerate(runtimes):
+            total = None
+            for want in wants:  # microbatch gradients add up in fp32 in the order they arrive
+                total = want[2][index].float() if total is None else total + want[2][index].float()
+            (shard,) = runtime.sharded_params
+            assert torch.equal(shard.grad.view(total.shape), total.bfloat16()), (step, index)
+            assert not runtime.is_unsharded
+    torch.cuda.synchronize()
