@@ -150,6 +150,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     ),
     "fsh_accumulate_grad": (c_int, [c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p]),
     "fsh_reduce_rows_f32": (c_int, [c_void_p, c_void_p, c_int64, c_int32, c_int64, c_int64, c_int32, c_float, c_void_p]),
+    "fsh_reduce_rows_bf16": (c_int, [c_void_p, c_void_p, c_int64, c_int32, c_int64, c_int64, c_int32, c_float, c_void_p]),
     "fsh_newton_schulz_workspace_bytes": (c_int64, [c_int64, c_int64, c_int64]),
     "fsh_newton_schulz": (
         c_int,

@@ -114,6 +114,43 @@ __global__ __launch_bounds__(kThreads) void reduce_rows_kernel(float* __restrict
   }
 }
 
+// The same fold over bf16 contributions: every term is widened to fp32 (and
+// pre-multiplied if asked), the terms are added in fp32 in rank order, and the
+// result is rounded to bf16 once.
+template <int MODE>
+__global__ __launch_bounds__(kThreads) void reduce_rows_bf16_kernel(uint16_t* __restrict__ out,
+                                                                   const uint16_t* __restrict__ src,
+                                                                   int64_t stride, int world, int64_t n,
+                                                                   float factor, int vec_ok) {
+  const int64_t tid = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t nthreads = static_cast<int64_t>(gridDim.x) * kThreads;
+  int64_t done = 0;
+  if (vec_ok) {
+    const int64_t groups = n / 8;
+    for (int64_t gidx = tid; gidx < groups; gidx += nthreads) {
+      float s[8], v[8];
+      unpack8(load_stream_u32x4(src + gidx * 8), s);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s[j] = fold_term<MODE>(s[j], factor);
+      for (int r = 1; r < world; ++r) {
+        unpack8(load_stream_u32x4(src + r * stride + gidx * 8), v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s[j] = s[j] + fold_term<MODE>(v[j], factor);
+      }
+      uint32_t bits[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) bits[j] = f32_to_bf16_bits(fold_finish<MODE>(s[j], factor));
+      *reinterpret_cast<u32x4*>(out + gidx * 8) = pack8(bits);
+    }
+    done = groups * 8;
+  }
+  for (int64_t i = done + tid; i < n; i += nthreads) {
+    float s = fold_term<MODE>(bf16_bits_to_f32(src[i]), factor);
+    for (int r = 1; r < world; ++r) s = s + fold_term<MODE>(bf16_bits_to_f32(src[r * stride + i]), factor);
+    out[i] = static_cast<uint16_t>(f32_to_bf16_bits(fold_finish<MODE>(s, factor)));
+  }
+}
+
 // m = bf16(lerp(m, g, 1-mu)); out = nesterov ? bf16(lerp(g, m, mu)) : m.
 // 8 elements (16 bytes) per thread and iteration when the three pointers are
 // 16-byte aligned, then a scalar tail; scalar throughout otherwise.
@@ -353,4 +390,36 @@ FSH_API int fsh_muon_apply_f32(float* param_dev, const void* direction_dev, int6
                      static_cast<hipStream_t>(stream), param_dev, static_cast<const uint16_t*>(direction_dev), numel,
                      decay_factor, neg_adjusted_lr, direction_scale, vec_ok);
   return check_launch("fsh_muon_apply_f32");
+}
+
+FSH_API int fsh_reduce_rows_bf16(void* out_dev, const void* src_dev, int64_t contribution_stride, int32_t world,
+                                 int64_t column_offset, int64_t numel, int32_t mode, float factor, void* stream) {
+  using namespace fsh;
+  if (numel < 0 || world <= 0 || column_offset < 0 || contribution_stride < 0)
+    return fail(FSH_EINVAL, "fsh_reduce_rows_bf16: bad sizes (world %d, numel %lld)", world, (long long)numel);
+  if (numel == 0) return FSH_OK;
+  if (!out_dev || !src_dev) return fail(FSH_EINVAL, "fsh_reduce_rows_bf16: null pointer");
+  if (!aligned(out_dev, 2) || !aligned(src_dev, 2)) return fail(FSH_EINVAL, "fsh_reduce_rows_bf16: misaligned");
+  if (mode < FSH_REDUCE_SUM || mode > FSH_REDUCE_POSTDIV)
+    return fail(FSH_EINVAL, "fsh_reduce_rows_bf16: unknown mode %d", mode);
+  const uint16_t* src = static_cast<const uint16_t*>(src_dev) + column_offset;
+  uint16_t* out = static_cast<uint16_t*>(out_dev);
+  const int vec_ok = aligned(out, 16) && aligned(src, 16) && (contribution_stride % 8 == 0);
+  const dim3 g(grid_for(ceil_div(numel, 8))), b(kThreads);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (mode) {
+    case FSH_REDUCE_SUM:
+      hipLaunchKernelGGL((reduce_rows_bf16_kernel<FSH_REDUCE_SUM>), g, b, 0, s, out, src, contribution_stride, world, numel, factor, vec_ok);
+      break;
+    case FSH_REDUCE_PREMUL:
+      hipLaunchKernelGGL((reduce_rows_bf16_kernel<FSH_REDUCE_PREMUL>), g, b, 0, s, out, src, contribution_stride, world, numel, factor, vec_ok);
+      break;
+    case FSH_REDUCE_POSTMUL:
+      hipLaunchKernelGGL((reduce_rows_bf16_kernel<FSH_REDUCE_POSTMUL>), g, b, 0, s, out, src, contribution_stride, world, numel, factor, vec_ok);
+      break;
+    default:
+      hipLaunchKernelGGL((reduce_rows_bf16_kernel<FSH_REDUCE_POSTDIV>), g, b, 0, s, out, src, contribution_stride, world, numel, factor, vec_ok);
+      break;
+  }
+  return check_launch("fsh_reduce_rows_bf16");
 }

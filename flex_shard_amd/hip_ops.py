@@ -292,21 +292,26 @@ def reduce_rows(
     out: torch.Tensor, contributions: torch.Tensor, column_offset: int, *, mode: int = REDUCE_SUM, factor: float = 1.0
 ) -> None:
     """``out[i] = fold_r contributions[r, column_offset + i]`` in rank order;
-    ``contributions`` is fp32 [W, row] with unit column stride."""
+    ``contributions`` is [W, row] with unit column stride, fp32 or bf16 like
+    ``out`` (bf16 terms are added in fp32 and the sum rounded once)."""
     _require_gpu(out, contributions)
-    if out.dtype != torch.float32 or contributions.dtype != torch.float32:
-        raise NotImplementedError("the fixed-order reduction is implemented for fp32 gradients")
+    if out.dtype != contributions.dtype or out.dtype not in (torch.float32, torch.bfloat16):
+        raise NotImplementedError(
+            f"the fixed-order reduction takes fp32 or bf16 contributions and an output of the same dtype, got "
+            f"{contributions.dtype} -> {out.dtype}"
+        )
     if contributions.ndim != 2 or contributions.stride(1) != 1 or not out.is_contiguous():
         raise ValueError("contributions must be [W, row] with unit column stride and out contiguous")
     world, row = contributions.shape
     if column_offset < 0 or column_offset + out.numel() > row:
         raise ValueError(f"range [{column_offset}, {column_offset + out.numel()}) outside rows of {row} elements")
     stride = contributions.stride(0) if world > 1 else row
-    status = _native.lib().fsh_reduce_rows_f32(
+    entry = "fsh_reduce_rows_f32" if out.dtype == torch.float32 else "fsh_reduce_rows_bf16"
+    status = getattr(_native.lib(), entry)(
         out.data_ptr(), contributions.data_ptr(), stride, world, column_offset, out.numel(), mode, factor,
         stream_ptr(out.device),
     )
-    _native.check(status, "fsh_reduce_rows_f32")
+    _native.check(status, entry)
 
 
 def newton_schulz_workspace_bytes(batch: int, rows: int, cols: int) -> int:

@@ -194,6 +194,12 @@ int fsh_accumulate_grad(float* acc_dev, const void* grad_dev, int32_t grad_dtype
 int fsh_reduce_rows_f32(float* out_dev, const float* src_dev, int64_t contribution_stride,
                         int32_t world, int64_t column_offset, int64_t numel, int32_t mode,
                         float factor, void* stream);
+/* The same fold over bf16 contributions into a bf16 range: terms widened to
+ * fp32 (pre-multiplied if asked), added in fp32 in rank order, one rounding to
+ * bf16 at the end.  (A ring reduce-scatter in bf16 rounds after every hop; this
+ * stand-in does not imitate that.) */
+int fsh_reduce_rows_bf16(void* out_dev, const void* src_dev, int64_t contribution_stride, int32_t world,
+                         int64_t column_offset, int64_t numel, int32_t mode, float factor, void* stream);
 
 /* ------------------------------------------------------------------------
  * 6. Newton-Schulz orthogonalization on MFMA.

@@ -273,6 +273,56 @@ def test_fixed_order_reduce_and_modes(device):
         hip_ops.reduce_rows(out, contrib, world * seg - 10)
 
 
+def test_fixed_order_reduce_of_bf16_contributions(device):
+    """bf16 contributions: widened to fp32, added in rank order in fp32, rounded
+    to bf16 once (checked against that fold written out in torch on the CPU;
+    no rounding per hop as a ring in bf16 would have)."""
+    gen = torch.Generator().manual_seed(6)
+    world, seg = 8, 12344
+    contrib = torch.randn(world, world * seg, generator=gen).bfloat16().to(device)
+    out = torch.empty(seg, device=device, dtype=torch.bfloat16)
+
+    def fold(rows, pre=None, post=None):
+        total = None
+        for row in rows:
+            term = row.float() if pre is None else row.float() * torch.tensor(pre, dtype=torch.float32)
+            total = term if total is None else total + term
+        if post is not None:
+            total = post(total)
+        return total.bfloat16()
+
+    third = float(np.float32(1 / 3))
+    for rank in (0, 5):
+        rows = [contrib[r, rank * seg : (rank + 1) * seg].cpu() for r in range(world)]
+        hip_ops.reduce_rows(out, contrib, rank * seg)
+        assert torch.equal(out.cpu(), fold(rows))
+        hip_ops.reduce_rows(out, contrib, rank * seg, mode=hip_ops.REDUCE_PREMUL, factor=1 / 3)
+        assert torch.equal(out.cpu(), fold(rows, pre=third))
+        hip_ops.reduce_rows(out, contrib, rank * seg, mode=hip_ops.REDUCE_POSTMUL, factor=0.125)
+        assert torch.equal(out.cpu(), fold(rows, post=lambda t: t * 0.125))
+        hip_ops.reduce_rows(out, contrib, rank * seg, mode=hip_ops.REDUCE_POSTDIV, factor=3.0)
+        assert torch.equal(out.cpu(), fold(rows, post=lambda t: t / 3.0))
+    # groups of eight and a tail of four in one launch
+    hip_ops.reduce_rows(out[:12340], contrib, 2 * seg)
+    assert torch.equal(out[:12340].cpu(), fold([contrib[r, 2 * seg : 2 * seg + 12340].cpu() for r in range(world)]))
+    # unaligned column offset and odd length take the scalar path
+    odd = torch.empty(1001, device=device, dtype=torch.bfloat16)
+    hip_ops.reduce_rows(odd, contrib, 17)
+    assert torch.equal(odd.cpu(), fold([contrib[r, 17:1018].cpu() for r in range(world)]))
+    with pytest.raises(NotImplementedError, match="same dtype"):
+        hip_ops.reduce_rows(torch.empty(seg, device=device), contrib, 0)
+    # through the one-GPU group: averaged bf16 gradients of three ranks
+    group = LocalReduceGroup(3, 1)
+    sends = [torch.randn(3 * 1000, generator=gen).bfloat16().to(device) for _ in range(3)]
+    for r in (0, 2):
+        group.deposit(r, sends[r])
+    from flex_shard_amd.custom_placements.utils import reduce_scatter_grads
+
+    recv = torch.empty(1000, device=device, dtype=torch.bfloat16)
+    reduce_scatter_grads(recv, sends[1], GradientReduction(), group)
+    assert torch.equal(recv.cpu(), fold([s[1000:2000].cpu() for s in sends], pre=float(np.float32(1.0) / np.float32(3.0))))
+
+
 def test_reduce_plan_table():
     avg, sm = GradientReduction(), GradientReduction(op=dist.ReduceOp.SUM)
     assert gradient_reduce_plan(sm, 8, torch.float32) == ("sum", None, None)
