@@ -191,6 +191,7 @@ class OwnedMuon:
         # batch of independent matrices (the reference views it as one,
         # dist_muon/optimizer.py:2082-2091): the step works on 2-D views.
         self._matrix_counts = [math.prod(p.shape[:-2]) for p in self.params]
+        self._stacked = any(p.ndim > 2 for p in self.params)
         self._matrices = self._as_matrices(self.params)
         self._momentum_matrices = self._as_matrices(self.momentum_buffers)
         # Matrices of one shape and dtype are orthogonalized as one batch; the step's
@@ -248,6 +249,10 @@ class OwnedMuon:
         # an update launch per group.  Same bits as _prepare_muon_input ->
         # _compute_muon_direction -> _apply_muon_update per matrix.
         grad_matrices = self._as_matrices(grads)
+        if self._stacked:
+            # views of a stacked parameter are taken per step: they follow a
+            # parameter whose storage was replaced (``p.data = ...``) since
+            self._matrices = self._as_matrices(self.params)
         for index in self._odd:
             p, g = self._matrices[index], grad_matrices[index]
             direction = _prepare_muon_input(

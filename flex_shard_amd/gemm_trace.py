@@ -24,7 +24,6 @@ from __future__ import annotations
 import argparse
 import collections
 import os
-import sys
 
 TRACE_LIB = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libflexshard_hip_trace.so")
 

@@ -810,7 +810,9 @@ class MuonStepPlan:
         """Per group: the parameters, their momentum buffers and their
         gradients, one of each per matrix, in the same order.  All three are
         read (and the first two written) by kernels queued on the current
-        stream.  ``neg_adjusted_lrs`` / ``direction_scales`` (one per group)
+        stream, and so are the plan's address tables, batch buffers and
+        workspaces: steps of one plan belong on one stream (or on streams
+        ordered one behind the other).  ``neg_adjusted_lrs`` / ``direction_scales`` (one per group)
         replace the step sizes and direction scales the plan was built with:
         the C call reads them from the host table at launch time, so a
         learning-rate schedule passes the current values on every step."""

@@ -933,6 +933,15 @@ def test_owned_muon_takes_stacked_parameters_as_batches_of_matrices(device, gold
     for a, b, c in zip(ours, separate, host, strict=True):
         assert torch.equal(a, b)
         assert (a.cpu().float() - c.float()).abs().max().item() <= tol
+    # a stacked parameter whose storage is replaced between steps is followed
+    moved = stacked[0].clone()
+    stacked[0].data = moved
+    grads = [torch.randn(s, generator=gen).to(dt) for s, dt in zip(shapes, dtypes)]
+    opt_stacked.step([g.to(device) for g in grads])
+    opt_separate.step([m.contiguous().to(device) for g in grads for m in g.reshape(-1, *g.shape[-2:]).unbind(0)])
+    assert stacked[0].data_ptr() == moved.data_ptr()
+    for a, b in zip(stacked[0].unbind(0), separate[:3], strict=True):
+        assert torch.equal(a, b)
     with pytest.raises(ValueError, match="Muon updates matrices"):
         OwnedMuon([torch.zeros(64, device=device, dtype=torch.bfloat16)])
 

@@ -16,7 +16,6 @@ from flex_shard_amd.testing import (
     make_param_infos,
     prepare_unshard_on_each_rank,
     seeded_bucket,
-    seeded_normal,
 )
 from oracle import cport, eager
 from oracle import layout as olayout

@@ -14,7 +14,6 @@ from flex_shard_amd.testing import (
     gather_rank_rows,
     local_rows,
     make_param_infos,
-    prepare_unshard_on_each_rank,
 )
 from oracle import cport
 from oracle import layout as olayout
