@@ -100,9 +100,11 @@ def _steady_us(fn, reps: int, settle_ms: float = 25.0) -> float:
     return ms / reps * 1e3
 
 
-def build_quant_workload(device, layers: int, rank: int = 0, spec=None, std: float = 0.02):
-    """Per layer: one rank's local shards as views of one flat bf16 storage (the
-    sharded bucket storage layout), their ParamInfos, and a reusable payload."""
+def build_quant_workload(device, layers: int, rank: int = 0, spec=None, std: float = 0.02,
+                         master_dtype: torch.dtype = torch.bfloat16):
+    """Per layer: one rank's local shards as views of one flat storage (the
+    sharded bucket storage layout; bf16, or fp32 masters that are quantized as
+    bf16), their ParamInfos, and a reusable payload."""
     import torch.nn as nn
 
     from flex_shard_amd import Fp8BucketedBlockShard
@@ -110,21 +112,25 @@ def build_quant_workload(device, layers: int, rank: int = 0, spec=None, std: flo
 
     placement = Fp8BucketedBlockShard(world_size=8, weight_factory=_factory)
     mesh = FakeMesh(8, rank)
-    meta = [(n, nn.Parameter(torch.empty(s, device="meta", dtype=torch.bfloat16)))
+    meta = [(n, nn.Parameter(torch.empty(s, device="meta", dtype=master_dtype)))
             for n, s in (spec or LLAMA3_8B_LAYER)]
     infos = make_param_infos(meta, placement, mesh)
+    for info in infos:
+        info.param_dtype = torch.bfloat16
     local_numel = infos[0].bucket_layout.local_numel
+    size = master_dtype.itemsize
     work = []
     for layer in range(layers):
-        storage = seeded_normal((local_numel,), std, 1000 + layer, device)
+        storage = seeded_normal((local_numel,), std, 1000 + layer, device, master_dtype)
         shards = [
-            storage[i.byte_offset // 2 : i.byte_offset // 2 + i.local_numel].view(i.local_shape) for i in infos
+            storage[i.byte_offset // size : i.byte_offset // size + i.local_numel].view(i.local_shape) for i in infos
         ]
         work.append((storage, shards))
     return placement, mesh, infos, work
 
 
-def bench_quant_pack(device, steps, warmup, layers, rank: int = 0, spec=None, std: float = 0.02, extras: bool = False):
+def bench_quant_pack(device, steps, warmup, layers, rank: int = 0, spec=None, std: float = 0.02, extras: bool = False,
+                     master_dtype: torch.dtype = torch.bfloat16):
     """One step = one pass over the `layers` layer buckets: one fused
     quantize+pack launch per bucket through the placement's contract entry,
     `prepare_unshard_bucket` (payload-cache bookkeeping, the launch, the
@@ -132,12 +138,13 @@ def bench_quant_pack(device, steps, warmup, layers, rank: int = 0, spec=None, st
     as a runtime with one bucket prefetched holds them."""
     import collections
 
-    placement, mesh, infos, work = build_quant_workload(device, layers, rank, spec, std)
+    placement, mesh, infos, work = build_quant_workload(device, layers, rank, spec, std, master_dtype)
     metadata = placement._quant_metadata_from_infos(infos)
     plan = metadata.rank_pack_plans[rank]
     elems = plan.qdata_numel
     scales = sum(sum(c.scale_numels) for c in plan.chunks)
-    algo_bytes = 3 * elems + 4 * scales  # 2 B read + 1 B write per element, 4 B per tile scale
+    # 2 B (4 B of an fp32 master) read + 1 B written per element, 4 B per tile scale
+    algo_bytes = (master_dtype.itemsize + 1) * elems + 4 * scales
     held = collections.deque(maxlen=2)
 
     def launch(layer):
@@ -218,15 +225,17 @@ def bench_quant_pack(device, steps, warmup, layers, rank: int = 0, spec=None, st
 
 
 def bench_other_shares(device):
-    """The same launch on two other shares: the
-    largest rank share of the Llama bucket (rank 6: rows of `down`, in_dim
-    14336) and rank 0 of the DeepSeek-V3 expert bucket (stacked w1 rows)."""
+    """The same launch on other shares: the largest rank share of the Llama
+    bucket (rank 6: rows of `down`, in_dim 14336), rank 0 of the DeepSeek-V3
+    expert bucket (stacked w1 rows), and the headline share kept as fp32
+    masters that are quantized as bf16 (4 B read + 1 B written per element)."""
     from flex_shard_amd.testing import DEEPSEEK_V3_EXPERTS
 
     out = {}
     for name, kwargs, steps in (
         ("llama3_8b_rank6", dict(layers=8, rank=6), 25),
         ("deepseek_v3_experts_rank0", dict(layers=2, rank=0, spec=DEEPSEEK_V3_EXPERTS, std=0.006), 20),
+        ("llama3_8b_rank0_fp32_masters", dict(layers=8, rank=0, master_dtype=torch.float32), 25),
     ):
         q = bench_quant_pack(device, steps, 2, **kwargs)
         q.pop("work")

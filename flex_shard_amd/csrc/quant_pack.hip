@@ -310,7 +310,28 @@ struct QuantFastParams {
   int64_t zero_len[2];
 };
 
-template <bool FULL>
+// Two floats -> two bf16 in one word (low half first), round to nearest even:
+// one v_cvt_pk_bf16_f32.  Finite values and infinities get the bits of
+// f32_to_bf16_bits; a NaN keeps its sign and payload (see canonical_nan_pair).
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t round_pair_to_bf16(float lo, float hi) {
+  const f32x2_t pair = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2_t));
+}
+// Each bf16 half that is a NaN becomes 0x7FC0, what f32_to_bf16_bits gives.
+__device__ __forceinline__ uint32_t canonical_nan_pair(uint32_t w) {
+  if ((w & 0x7FFFu) > 0x7F80u) w = (w & 0xFFFF0000u) | 0x7FC0u;
+  if ((w & 0x7FFF0000u) > 0x7F800000u) w = (w & 0xFFFFu) | 0x7FC00000u;
+  return w;
+}
+
+// F32: the shard is an fp32 master; every element is rounded to bf16 as it is
+// loaded (two 16-byte loads per eight elements), four of a thread's eight tile
+// rows at a time: 79 registers and six workgroups per compute unit instead of
+// 91 and five with all sixteen loads in flight (forced to 72 or 64 registers
+// the compiler spills and the launch is 4 % slower).
+template <bool FULL, bool F32>
 __device__ __forceinline__ void quant_tile128_fast(const FastChunk& ch, uint32_t tr, uint32_t tc, float eps,
                                                    uint32_t* lds) {
   const uint32_t tid = threadIdx.x;
@@ -321,18 +342,46 @@ __device__ __forceinline__ void quant_tile128_fast(const FastChunk& ch, uint32_t
   const uint32_t rows = static_cast<uint32_t>(ch.rows);
   const int64_t src_row_bytes = ch.src_row_bytes;
   const int64_t dst_row_bytes = ch.in_dim;
-  const uint8_t* sp = ch.src + static_cast<int64_t>(row0) * src_row_bytes + static_cast<int64_t>(col) * 2;
+  const uint8_t* sp = ch.src + static_cast<int64_t>(row0) * src_row_bytes + static_cast<int64_t>(col) * (F32 ? 4 : 2);
   uint8_t* dp = ch.qdst + static_cast<int64_t>(row0) * dst_row_bytes + col;
   float* scale_slot = ch.scales + static_cast<int64_t>(tr) * ch.tiles_c + tc;
 
   u32x4 v[8];
+  if (!F32) {
 #pragma unroll
-  for (int k = 0; k < 8; ++k) {
-    if (FULL) {
-      v[k] = load_stream_u32x4(sp + 16 * k * src_row_bytes);
-    } else {
-      v[k] = u32x4{0, 0, 0, 0};
-      if (col_ok && row0 + 16u * k < rows) v[k] = load_stream_u32x4(sp + 16 * k * src_row_bytes);
+    for (int k = 0; k < 8; ++k) {
+      if (FULL) {
+        v[k] = load_stream_u32x4(sp + 16 * k * src_row_bytes);
+      } else {
+        v[k] = u32x4{0, 0, 0, 0};
+        if (col_ok && row0 + 16u * k < rows) v[k] = load_stream_u32x4(sp + 16 * k * src_row_bytes);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      f32x4 a[4], b[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int k = 4 * half + j;
+        a[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        b[j] = a[j];
+        if (FULL || (col_ok && row0 + 16u * k < rows)) {
+          a[j] = load_stream_f32x4(sp + 16 * k * src_row_bytes);
+          b[j] = load_stream_f32x4(sp + 16 * k * src_row_bytes + 16);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int k = 4 * half + j;
+        v[k].x = round_pair_to_bf16(a[j].x, a[j].y);
+        v[k].y = round_pair_to_bf16(a[j].z, a[j].w);
+        v[k].z = round_pair_to_bf16(b[j].x, b[j].y);
+        v[k].w = round_pair_to_bf16(b[j].z, b[j].w);
+      }
+      // The second half's loads stay behind the first half's conversions
+      // (the scheduler by itself hoists them above).
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 
@@ -346,7 +395,20 @@ __device__ __forceinline__ void quant_tile128_fast(const FastChunk& ch, uint32_t
     m = pk_max_u16(m, v[k].z & 0x7FFF7FFFu);
     m = pk_max_u16(m, v[k].w & 0x7FFF7FFFu);
   }
-  const uint32_t lo = m & 0xFFFFu, hi = m >> 16;
+  uint32_t lo = m & 0xFFFFu, hi = m >> 16;
+  if (F32 && (lo > hi ? lo : hi) > 0x7F80u) {
+    // This thread rounded a NaN.  The hardware conversion keeps its sign and
+    // payload; the quantization's NaN is the canonical one (0x7FC0), whose
+    // bits reach the stored scale and the sign of the tile's bytes.
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      v[k].x = canonical_nan_pair(v[k].x);
+      v[k].y = canonical_nan_pair(v[k].y);
+      v[k].z = canonical_nan_pair(v[k].z);
+      v[k].w = canonical_nan_pair(v[k].w);
+    }
+    lo = hi = 0x7FC0u;
+  }
   m = block_max_u32(lo > hi ? lo : hi, lds);
 
   float scale, recip;
@@ -387,12 +449,37 @@ __global__ __launch_bounds__(kThreads) void quantize_pack_bf16_kernel(const Quan
   const bool full = (tr + 1) * 128u <= static_cast<uint32_t>(ch.rows) &&
                     (tc + 1) * 128u <= static_cast<uint32_t>(ch.in_dim);
   if (full)
-    quant_tile128_fast<true>(ch, tr, tc, prm.eps, lds);
+    quant_tile128_fast<true, false>(ch, tr, tc, prm.eps, lds);
   else
-    quant_tile128_fast<false>(ch, tr, tc, prm.eps, lds);
+    quant_tile128_fast<false, false>(ch, tr, tc, prm.eps, lds);
 }
 
+// The same launch for fp32 master shards quantized as bf16 (the parameter
+// dtype of a mixed-precision policy): 4 B read + 1 B written per element.
 template <int N>
+__global__ __launch_bounds__(kThreads) void quantize_pack_f32_master_kernel(const QuantFastParams<N> prm) {
+  __shared__ uint32_t lds[4];
+  const int32_t bid = static_cast<int32_t>(blockIdx.x);
+  int c = 0;
+#pragma unroll
+  for (int i = 0; i < N; ++i) c += bid >= prm.next_begin[i] ? 1 : 0;
+  if (c >= prm.nchunks) {
+    zero_pad_slice(prm.payload, prm.zero_begin, prm.zero_len, bid - prm.chunks[c].tile_begin);
+    return;
+  }
+  const FastChunk ch = prm.chunks[c];
+  const uint32_t t = static_cast<uint32_t>(bid - ch.tile_begin);
+  const uint32_t tr = t / static_cast<uint32_t>(ch.tiles_c);
+  const uint32_t tc = t - tr * static_cast<uint32_t>(ch.tiles_c);
+  const bool full = (tr + 1) * 128u <= static_cast<uint32_t>(ch.rows) &&
+                    (tc + 1) * 128u <= static_cast<uint32_t>(ch.in_dim);
+  if (full)
+    quant_tile128_fast<true, true>(ch, tr, tc, prm.eps, lds);
+  else
+    quant_tile128_fast<false, true>(ch, tr, tc, prm.eps, lds);
+}
+
+template <int N, bool F32>
 void launch_bf16_kernel(const QuantParams& prm, int64_t tiles, int64_t grid, hipStream_t stream) {
   QuantFastParams<N> fast;
   memset(&fast, 0, sizeof(fast));
@@ -404,7 +491,7 @@ void launch_bf16_kernel(const QuantParams& prm, int64_t tiles, int64_t grid, hip
     out.src = in.src;
     out.qdst = prm.payload + in.qdata_offset;
     out.scales = reinterpret_cast<float*>(prm.payload + in.scale_offset);
-    out.src_row_bytes = in.src_row_stride * 2;
+    out.src_row_bytes = in.src_row_stride * (F32 ? 4 : 2);
     out.rows = static_cast<int32_t>(in.rows);
     out.in_dim = static_cast<int32_t>(in.in_dim);
     out.tiles_c = in.tiles_c;
@@ -419,10 +506,14 @@ void launch_bf16_kernel(const QuantParams& prm, int64_t tiles, int64_t grid, hip
     fast.zero_begin[z] = prm.zero_begin[z];
     fast.zero_len[z] = prm.zero_len[z];
   }
-  fast.eps = prm.eps[FSH_SRC_BF16];
+  fast.eps = prm.eps[F32 ? FSH_SRC_F32_AS_BF16 : FSH_SRC_BF16];
   fast.nchunks = nchunks;
-  hipLaunchKernelGGL(quantize_pack_bf16_kernel<N>, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), 0, stream,
-                     fast);
+  if (F32)
+    hipLaunchKernelGGL(quantize_pack_f32_master_kernel<N>, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), 0,
+                       stream, fast);
+  else
+    hipLaunchKernelGGL(quantize_pack_bf16_kernel<N>, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), 0, stream,
+                       fast);
 }
 
 float bf16_round_host(float f) {
@@ -551,7 +642,7 @@ static int quantize_pack_impl(const fsh_quant_chunk* chunks, int32_t nchunks, vo
   prm.eps[FSH_SRC_F16] = prm.eps[FSH_SRC_F32_AS_F16] = eps_mode == FSH_EPS_FP32 ? eps32 : 0.0f;
 
   int64_t tiles = 0;
-  bool all_bf16_fast = true;
+  bool all_bf16_fast = true, all_f32_master_fast = true;
   for (int i = 0; i < nchunks; ++i) {
     const fsh_quant_chunk& in = chunks[i];
     if (in.src_dev == nullptr || in.rows <= 0 || in.in_dim <= 0 || in.src_row_stride < in.in_dim)
@@ -582,8 +673,9 @@ static int quantize_pack_impl(const fsh_quant_chunk* chunks, int32_t nchunks, vo
     out.src_kind = in.src_kind;
     out.fast = !half_kind && block == 128 && aligned(in.src_dev, 16) && (in.src_row_stride * elem) % 16 == 0 &&
                in.in_dim % 8 == 0 && in.qdata_offset % 8 == 0;
-    all_bf16_fast = all_bf16_fast && out.fast && in.src_kind == FSH_SRC_BF16 && in.rows < (1LL << 30) &&
-                    in.in_dim < (1LL << 30);
+    const bool small = in.rows < (1LL << 30) && in.in_dim < (1LL << 30);
+    all_bf16_fast = all_bf16_fast && out.fast && in.src_kind == FSH_SRC_BF16 && small;
+    all_f32_master_fast = all_f32_master_fast && out.fast && in.src_kind == FSH_SRC_F32_AS_BF16 && small;
     tiles += tiles_r * tiles_c;
   }
   prm.total_tiles = tiles;
@@ -599,9 +691,14 @@ static int quantize_pack_impl(const fsh_quant_chunk* chunks, int32_t nchunks, vo
   if (!launch) return FSH_OK;
   if (all_bf16_fast) {
     if (nchunks < 8)
-      launch_bf16_kernel<8>(prm, tiles, grid, static_cast<hipStream_t>(stream));
+      launch_bf16_kernel<8, false>(prm, tiles, grid, static_cast<hipStream_t>(stream));
     else
-      launch_bf16_kernel<FSH_MAX_QUANT_CHUNKS>(prm, tiles, grid, static_cast<hipStream_t>(stream));
+      launch_bf16_kernel<FSH_MAX_QUANT_CHUNKS, false>(prm, tiles, grid, static_cast<hipStream_t>(stream));
+  } else if (all_f32_master_fast && nchunks > 0) {
+    if (nchunks < 8)
+      launch_bf16_kernel<8, true>(prm, tiles, grid, static_cast<hipStream_t>(stream));
+    else
+      launch_bf16_kernel<FSH_MAX_QUANT_CHUNKS, true>(prm, tiles, grid, static_cast<hipStream_t>(stream));
   } else {
     hipLaunchKernelGGL(quantize_pack_kernel, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), 0,
                        static_cast<hipStream_t>(stream), prm);

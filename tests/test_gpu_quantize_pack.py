@@ -173,6 +173,60 @@ def test_fp32_master_is_quantized_as_bf16(device, golden):
 
 
 
+@pytest.mark.parametrize("nparams,world", [(3, 1), (9, 2), (26, 1)])
+def test_fp32_master_buckets_on_the_vector_kernel(device, nparams, world):
+    """fp32 master shards with a bf16 parameter dtype on 128x128 tiles take a
+    vector kernel of their own (8- and 24-entry chunk lookup, whole and
+    partial tiles), which rounds to bf16 as it loads.  Every element's low 16
+    bits are set to one of the tails that decide that rounding (exact, just
+    above, just below a tie, ties to even in both directions), and single
+    tiles hold fp32 denormals, values that round up to infinity, an infinity,
+    and NaNs of both signs; against the C oracle on the values cast by torch.
+    A NaN tile's bytes are compared without their sign (a NaN's sign depends on
+    the platform), its scale must be NaN."""
+    gen = torch.Generator().manual_seed(100 * nparams + world)
+    shapes = [((256, 256), (130, 136), (384, 128), (64, 200), (128, 520))[i % 5] for i in range(nparams)]
+    tails = torch.tensor([0x0000, 0x0001, 0x7FFF, 0x8000, 0x8001, 0xFFFF], dtype=torch.int32)
+    masters = []
+    for shape in shapes:
+        bits = (torch.randn(shape, generator=gen) * 0.02).view(torch.int32)
+        pick = torch.randint(0, len(tails), shape, generator=gen)
+        masters.append(((bits & ~0xFFFF) | tails[pick]).view(torch.float32))
+    masters[0][:128, :128] *= 2.0**-120  # fp32 denormals and tiny normals
+    masters[0][128, 128] = 3.4e38  # rounds up to the bf16 infinity
+    masters[0][128:, :128].view(torch.int32)[5, 7] = 0x7F800000  # an infinity of its own tile
+    masters[1][0, 0] = float("nan")
+    masters[2][130, 5] = -float("nan")
+    nan_tiles = {1: [(0, 0)], 2: [(1, 0)]}
+    named = [(f"w{i}", nn.Parameter(m.to(device), requires_grad=False)) for i, m in enumerate(masters)]
+    pl = Fp8BucketedBlockShard(world_size=world, weight_factory=_factory)
+    lay = olayout.quant_layout(shapes, 128, world)
+    qs, ss = zip(*[cport.quantize_blockwise(m, 128, cast_to_bf16=True) for m in masters])
+    eq, es = zip(*[cport.quantize_blockwise(m.bfloat16(), 128) for m in masters])
+    for a, b, c, d in zip(qs, eq, ss, es):  # the oracle's own rounding equals torch's cast (NaN signs aside)
+        assert ((a == b) | (((a & 0x7F) == 0x7F) & ((b & 0x7F) == 0x7F))).all()
+        assert ((_bits(c) == _bits(d)) | (c.isnan() & d.isnan())).all()
+    for rank in range(world):
+        mesh = FakeMesh(world, rank)
+        infos = make_param_infos(named, pl, mesh)
+        for info in infos:
+            info.param_dtype = torch.bfloat16
+        shards = [local_rows(p, i) for (_, p), i in zip(named, infos)]
+        got = pl.prepare_unshard_bucket(shards, infos, mesh, None).buffers[0].cpu()
+        want = olayout.pack_rank_payload(lay, rank, list(qs), list(ss), 128)
+        same = got == want
+        if not bool(same.all()):
+            # only NaN tiles may differ, and only in the sign bit of their bytes
+            diff = (~same).nonzero().view(-1)
+            assert ((got[diff] & 0x7F) == 0x7F).all() and ((want[diff] & 0x7F) == 0x7F).all(), f"rank {rank}"
+    full_q = [q.clone() for q in qs]
+    for index, tiles in nan_tiles.items():
+        if index < nparams:
+            for tr, tc in tiles:
+                tile = full_q[index][128 * tr : 128 * tr + 128, 128 * tc : 128 * tc + 128]
+                assert ((tile & 0x7F) == 0x7F).all() and ss[index][tr, tc].isnan()
+
+
 @pytest.mark.parametrize("shape,block", [((6, 4), 4), ((12, 6), 4), ((130, 129), 128), ((256, 384), 128), ((64, 64), 16), ((1, 3), 4)])
 def test_fp16_shards_quantize_like_their_fp32_values(device, shape, block):
     """An fp16 weight (and an fp32 master quantized as fp16) against the eager
