@@ -79,6 +79,10 @@ __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
   return sign | h;
 }
 // The fp16 value nearest to f, as a float.
+// fp16 bits (low 16 of `h`) -> float, exact.
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(h)));
+}
 __device__ __forceinline__ float f32_round_to_f16(float f) {
   return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(f32_to_f16_bits(f))));
 }

@@ -70,8 +70,9 @@ __device__ __forceinline__ uint32_t block_max_u32(uint32_t v, uint32_t* lds) {
 // Thread t owns columns 8*(t%16) .. +7 of rows (t/16) + 16k, k = 0..7.
 // Per load instruction a wavefront reads four full 256-byte tile rows.
 
-// bf16 source, or fp32 master rounded to bf16 on load: the tile lives in
-// registers as 32 dwords of packed bf16.
+// bf16 or fp16 source, or fp32 master rounded to one of them on load: the
+// tile lives in registers as 32 dwords of packed 16-bit values.  (Magnitude
+// bits order like the values in both formats, NaN patterns above infinity.)
 template <int KIND>
 __device__ __forceinline__ void quant_tile128_bf16(const QuantChunkDev& ch, int64_t tr, int64_t tc,
                                                    uint8_t* payload, float eps, uint32_t* lds) {
@@ -88,16 +89,23 @@ __device__ __forceinline__ void quant_tile128_bf16(const QuantChunkDev& ch, int6
     const int64_t row = row_base + 16 * k;
     v[k] = u32x4{0, 0, 0, 0};
     if (col_ok && row < ch.rows) {
-      if (KIND == FSH_SRC_BF16) {
+      if (KIND == FSH_SRC_BF16 || KIND == FSH_SRC_F16) {
         v[k] = load_stream_u32x4(ch.src + (row * ch.src_row_stride + col) * 2);
       } else {
         const uint8_t* p = ch.src + (row * ch.src_row_stride + col) * 4;
         const f32x4 a = load_stream_f32x4(p);
         const f32x4 b = load_stream_f32x4(p + 16);
-        v[k].x = f32_to_bf16_bits(a.x) | (f32_to_bf16_bits(a.y) << 16);
-        v[k].y = f32_to_bf16_bits(a.z) | (f32_to_bf16_bits(a.w) << 16);
-        v[k].z = f32_to_bf16_bits(b.x) | (f32_to_bf16_bits(b.y) << 16);
-        v[k].w = f32_to_bf16_bits(b.z) | (f32_to_bf16_bits(b.w) << 16);
+        if (KIND == FSH_SRC_F32_AS_BF16) {
+          v[k].x = f32_to_bf16_bits(a.x) | (f32_to_bf16_bits(a.y) << 16);
+          v[k].y = f32_to_bf16_bits(a.z) | (f32_to_bf16_bits(a.w) << 16);
+          v[k].z = f32_to_bf16_bits(b.x) | (f32_to_bf16_bits(b.y) << 16);
+          v[k].w = f32_to_bf16_bits(b.z) | (f32_to_bf16_bits(b.w) << 16);
+        } else {
+          v[k].x = f32_to_f16_bits(a.x) | (f32_to_f16_bits(a.y) << 16);
+          v[k].y = f32_to_f16_bits(a.z) | (f32_to_f16_bits(a.w) << 16);
+          v[k].z = f32_to_f16_bits(b.x) | (f32_to_f16_bits(b.y) << 16);
+          v[k].w = f32_to_f16_bits(b.z) | (f32_to_f16_bits(b.w) << 16);
+        }
       }
     }
   }
@@ -115,8 +123,9 @@ __device__ __forceinline__ void quant_tile128_bf16(const QuantChunkDev& ch, int6
   const uint32_t lo = m & 0xFFFFu, hi = m >> 16;
   m = block_max_u32(lo > hi ? lo : hi, lds);
 
+  constexpr bool kHalf = KIND == FSH_SRC_F16 || KIND == FSH_SRC_F32_AS_F16;
   float scale, recip;
-  tile_scale(bf16_bits_to_f32(m), eps, scale, recip);
+  tile_scale(kHalf ? f16_bits_to_f32(m) : bf16_bits_to_f32(m), eps, scale, recip);
   if (tid == 0)
     *reinterpret_cast<float*>(payload + ch.scale_offset + 4 * (tr * ch.tiles_c + tc)) = recip;
 
@@ -128,8 +137,8 @@ __device__ __forceinline__ void quant_tile128_bf16(const QuantChunkDev& ch, int6
       uint32_t w[2] = {0, 0};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float e0 = u32_as_f32(d[j] << 16) * scale;
-        const float e1 = u32_as_f32(d[j] & 0xFFFF0000u) * scale;
+        const float e0 = (kHalf ? f16_bits_to_f32(d[j] & 0xFFFFu) : u32_as_f32(d[j] << 16)) * scale;
+        const float e1 = (kHalf ? f16_bits_to_f32(d[j] >> 16) : u32_as_f32(d[j] & 0xFFFF0000u)) * scale;
         w[j >> 1] = cvt2_fp8(e0, e1, w[j >> 1], (j & 1) != 0);
       }
       store_stream_u32x2(payload + ch.qdata_offset + row * ch.in_dim + col, w[0], w[1]);
@@ -268,6 +277,10 @@ __global__ __launch_bounds__(kThreads) void quantize_pack_kernel(const QuantPara
       quant_tile128_bf16<FSH_SRC_BF16>(ch, tr, tc, prm.payload, eps, lds);
     else if (ch.src_kind == FSH_SRC_F32_AS_BF16)
       quant_tile128_bf16<FSH_SRC_F32_AS_BF16>(ch, tr, tc, prm.payload, eps, lds);
+    else if (ch.src_kind == FSH_SRC_F16)
+      quant_tile128_bf16<FSH_SRC_F16>(ch, tr, tc, prm.payload, eps, lds);
+    else if (ch.src_kind == FSH_SRC_F32_AS_F16)
+      quant_tile128_bf16<FSH_SRC_F32_AS_F16>(ch, tr, tc, prm.payload, eps, lds);
     else
       quant_tile128_f32(ch, tr, tc, prm.payload, eps, lds);
   } else {
@@ -659,7 +672,6 @@ static int quantize_pack_impl(const fsh_quant_chunk* chunks, int32_t nchunks, vo
       return fail(FSH_EINVAL, "fsh_quantize_pack: chunk %d scales at %lld misaligned or outside payload", i,
                   (long long)in.scale_offset);
     const int64_t elem = (in.src_kind == FSH_SRC_BF16 || in.src_kind == FSH_SRC_F16) ? 2 : 4;
-    const bool half_kind = in.src_kind == FSH_SRC_F16 || in.src_kind == FSH_SRC_F32_AS_F16;
     if (!aligned(in.src_dev, elem)) return fail(FSH_EINVAL, "fsh_quantize_pack: chunk %d source misaligned", i);
     QuantChunkDev& out = prm.chunks[i];
     out.src = static_cast<const uint8_t*>(in.src_dev);
@@ -671,7 +683,7 @@ static int quantize_pack_impl(const fsh_quant_chunk* chunks, int32_t nchunks, vo
     out.tile_begin = tiles;
     out.tiles_c = static_cast<int32_t>(tiles_c);
     out.src_kind = in.src_kind;
-    out.fast = !half_kind && block == 128 && aligned(in.src_dev, 16) && (in.src_row_stride * elem) % 16 == 0 &&
+    out.fast = block == 128 && aligned(in.src_dev, 16) && (in.src_row_stride * elem) % 16 == 0 &&
                in.in_dim % 8 == 0 && in.qdata_offset % 8 == 0;
     const bool small = in.rows < (1LL << 30) && in.in_dim < (1LL << 30);
     all_bf16_fast = all_bf16_fast && out.fast && in.src_kind == FSH_SRC_BF16 && small;

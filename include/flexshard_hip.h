@@ -55,7 +55,7 @@ const char* fsh_last_error(void);
 #define FSH_SRC_BF16 0        /* bf16 shard, quantized as is                  */
 #define FSH_SRC_F32 1         /* fp32 shard, quantized as fp32                */
 #define FSH_SRC_F32_AS_BF16 2 /* fp32 master shard, rounded to bf16 first     */
-#define FSH_SRC_F16 3         /* fp16 shard, quantized as is (element path)   */
+#define FSH_SRC_F16 3         /* fp16 shard, quantized as is                  */
 #define FSH_SRC_F32_AS_F16 4  /* fp32 master shard, rounded to fp16 first     */
 
 /* Floor applied to a tile's amax. */

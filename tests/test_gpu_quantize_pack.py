@@ -227,7 +227,7 @@ def test_fp32_master_buckets_on_the_vector_kernel(device, nparams, world):
                 assert ((tile & 0x7F) == 0x7F).all() and ss[index][tr, tc].isnan()
 
 
-@pytest.mark.parametrize("shape,block", [((6, 4), 4), ((12, 6), 4), ((130, 129), 128), ((256, 384), 128), ((64, 64), 16), ((1, 3), 4)])
+@pytest.mark.parametrize("shape,block", [((6, 4), 4), ((12, 6), 4), ((130, 129), 128), ((256, 384), 128), ((130, 136), 128), ((64, 64), 16), ((1, 3), 4)])
 def test_fp16_shards_quantize_like_their_fp32_values(device, shape, block):
     """An fp16 weight (and an fp32 master quantized as fp16) against the eager
     restatement of the reference on fp16 input.  fp16 to fp32 is exact and no
