@@ -74,6 +74,39 @@ def test_host_side_argument_checks_need_no_gpu():
     assert lib.fsh_fp8_gemm_1x128_128x1(None, None, None, None, None, 8, 8, 100, 128, 128, 8, None) == -22
 
 
+def test_more_argument_checks_that_need_no_gpu():
+    """Sizes, null pointers and modes are refused before anything is queued,
+    so these calls are safe where there is no GPU; an empty request is a no-op."""
+    lib = _native.lib()
+    fake = 4096  # an aligned address that is never dereferenced: every call below fails (or returns) before a launch
+    EINVAL, ENOTSUP = -22, -95
+    assert lib.fsh_reduce_rows_f32(None, None, 0, 0, 0, 4, 0, 1.0, None) == EINVAL  # world 0
+    assert lib.fsh_reduce_rows_f32(None, None, 8, 2, 0, 4, 0, 1.0, None) == EINVAL  # null pointers
+    assert lib.fsh_reduce_rows_f32(fake, fake, 8, 2, 0, 4, 9, 1.0, None) == EINVAL
+    assert b"mode" in lib.fsh_last_error()
+    assert lib.fsh_reduce_rows_f32(None, None, 8, 2, 0, 0, 0, 1.0, None) == 0
+    assert lib.fsh_reduce_rows_bf16(None, None, 0, 0, 0, 4, 0, 1.0, None) == EINVAL
+    assert lib.fsh_reduce_rows_bf16(fake, fake, 8, 2, 0, 8, 9, 1.0, None) == EINVAL
+    assert b"fsh_reduce_rows_bf16" in lib.fsh_last_error()
+    assert lib.fsh_reduce_rows_bf16(None, None, 8, 2, 0, 0, 0, 1.0, None) == 0
+    assert lib.fsh_zero_segments(None, None, None, 1, 1, 4, None) == EINVAL
+    assert lib.fsh_zero_segments(None, None, None, 0, 1, 4, None) == 0
+    assert lib.fsh_pack_segments(None, None, None, None, None, 1, 1, 0, 1, None, None) == EINVAL
+    assert lib.fsh_pack_segments(fake, fake, fake, fake, fake, 1, 1, 7, 1, fake, None) == EINVAL  # unknown dtype pair
+    assert lib.fsh_pack_segments(None, None, None, None, None, 0, 0, 0, 1, None, None) == 0
+    assert lib.fsh_quant_pack_plan_create(None, 1, 0, 0, 0, 0, 0, 128, 0, None) == EINVAL  # no place for the handle
+    handle = ctypes.c_void_p()
+    assert lib.fsh_quant_pack_plan_create(None, 1, 0, 0, 0, 0, 0, 128, 0, ctypes.byref(handle)) == EINVAL
+    assert handle.value is None
+    assert lib.fsh_quant_pack_plan_launch(None, None, None) == EINVAL
+    lib.fsh_quant_pack_plan_destroy(None)  # destroying nothing is allowed
+    # the allocation-free Newton-Schulz refuses what its fixed scratch cannot hold
+    assert lib.fsh_newton_schulz_noalloc(fake, 0, 8, 8, 1.0, 1.0, 1.0, 5, 1e-7, None) == EINVAL
+    assert lib.fsh_newton_schulz_noalloc(fake, 24, 7168, 2048, 1.0, 1.0, 1.0, 5, 1e-7, None) == ENOTSUP
+    assert b"static scratch" in lib.fsh_last_error()
+    assert lib.fsh_newton_schulz_noalloc(fake, 1 << 20, 8, 8, 1.0, 1.0, 1.0, 5, 1e-7, None) == ENOTSUP
+
+
 def test_no_cpu_compute_path():
     with pytest.raises(RuntimeError, match="GPU"):
         hip_ops.accumulate_grad(torch.zeros(4), torch.zeros(4, dtype=torch.bfloat16))
