@@ -833,7 +833,7 @@ def main() -> None:
                     help="also run a plain 256 MiB -> 256 MiB segment copy, the known-size kernel that the "
                     "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
     ap.add_argument("--only", choices=("muon", "fp8_linear", "runtime_layer_step", "unpack", "gradients",
-                                       "side_stream_copies"),
+                                       "side_stream_copies", "other_shares"),
                     help="profiling aid: run only this secondary section (for counter runs, which slow "
                     "every kernel down) and print its figures instead of the benchmark line")
     args = ap.parse_args()
@@ -863,6 +863,9 @@ def main() -> None:
         return
     if args.only == "muon":
         print(json.dumps({"muon_newton_schulz": bench_muon(device)}))
+        return
+    if args.only == "other_shares":
+        print(json.dumps({"quantize_pack_other_shares": bench_other_shares(device)}))
         return
     if args.only == "runtime_layer_step":
         print(json.dumps({"runtime_layer_step": bench_runtime_layer_step(device)}))
