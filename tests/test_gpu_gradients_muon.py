@@ -323,6 +323,33 @@ def test_fixed_order_reduce_of_bf16_contributions(device):
     assert torch.equal(recv.cpu(), fold([s[1000:2000].cpu() for s in sends], pre=float(np.float32(1.0) / np.float32(3.0))))
 
 
+def test_gradient_kernels_index_beyond_two_to_the_31(device):
+    """More than 2^31 elements: the accumulation of a bf16 gradient into an
+    fp32 bucket and the fixed-order reduction of a rank range whose elements
+    lie beyond 2^32 bytes of the contributions, checked on slices at both ends
+    against the same arithmetic in torch."""
+    n = 2**31 + 4096 + 3
+    acc = torch.zeros(n, device=device)
+    grad = torch.empty(n, device=device, dtype=torch.bfloat16)
+    grad[: 1 << 20].normal_()
+    grad[1 << 20 :] = grad[: 1 << 20].repeat((n >> 20) + 1)[: n - (1 << 20)]
+    hip_ops.accumulate_grad(acc, grad, overwrite=True)
+    hip_ops.accumulate_grad(acc, grad)
+    for sl in (slice(0, 5000), slice(2**31 - 2500, 2**31 + 2500), slice(n - 5000, n)):
+        assert torch.equal(acc[sl], grad[sl].float() + grad[sl].float())
+    del acc, grad
+    world, seg = 2, 2**30 + 8
+    contrib = torch.empty((world, world * seg), device=device)
+    contrib[:, : 1 << 20].normal_()
+    contrib[:, 1 << 20 :] = contrib[:, : 1 << 20].repeat(1, (world * seg >> 20) + 1)[:, : world * seg - (1 << 20)]
+    contrib[1] *= 3.0
+    out = torch.empty(seg, device=device)
+    hip_ops.reduce_rows(out, contrib, seg)  # rank 1's range: columns seg .. 2 seg, row 1 starts 2^33 bytes in
+    for sl in (slice(0, 5000), slice(seg - 5000, seg)):
+        want = contrib[0, seg:][sl] + contrib[1, seg:][sl]
+        assert torch.equal(out[sl], want)
+
+
 def test_reduce_plan_table():
     avg, sm = GradientReduction(), GradientReduction(op=dist.ReduceOp.SUM)
     assert gradient_reduce_plan(sm, 8, torch.float32) == ("sum", None, None)

@@ -442,3 +442,77 @@ def test_llama_gathered_layout_unpack_full_size(device, golden):
     oq, osc = cport.quantize_blockwise(k, 128)
     assert torch.equal(result.full_params[1].view(torch.uint8).cpu(), oq)
     assert torch.equal(dequant[1].cpu().view(torch.int16), cport.dequant_blockwise(oq, osc, 128).view(torch.int16))
+
+
+@pytest.mark.parametrize("world", [1, 8])
+def test_offsets_beyond_two_gib(device, world):
+    """A bucket of nine [16384, 16384] matrices (2.4 G elements): byte offsets
+    in one rank's payload (world 1), in the gathered rows and in the compact
+    buffer pass 2^31, those of the bf16 dequantization pass 2^32.  Bands of 128
+    rows from the first, a middle and the last parameter against the C oracle,
+    through pack, gather, unpack and dequantization."""
+    n, dim = 9, 16384
+    spec = tuple((f"w{i}", (dim, dim)) for i in range(n))
+    factory = RecordingFactory()
+    pl = Fp8BucketedBlockShard(world_size=world, weight_factory=factory)
+    named = seeded_bucket(spec, 0.02, 4200, device)
+    prepared = prepare_unshard_on_each_rank(pl, named, world)
+    rows = gather_rank_rows(prepared)
+    assert rows.numel() > 2**31
+    del prepared[1:]
+    result, dequant = pl.finish_prepared_unshard_with_dequant(prepared[0], rows)
+    assert result.full_params[-1].data_ptr() - result.full_params[0].data_ptr() >= 2**31
+    assert dequant[-1].data_ptr() - dequant[0].data_ptr() >= 2**32
+    for index in (0, 4, n - 1):
+        weight = named[index][1].detach()
+        for band in (0, 77, dim // 128 - 1):
+            lo, hi = band * 128, (band + 1) * 128
+            oq, osc = cport.quantize_blockwise(weight[lo:hi].cpu(), 128)
+            assert torch.equal(result.full_params[index].view(torch.uint8)[lo:hi].cpu(), oq), (index, band)
+            assert torch.equal(factory.calls[index][1][band].cpu().view(torch.int32), osc.view(-1).view(torch.int32))
+            want = cport.dequant_blockwise(oq, osc, 128)
+            assert torch.equal(dequant[index][lo:hi].cpu().view(torch.int16), want.view(torch.int16)), (index, band)
+    # every parameter, on the GPU: the gathered bytes are those of quantizing the whole matrix
+    from flex_shard_amd.custom_placements.fp8_bucketed_block_shard import _quantize_dense_weight_to_blockwise_fp8
+
+    for index, (fqn, p) in enumerate(named):
+        wq, ws = _quantize_dense_weight_to_blockwise_fp8(p.detach(), 128, E4M3)
+        assert torch.equal(result.full_params[index].view(torch.uint8), wq.view(torch.uint8)), fqn
+        assert torch.equal(factory.calls[index][1].view(torch.int32), ws.view(torch.int32)), fqn
+        del wq, ws
+
+
+def test_segment_kernels_with_offsets_beyond_two_to_the_32_bytes(device):
+    """Copy, zero and casting pack of segments whose source and destination
+    offsets lie beyond 2^32 bytes of their buffers (int64 tables end to end)."""
+    from flex_shard_amd.custom_placements._copy_kernels import pack_segments_into_flat_buffer
+
+    n = 2**32 + (1 << 22)
+    src = torch.empty(n, dtype=torch.uint8, device=device)
+    src[-(1 << 22) :].random_(0, 256)
+    src[:4096].random_(0, 256)
+    dst = torch.full((n,), 9, dtype=torch.uint8, device=device)
+    far = 2**32 + 12345
+    desc = SegmentCopyDescriptor.create(
+        src_offsets=[far, 17], numels=[1_000_001, 3000], dst_offsets=[far + 4097, 2**32 + 5], device=device
+    )
+    copy_segments(src, dst, desc)
+    assert torch.equal(dst[far + 4097 : far + 4097 + 1_000_001], src[far : far + 1_000_001])
+    assert torch.equal(dst[2**32 + 5 : 2**32 + 3005], src[17:3017])
+    assert (dst[2**32 + 3005 : far + 4097] == 9).all() and (dst[far + 4097 + 1_000_001 :] == 9).all()
+    zero_segments(dst, desc)
+    assert (dst[far + 4097 : far + 4097 + 1_000_001] == 0).all() and (dst[2**32 + 5 : 2**32 + 3005] == 0).all()
+    assert dst[2**32 + 4].item() == 9 and dst[2**32 + 3005].item() == 9
+    del src, dst
+    # bf16 -> fp32 pack: source element 2^31 + ..., destination element 2^31 + ... (8.6 GB into the output)
+    m = 2**31 + (1 << 21)
+    grads = torch.empty(m, dtype=torch.bfloat16, device=device)
+    grads[-(1 << 21) :].normal_()
+    out = torch.ones(m, dtype=torch.float32, device=device)
+    start, zeros_at = 2**31 + 1000, 2**31 + 700_000
+    keep = pack_segments_into_flat_buffer([grads], [0, -1], [start, 0], [600_000, 5000], [start + 8, zeros_at], out)
+    assert keep is not None
+    assert torch.equal(out[start + 8 : start + 8 + 600_000], grads[start : start + 600_000].float())
+    assert (out[zeros_at : zeros_at + 5000] == 0).all()
+    assert (out[start + 8 + 600_000 : zeros_at] == 1).all() and (out[2**31 - 4096 : start + 8] == 1).all()
+
