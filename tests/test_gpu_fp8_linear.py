@@ -222,3 +222,33 @@ def test_projections_that_share_an_activation_quantize_it_once(device):
     again_outs, again_grads = run()
     for (gx, gw), (px, pw) in zip(again_grads, grads):
         assert torch.equal(gx, px) and torch.equal(gw, pw)
+
+
+def test_products_whose_output_passes_two_to_the_32_bytes(device):
+    """65 536 tokens x 32 768 outputs (4.3 GB of bf16), a short contraction:
+    the corners of the forward product and of the weight-gradient product
+    with small-integer operands and power-of-two scales, where every order of
+    summation gives the same bits, against the eager restatement on the host."""
+    from oracle import eager
+
+    gen = torch.Generator().manual_seed(41)
+    m, n, k = 65536, 32768, 128
+    ints = lambda shape, high: torch.randint(-high, high + 1, shape, generator=gen).float().to(torch.float8_e4m3fn)
+    pow2 = lambda shape: torch.exp2(torch.randint(-2, 3, shape, generator=gen).float())
+    xq, wq, xs, ws = ints((m, k), 1), ints((n, k), 1), pow2((1, m)), pow2((n // 128, 1))
+    got = hip_ops.fp8_gemm_1x128_128x128(xq.to(device), xs.to(device), wq.to(device), ws.to(device))
+    assert got.numel() * got.element_size() >= 2**32
+    for rows, cols in ((slice(0, 300), slice(0, 384)), (slice(m - 300, m), slice(n - 384, n)), (slice(0, 130), slice(n - 128, n))):
+        blocks = slice(cols.start // 128, cols.stop // 128)  # the selected output columns are whole scale blocks
+        want = eager.fp8_gemm_1x128_128x128(xq[rows], xs[:, rows], wq[cols], ws[blocks], out_dtype=torch.float32)
+        assert torch.equal(got[rows, cols].cpu(), want.bfloat16())
+    del got
+    # weight gradient [n, m2] over 128 tokens: outputs beyond 2^32 bytes as well
+    m2 = 65536
+    aq, bq, a_s, b_s = ints((n, k), 2), ints((m2, k), 2), pow2((1, n)), pow2((1, m2))
+    got = hip_ops.fp8_gemm_1x128_128x1(aq.to(device), a_s.to(device), bq.to(device), b_s.to(device))
+    assert tuple(got.shape) == (n, m2)
+    for rows, cols in ((slice(0, 300), slice(0, 300)), (slice(n - 300, n), slice(m2 - 300, m2))):
+        want = eager.fp8_gemm_1x128_128x1(aq[rows], a_s[:, rows], bq[cols], b_s[:, cols], out_dtype=torch.float32)
+        assert torch.equal(got[rows, cols].cpu(), want.bfloat16())
+

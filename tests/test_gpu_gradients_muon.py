@@ -973,6 +973,26 @@ def test_owned_muon_takes_stacked_parameters_as_batches_of_matrices(device, gold
         OwnedMuon([torch.zeros(64, device=device, dtype=torch.bfloat16)])
 
 
+def test_newton_schulz_batch_beyond_two_to_the_32_bytes(device):
+    """160 matrices of [7168, 2048]: the batch (4.7 GB) and every workspace
+    buffer pass 2^32 bytes.  The first and the last 24 matrices must come out
+    with the bits of a 24-matrix call on their own (same kernels and k order;
+    only the addresses differ)."""
+    batch, rows, cols = 160, 7168, 2048
+    x = torch.empty((batch, rows, cols), device=device, dtype=torch.bfloat16)
+    x[:24].normal_()
+    x[-24:].normal_()
+    x[24:-24] = x[:8].repeat((batch - 48) // 8, 1, 1)
+    assert x.numel() * 2 > 2**32
+    first, last = x[:24].clone(), x[-24:].clone()
+    hip_ops.newton_schulz(x, (3.4445, -4.7750, 2.0315), 5, 1e-7)
+    hip_ops.newton_schulz(first, (3.4445, -4.7750, 2.0315), 5, 1e-7)
+    hip_ops.newton_schulz(last, (3.4445, -4.7750, 2.0315), 5, 1e-7)
+    assert torch.equal(x[:24], first)
+    assert torch.equal(x[-24:], last)
+    assert torch.equal(x[24:32], x[:8]) and torch.equal(x[-32:-24], x[:8])
+
+
 # ------------------------------------------- config 5 at the benchmarked size
 CONFIG5_SHAPES = [(7168, 2048)] * 24 + [(2048, 2048)] * 24
 
