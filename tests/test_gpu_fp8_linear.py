@@ -229,8 +229,6 @@ def test_products_whose_output_passes_two_to_the_32_bytes(device):
     the corners of the forward product and of the weight-gradient product
     with small-integer operands and power-of-two scales, where every order of
     summation gives the same bits, against the eager restatement on the host."""
-    from oracle import eager
-
     gen = torch.Generator().manual_seed(41)
     m, n, k = 65536, 32768, 128
     ints = lambda shape, high: torch.randint(-high, high + 1, shape, generator=gen).float().to(torch.float8_e4m3fn)

@@ -348,3 +348,34 @@ def test_llama_sized_gradients_on_sampled_entries(device):
         want = float(g_col @ x_col)
         scale = float(g_col.abs() @ x_col.abs())
         assert abs(float(grad_w[o, i]) - want) <= RTOL * abs(want) + 1e-5 * scale
+
+
+def test_quantizers_and_transpose_on_a_matrix_beyond_two_to_the_32_bytes(device):
+    """[65536, 32768] bf16 (4.3 GB): both quantizers, the one-pass form of both
+    and the byte transpose, whose input and output offsets pass 2^31 elements;
+    corners against the eager restatement on the host."""
+    rows, cols = 65536, 32768
+    x = torch.empty((rows, cols), device=device, dtype=torch.bfloat16)
+    x[:512].normal_()
+    x[512:] = x[:512].repeat(rows // 512 - 1, 1)
+    x[-384:].normal_()
+    q, s = hip_ops.act_quant_1x128(x)
+    qt, st = hip_ops.act_quant_128x1_transposed(x)
+    both = hip_ops.act_quant_both(x)
+    for a, b in zip(both, (q, s, qt, st)):
+        assert torch.equal(a.view(torch.uint8) if a.dtype != torch.float32 else a.view(torch.int32),
+                           b.view(torch.uint8) if b.dtype != torch.float32 else b.view(torch.int32))
+    del both
+    for r, c in ((slice(0, 256), slice(0, 256)), (slice(rows - 256, rows), slice(cols - 256, cols))):
+        corner = x[r, c].cpu()
+        wq, ws = eager.act_quant_1x128(corner)
+        assert torch.equal(q[r, c].cpu().view(torch.uint8), wq.view(torch.uint8))
+        assert torch.equal(s[c.start // 128 : c.stop // 128, r].cpu().view(torch.int32), ws.view(torch.int32))
+        wqt, wst = eager.act_quant_128x1_transposed(corner)
+        assert torch.equal(qt[c, r].cpu().view(torch.uint8), wqt.view(torch.uint8))
+        assert torch.equal(st[r.start // 128 : r.stop // 128, c].cpu().view(torch.int32), wst.view(torch.int32))
+    t = hip_ops.fp8_transpose(q)
+    assert tuple(t.shape) == (cols, rows)
+    for r, c in ((slice(0, 300), slice(0, 300)), (slice(rows - 300, rows), slice(cols - 300, cols))):
+        assert torch.equal(t[c, r].view(torch.uint8), q[r, c].view(torch.uint8).t())
+
